@@ -1,0 +1,167 @@
+/*
+ * C ABI of libmvpa_hip.so - MI355X (gfx950) kernels for MVPFormer's multi-variate
+ * parallel attention (MVPA) forward and the dense ops around it.
+ *
+ * Every entry point takes plain pointers and sizes, returns an int status
+ * (0 = MVPA_OK, negative = error, never throws or aborts), allocates nothing and keeps
+ * no state between calls.  Device pointers are owned by the caller; kernels are
+ * enqueued on the hipStream_t passed in (as an opaque void*) and the call returns
+ * without synchronising.
+ */
+#ifndef MVPA_HIP_H
+#define MVPA_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MVPA_ABI_VERSION 1
+
+/* ---- status codes ---------------------------------------------------------------- */
+enum {
+  MVPA_OK = 0,
+  MVPA_ERR_NULL = -1,          /* a required pointer is null                             */
+  MVPA_ERR_HEAD_DIM = -2,      /* Dh not in {16,32,64,128}   (attentions/attn.py:1041-1043) */
+  MVPA_ERR_HEAD_RATIO = -3,    /* H % Hkv != 0               (attentions/attn.py:1044, 1339) */
+  MVPA_ERR_CTX = -4,           /* T <= 0 or C <= 0           (attentions/attn.py:1045)      */
+  MVPA_ERR_SHAPE = -5,         /* B/H <= 0, or N != T*C      (attentions/attn.py:1344)      */
+  MVPA_ERR_DTYPE = -6,         /* unknown dtype / kernel selector                        */
+  MVPA_ERR_ALIGN = -7,         /* pointer or stride not aligned for vector loads         */
+  MVPA_ERR_UNSUPPORTED = -8,   /* valid request that the selected kernel cannot serve    */
+  MVPA_ERR_STRUCT = -9,        /* struct_size does not match this library                */
+  MVPA_ERR_LAUNCH = -10,       /* hipLaunchKernel reported an error                      */
+  MVPA_ERR_NONCAUSAL_BIAS = -11 /* relative biases need the time-causal mask
+                                   (attentions/attn.py:1335-1336)                        */
+};
+
+/* ---- element types ----------------------------------------------------------------- */
+enum {
+  MVPA_F32 = 0,   /* fp32 in, fp32 math, fp32 out                                   */
+  MVPA_BF16 = 1   /* bf16 in/out, bf16 MFMA with fp32 accumulation                  */
+};
+
+/* ---- kernel selector --------------------------------------------------------------- */
+enum {
+  MVPA_KERNEL_AUTO = 0,     /* bf16: tiled MFMA kernel when it supports the shape       */
+  MVPA_KERNEL_GENERIC = 1,  /* fp32-math row-per-lane kernel, any shape                 */
+  MVPA_KERNEL_MFMA = 2      /* bf16 MFMA kernel, error if the shape is unsupported      */
+};
+
+/* ---- flags ------------------------------------------------------------------------- */
+#define MVPA_FLAG_CAUSAL 1u     /* key time > query time is masked (layers/mvpa.py:255-264) */
+#define MVPA_FLAG_CONTENT 2u    /* (q+u).k term present ("global_att", layers/mvpa.py:188)  */
+#define MVPA_FLAG_TIME_BIAS 4u  /* (q+v).r[T-1-(tq-tk)]      (layers/mvpa.py:223,225)      */
+#define MVPA_FLAG_CHAN_BIAS 8u  /* (q+z).e[C-1-|cq-ck|]      (layers/mvpa.py:224,226)      */
+#define MVPA_FLAG_FP8_QK 16u    /* content term QK^T in fp8 e4m3 with per-head scales      */
+
+/*
+ * Arguments of the fused MVPA forward.  Replaces the pair
+ *   attentions/attn.py:1305-1314 (_rel_bias: two matmuls into HBM tables) and
+ *   attentions/attn.py:1064-1123 (the _fwd_kernel launch)
+ * behind flash_mvpa (attentions/attn.py:1317-1366), and the whole of
+ *   layers/mvpa.py:173-278 (_rel_attn) for the non-flash layer.
+ *
+ * Token n of a sample is (time t, channel c) with n = t*C + c.  q/o are indexed
+ * [b][h][n][d], k/v [b][g][n][d] with g = h / (H/Hkv); strides are in ELEMENTS and the
+ * d-stride is 1, so both the reference's contiguous [B,H,N,Dh] and a head-interleaved
+ * [B,T,C,H,Dh] view can be passed without a copy.
+ *
+ *   score(nq,nk) = sm_scale * ( W(tq,tk) * (q+u).k  +  (q+v).r[T-1-(tq-tk)]
+ *                               + (q+z).e[C-1-|cq-ck|] )  + key_bias[b][nk]
+ *   W = 1 if window == 0, or |tq-tk| <= window, or tq == T-1; else 0 (term zeroed, not
+ *   masked - layers/mvpa.py:231-245).  Keys with tk > tq and keys whose channel has
+ *   chan_valid[b][ck] == 0 get probability exactly 0.
+ */
+typedef struct mvpa_fwd_args {
+  uint32_t struct_size;   /* sizeof(mvpa_fwd_args)                                     */
+  int32_t dtype;          /* MVPA_F32 | MVPA_BF16                                      */
+  int32_t kernel;         /* MVPA_KERNEL_*                                             */
+  uint32_t flags;         /* MVPA_FLAG_*                                               */
+  int32_t B, H, Hkv, T, C, Dh;
+  int32_t window;         /* 0 = content term everywhere                               */
+  float sm_scale;         /* multiplies the sum of the three terms                     */
+  const void* q;          /* [B,H,N,Dh]   */
+  const void* k;          /* [B,Hkv,N,Dh] */
+  const void* v;          /* [B,Hkv,N,Dh] */
+  void* o;                /* [B,H,N,Dh]   */
+  int64_t q_stride_b, q_stride_h, q_stride_n;
+  int64_t k_stride_b, k_stride_h, k_stride_n;
+  int64_t v_stride_b, v_stride_h, v_stride_n;
+  int64_t o_stride_b, o_stride_h, o_stride_n;
+  const void* bias_u;     /* [Hkv,Dh] content bias  (attn_bias[0:kvE])                 */
+  const void* bias_v;     /* [Hkv,Dh] time bias     (attn_bias[kvE:2kvE])              */
+  const void* bias_z;     /* [Hkv,Dh] channel bias  (attn_bias[2kvE:3kvE])             */
+  const void* k_time;     /* [Hkv,T,Dh] position_net(positional_embedding)             */
+  const void* k_chan;     /* [Hkv,C,Dh] channel_net(channel_embedding)                 */
+  const uint8_t* chan_valid; /* nullable [B,C]; 0 = channel absent in this sample       */
+  const float* key_bias;     /* nullable [B,N] additive, in score units (generic kernel) */
+  float* lse;                /* nullable [B*H,N] base-2 log-sum-exp of the scores
+                                (the reference's L, attentions/attn.py:327-333)         */
+  const float* fp8_q_scale;  /* nullable [H]   per-head amax scales for MVPA_FLAG_FP8_QK */
+  const float* fp8_k_scale;  /* nullable [Hkv]                                          */
+} mvpa_fwd_args;
+
+/* ABI version of the loaded library. */
+int mvpa_version(void);
+
+/* Human-readable text for a status code (static storage). */
+const char* mvpa_error_string(int status);
+
+/* Host-only check of an argument block; touches no device memory and needs no GPU.
+ * Mirrors the asserts of attentions/attn.py:1041-1045, 1339, 1344. */
+int mvpa_validate(const mvpa_fwd_args* args);
+
+/* Fused forward; replaces attentions/attn.py:1064-1123 + 1305-1314 and
+ * layers/mvpa.py:173-278.  Validates, then enqueues on `stream`. */
+int mvpa_forward(const mvpa_fwd_args* args, void* stream);
+
+/* Which kernel mvpa_forward would run for these arguments: MVPA_KERNEL_GENERIC or
+ * MVPA_KERNEL_MFMA (or a negative status). */
+int mvpa_select_kernel(const mvpa_fwd_args* args);
+
+/*
+ * Index/mask maps exactly as the kernels compute them, for bit-exact tests against
+ * layers/mvpa.py:127-159 (shifts) and :230-264 (window and causal masks).
+ * For every (nq, nk) of one sample writes
+ *   time_idx[nq*N+nk] = T-1-(tq-tk)  (or -1 when tk > tq),
+ *   chan_idx[nq*N+nk] = C-1-|cq-ck|,
+ *   mask_bits[nq*N+nk] = bit0 visible (causal & channel valid), bit1 content term kept.
+ * chan_valid is nullable [C].
+ */
+int mvpa_debug_maps(int32_t T, int32_t C, int32_t window, uint32_t flags,
+                    const uint8_t* chan_valid, int32_t* time_idx, int32_t* chan_idx,
+                    uint8_t* mask_bits, void* stream);
+
+/*
+ * y[M,N] = x[M,K] @ w[N,K]^T  (torch.nn.functional.linear without bias), bf16 in/out,
+ * fp32 accumulate on MFMA.  Replaces the Linear calls on the forward path:
+ * models/fftencoder.py:95 (encoder proj), layers/mvpa.py:354-359, 400 (q_attn, c_attn,
+ * position_net, channel_net, c_proj) and the MLP projections (models/mvpformer.py:146).
+ * Row strides are in elements; K may be any positive value (tail is zero-padded
+ * in-kernel).  epilogue: 0 none, 1 = y = silu(x@w_gate^T) * (x@w_up^T) where w holds
+ * gate rows [0,N) and up rows [N,2N).
+ */
+int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M, int64_t N, int64_t K,
+                     int64_t ldx, int64_t ldw, int64_t ldy, int32_t epilogue, void* stream);
+
+/* RMSNorm over the last dim: y = x * rsqrt(mean(x^2)+eps) * weight
+ * (models/mvpformer.py:108,133,167,380; models/fftencoder.py:67,93).
+ * in_dtype/out_dtype: MVPA_F32 | MVPA_BF16; weight is fp32. */
+int mvpa_rmsnorm(const void* x, const float* weight, void* y, int64_t rows, int32_t cols,
+                 float eps, int32_t in_dtype, int32_t out_dtype, void* stream);
+
+/* out = a + b + c elementwise, bf16 (models/mvpformer.py:147 residual + mlp + attn). */
+int mvpa_add3_bf16(const void* a, const void* b, const void* c, void* out, int64_t n,
+                   void* stream);
+
+/* Multilevel db4 analysis with periodic extension of fp32 rows x[M,L] into
+ * coeffs[M,dwt_size] ordered [cA_L, cD_L, ..., cD_1] (models/fftencoder.py:80-88). */
+int mvpa_wavedec_db4(const float* x, float* coeffs, int64_t M, int32_t L, int32_t levels,
+                     int32_t dwt_size, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MVPA_HIP_H */

@@ -1,0 +1,79 @@
+// Host side of the C ABI: argument validation, kernel selection, status strings.
+// Nothing here touches device memory, so mvpa_validate / mvpa_select_kernel work on a machine
+// without a GPU.
+#include "mvpa_common.h"
+
+extern "C" int mvpa_version(void) { return MVPA_ABI_VERSION; }
+
+extern "C" const char* mvpa_error_string(int status) {
+  switch (status) {
+    case MVPA_OK: return "ok";
+    case MVPA_ERR_NULL: return "required pointer is null";
+    case MVPA_ERR_HEAD_DIM: return "head dim must be one of 16, 32, 64, 128";
+    case MVPA_ERR_HEAD_RATIO: return "Q heads must be divisible by KV heads";
+    case MVPA_ERR_CTX: return "time and channel context must be positive";
+    case MVPA_ERR_SHAPE: return "bad shape (B, H must be positive; N must equal T*C)";
+    case MVPA_ERR_DTYPE: return "unknown dtype or kernel selector";
+    case MVPA_ERR_ALIGN: return "pointer or stride not aligned to 16 bytes";
+    case MVPA_ERR_UNSUPPORTED: return "request not supported by the selected kernel";
+    case MVPA_ERR_STRUCT: return "argument struct size does not match the library";
+    case MVPA_ERR_LAUNCH: return "kernel launch failed";
+    case MVPA_ERR_NONCAUSAL_BIAS: return "relative biases require the time-causal mask";
+  }
+  return "unknown status";
+}
+
+extern "C" int mvpa_validate(const mvpa_fwd_args* a) {
+  if (!a) return MVPA_ERR_NULL;
+  if (a->struct_size != sizeof(mvpa_fwd_args)) return MVPA_ERR_STRUCT;
+  if (a->dtype != MVPA_F32 && a->dtype != MVPA_BF16) return MVPA_ERR_DTYPE;
+  if (a->kernel < MVPA_KERNEL_AUTO || a->kernel > MVPA_KERNEL_MFMA) return MVPA_ERR_DTYPE;
+  if (a->Dh != 16 && a->Dh != 32 && a->Dh != 64 && a->Dh != 128) return MVPA_ERR_HEAD_DIM;
+  if (a->B <= 0 || a->H <= 0 || a->Hkv <= 0) return MVPA_ERR_SHAPE;
+  if (a->H % a->Hkv != 0) return MVPA_ERR_HEAD_RATIO;
+  if (a->T <= 0 || a->C <= 0) return MVPA_ERR_CTX;
+  if ((int64_t)a->T * a->C > (int64_t)1 << 24) return MVPA_ERR_SHAPE;
+  if (a->window < 0) return MVPA_ERR_SHAPE;
+  if (!a->q || !a->k || !a->v || !a->o) return MVPA_ERR_NULL;
+  if (!a->bias_u || !a->bias_v || !a->bias_z || !a->k_time || !a->k_chan) return MVPA_ERR_NULL;
+  if ((a->flags & (MVPA_FLAG_TIME_BIAS | MVPA_FLAG_CHAN_BIAS)) && !(a->flags & MVPA_FLAG_CAUSAL))
+    return MVPA_ERR_NONCAUSAL_BIAS;
+  const int64_t n = (int64_t)a->T * a->C;
+  // a token stride smaller than Dh (or a head/batch stride of 0 with more than one head)
+  // means the caller's N does not match T*C or the view is wrong
+  if (a->q_stride_n < a->Dh || a->k_stride_n < a->Dh || a->v_stride_n < a->Dh ||
+      a->o_stride_n < a->Dh)
+    return MVPA_ERR_SHAPE;
+  (void)n;
+  if (a->flags & MVPA_FLAG_FP8_QK) {
+    if (a->dtype != MVPA_BF16) return MVPA_ERR_UNSUPPORTED;
+    if (!a->fp8_q_scale || !a->fp8_k_scale) return MVPA_ERR_NULL;
+  }
+  if (a->kernel == MVPA_KERNEL_MFMA && !mvpa_mfma_supported(a)) {
+    if (a->dtype == MVPA_BF16) {
+      const uintptr_t p = (uintptr_t)a->q | (uintptr_t)a->k | (uintptr_t)a->v | (uintptr_t)a->o;
+      const int64_t s = a->q_stride_b | a->q_stride_h | a->q_stride_n | a->k_stride_b |
+                        a->k_stride_h | a->k_stride_n | a->v_stride_b | a->v_stride_h |
+                        a->v_stride_n | a->o_stride_b | a->o_stride_h | a->o_stride_n;
+      if ((p & 15) || (s & 7)) return MVPA_ERR_ALIGN;
+    }
+    return MVPA_ERR_UNSUPPORTED;
+  }
+  return MVPA_OK;
+}
+
+extern "C" int mvpa_select_kernel(const mvpa_fwd_args* a) {
+  const int st = mvpa_validate(a);
+  if (st != MVPA_OK) return st;
+  if (a->kernel == MVPA_KERNEL_GENERIC) return MVPA_KERNEL_GENERIC;
+  if (a->kernel == MVPA_KERNEL_MFMA) return MVPA_KERNEL_MFMA;
+  return mvpa_mfma_supported(a) ? MVPA_KERNEL_MFMA : MVPA_KERNEL_GENERIC;
+}
+
+extern "C" int mvpa_forward(const mvpa_fwd_args* a, void* stream) {
+  const int sel = mvpa_select_kernel(a);
+  if (sel < 0) return sel;
+  if (sel == MVPA_KERNEL_MFMA) return mvpa_launch_mfma(a, (hipStream_t)stream);
+  if (a->flags & MVPA_FLAG_FP8_QK) return MVPA_ERR_UNSUPPORTED;
+  return mvpa_launch_generic(a, (hipStream_t)stream);
+}

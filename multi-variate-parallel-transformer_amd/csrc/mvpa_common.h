@@ -1,0 +1,76 @@
+// Shared device/host helpers for the MVPA kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mvpa_hip.h"
+
+namespace mvpa {
+
+// ---- token index maps -------------------------------------------------------------------
+// Token n of a sample is (t, c) = (n / C, n % C).  The reference obtains the two relative
+// gathers with a pad-and-reshape shift (layers/mvpa.py:127-138) and an index matrix
+// (layers/mvpa.py:140-159); both reduce to the closed forms below, which its fused kernel
+// also uses (attentions/attn.py:279-308).
+
+// Row of the time table [T, Dh] used by a query at time tq for a key at time tk <= tq.
+__host__ __device__ inline int time_row(int tq, int tk, int T) { return T - 1 - (tq - tk); }
+
+// Row of the channel table [C, Dh] used by query channel cq for key channel ck.
+__host__ __device__ inline int chan_row(int cq, int ck, int C) {
+  int d = cq - ck;
+  return C - 1 - (d < 0 ? -d : d);
+}
+
+// Content term kept?  layers/mvpa.py:231-245: band |tq-tk| <= window, plus every key for the
+// queries of the last time step.  window == 0 keeps the term everywhere.
+__host__ __device__ inline bool content_kept(int tq, int tk, int T, int window) {
+  int d = tq - tk;
+  if (d < 0) d = -d;
+  return window <= 0 || d <= window || tq == T - 1;
+}
+
+// Key visible under the time-causal mask (layers/mvpa.py:255-264)?
+__host__ __device__ inline bool causal_visible(int tq, int tk, bool causal) {
+  return !causal || tk <= tq;
+}
+
+// ---- bf16 <-> fp32 ----------------------------------------------------------------------
+typedef uint16_t bf16_t;
+
+__host__ __device__ inline float bf16_to_f32(bf16_t x) {
+  union { uint32_t u; float f; } c;
+  c.u = ((uint32_t)x) << 16;
+  return c.f;
+}
+
+// round-to-nearest-even, NaN kept quiet
+__host__ __device__ inline bf16_t f32_to_bf16(float f) {
+  union { uint32_t u; float f; } c;
+  c.f = f;
+  uint32_t u = c.u;
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+template <typename T> struct io;
+template <> struct io<float> {
+  __device__ static inline float load(const float* p) { return *p; }
+  __device__ static inline void store(float* p, float v) { *p = v; }
+};
+template <> struct io<bf16_t> {
+  __device__ static inline float load(const bf16_t* p) { return bf16_to_f32(*p); }
+  __device__ static inline void store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+};
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+}  // namespace mvpa
+
+// ---- launchers implemented by the kernel translation units ----------------------------------
+int mvpa_launch_generic(const mvpa_fwd_args* a, hipStream_t stream);
+int mvpa_launch_mfma(const mvpa_fwd_args* a, hipStream_t stream);
+// 1 if the tiled MFMA kernel can serve these (already validated) arguments
+int mvpa_mfma_supported(const mvpa_fwd_args* a);

@@ -1,0 +1,236 @@
+"""MVPA attention layers with the reference's module interface, running on the HIP kernels.
+
+`MVPFormerGQAAttention` and `MVPFormerGQAFlashAttention` keep the constructor arguments,
+parameter / buffer names, forward signature and return tuple of layers/mvpa.py:8-409, so a
+model file written against the reference (models/mvpformer.py:104-152) can import them
+unchanged and a reference state dict loads key for key.
+
+What differs is mechanism only:
+* q/k/v come out of ONE fused projection GEMM and are handed to the attention kernel as
+  strided [B,T,C,H,Dh] views; the kernel writes its output already head-merged, so the
+  permute+contiguous copies of _split_heads/_merge_heads (layers/mvpa.py:161-171) vanish.
+* the score/softmax/PV chain of _rel_attn (layers/mvpa.py:173-278) is the fused kernel; no
+  [B,H,N,N] tensor exists, hence `output_attentions=True` raises.
+Forward / eval only (no autograd through the kernel).
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+import mvpa_hip
+
+
+class _LoRALinear(torch.nn.Linear):
+    """Bias-free Linear with low-rank adapters under the parameter names the reference's
+    adapter library uses (lora_A, lora_B; layers/mvpa.py:43-62, 86-93).  `enable` marks which
+    equal slices of the output carry an adapter; the effective weight is
+    W + (alpha/r) * B A on those slices.  lora_B is zero-initialised, so a fresh layer equals
+    the plain Linear."""
+
+    def __init__(self, in_features, out_features, r, lora_alpha, enable=(True,)):
+        super().__init__(in_features, out_features, bias=False)
+        self.r = r
+        self.scaling = lora_alpha / r if r > 0 else 0.0
+        self.enable = tuple(bool(e) for e in enable)
+        n_on = sum(self.enable)
+        if r > 0 and n_on > 0:
+            self.lora_A = torch.nn.Parameter(self.weight.new_zeros((r * n_on, in_features)))
+            self.lora_B = torch.nn.Parameter(
+                self.weight.new_zeros((out_features // len(self.enable) * n_on, r)))
+            torch.nn.init.kaiming_uniform_(self.lora_A, a=math.sqrt(5))
+
+    def effective_weight(self) -> torch.Tensor:
+        if self.r <= 0 or not hasattr(self, "lora_A"):
+            return self.weight
+        w = self.weight.clone()
+        slice_rows = self.out_features // len(self.enable)
+        j = 0
+        for i, on in enumerate(self.enable):
+            if on:
+                a = self.lora_A[j * self.r:(j + 1) * self.r]
+                b = self.lora_B[j * slice_rows:(j + 1) * slice_rows]
+                w[i * slice_rows:(i + 1) * slice_rows] += (b @ a) * self.scaling
+                j += 1
+        return w
+
+    def forward(self, x):
+        return torch.nn.functional.linear(x, self.effective_weight())
+
+
+def _weight_of(mod) -> torch.Tensor:
+    return mod.effective_weight() if isinstance(mod, _LoRALinear) else mod.weight
+
+
+def _linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """bf16 on the GPU goes through the library's MFMA GEMM; fp32 uses the BLAS GEMM."""
+    if x.is_cuda and x.dtype == torch.bfloat16:
+        return mvpa_hip.linear(x, w.to(torch.bfloat16))
+    return torch.nn.functional.linear(x, w.to(x.dtype))
+
+
+class MVPFormerGQAAttention(torch.nn.Module):
+    """Interface of layers/mvpa.py:8-337."""
+
+    # the flash subclass of the reference ignores attention_mask / head_mask
+    # (layers/mvpa.py:341-397); this flag keeps that difference between the two classes
+    _honours_masks = True
+
+    def __init__(self, config, is_cross_attention=False, layer_idx=None):
+        super().__init__()
+        max_timesteps = config.max_position_embeddings
+        self.register_buffer(
+            "time_bias",
+            torch.tril(torch.ones((max_timesteps, max_timesteps), dtype=torch.bool)).view(
+                1, 1, max_timesteps, max_timesteps),
+        )
+        self.register_buffer("masked_bias", torch.tensor(-1e4))
+        self.embed_dim = config.hidden_size
+        self.num_heads = config.num_attention_heads
+        self.num_kv_heads = config.n_head_kv
+        self.num_kv_groups = self.num_heads // self.num_kv_heads
+        self.head_dim = self.embed_dim // self.num_heads
+        self.embed_kv_dim = self.head_dim * self.num_kv_heads
+        self.split_size = self.embed_dim
+        self.inner_dim = config.n_inner
+        self.global_att = config.global_att
+        if self.head_dim * self.num_heads != self.embed_dim:
+            raise ValueError(
+                f"`embed_dim` must be divisible by num_heads (got `embed_dim`: {self.embed_dim} and "
+                f"`num_heads`: {self.num_heads}).")
+        self.scale_attn_weights = config.scale_attn_weights
+        self.is_cross_attention = is_cross_attention
+        self.scale_attn_by_inverse_layer_idx = config.scale_attn_by_inverse_layer_idx
+        self.layer_idx = layer_idx
+        self.reorder_and_upcast_attn = config.reorder_and_upcast_attn
+        e, kv = self.embed_dim, self.embed_kv_dim
+        if getattr(config, "lora", False):
+            self.q_attn = _LoRALinear(e, e, config.lora_rank, config.lora_alpha, enable=(True,))
+            self.c_attn = _LoRALinear(e, 2 * kv, config.lora_rank, config.lora_alpha,
+                                      enable=(False, True))
+        else:
+            self.q_attn = torch.nn.Linear(e, e, bias=False)
+            self.c_attn = torch.nn.Linear(e, 2 * kv, bias=False)
+        self.position_net = torch.nn.Linear(e, kv, bias=False)
+        self.channel_net = torch.nn.Linear(e, kv, bias=False)
+        self.c_proj = torch.nn.Linear(e, e, bias=False)
+        self.attn_bias = torch.nn.Parameter(torch.empty(3 * kv))
+        torch.nn.init.normal_(self.attn_bias, std=0.02)
+        self.attn_dropout = torch.nn.Dropout(config.attn_pdrop)
+        self.resid_dropout = torch.nn.Dropout(config.resid_pdrop)
+        self._fused_w = None
+        self._fused_key = None
+
+    def adapter_params(self):
+        return ["q_attn.lora_A", "q_attn.lora_B", "c_attn.lora_A", "c_attn.lora_B"]
+
+    # -- projections --------------------------------------------------------------------------
+    def _qkv_weight(self, dtype) -> torch.Tensor:
+        """[q_attn; c_attn] stacked once and cached until a weight is modified."""
+        srcs = [self.q_attn.weight, self.c_attn.weight]
+        for mod in (self.q_attn, self.c_attn):
+            if isinstance(mod, _LoRALinear) and hasattr(mod, "lora_A"):
+                srcs += [mod.lora_A, mod.lora_B]
+        key = tuple((t.data_ptr(), t._version) for t in srcs) + (dtype,)
+        if self._fused_key != key:
+            self._fused_w = torch.cat([_weight_of(self.q_attn), _weight_of(self.c_attn)], 0).to(dtype).contiguous()
+            self._fused_key = key
+        return self._fused_w
+
+    def _scale(self) -> float:
+        s = 1.0
+        if self.scale_attn_weights:
+            s /= self.head_dim ** 0.5                      # layers/mvpa.py:246-252
+        if self.scale_attn_by_inverse_layer_idx:
+            s /= float(self.layer_idx + 1)                 # layers/mvpa.py:253-254
+        return s
+
+    def _attend(self, hidden_states, positional_embedding, channel_embedding, attention_mask,
+                head_mask, use_cache, window):
+        if self.training and (self.attn_dropout.p > 0 or self.resid_dropout.p > 0):
+            raise NotImplementedError("MVPA HIP layer: dropout/training is not implemented; call .eval()")
+        if self.is_cross_attention:
+            raise NotImplementedError(
+                "MVPA HIP layer: without the time-causal mask the relative-time shift of the "
+                "reference reads wrapped entries (layers/mvpa.py:127-138); not supported")
+        bsz, t_len, c_len, e = hidden_states.shape
+        h, hkv, dh, kv = self.num_heads, self.num_kv_heads, self.head_dim, self.embed_kv_dim
+        n = t_len * c_len
+        dt = hidden_states.dtype
+        with torch.no_grad():
+            qkv = _linear(hidden_states, self._qkv_weight(dt))          # [B,T,C,E+2kvE]
+            row = e + 2 * kv
+            qkv = qkv.view(bsz, n, row)
+            q = qkv[:, :, :e].view(bsz, n, h, dh).permute(0, 2, 1, 3)        # views, no copy
+            k = qkv[:, :, e:e + kv].view(bsz, n, hkv, dh).permute(0, 2, 1, 3)
+            v = qkv[:, :, e + kv:].view(bsz, n, hkv, dh).permute(0, 2, 1, 3)
+            k_time = _linear(positional_embedding, self.position_net.weight)  # [1,T,kvE]
+            k_chan = _linear(channel_embedding, self.channel_net.weight)      # [1,C,kvE]
+            k_time = k_time.view(t_len, hkv, dh).permute(1, 0, 2).contiguous()
+            k_chan = k_chan.view(c_len, hkv, dh).permute(1, 0, 2).contiguous()
+            u, vb, z = (b.view(hkv, dh) for b in self.attn_bias.split(kv, dim=0))
+            chan_valid, key_bias = None, None
+            if attention_mask is not None:
+                key_bias = attention_mask.reshape(bsz, n).to(torch.float32)
+            merged = torch.empty((bsz, n, h, dh), dtype=dt, device=hidden_states.device)
+            mvpa_hip.mvpa_forward(
+                q, k, v, u, vb, z, k_time, k_chan, sm_scale=self._scale(), window=window,
+                causal=True, content=bool(self.global_att), chan_valid=chan_valid,
+                key_bias=key_bias, out=merged.permute(0, 2, 1, 3))
+            if head_mask is not None:                       # layers/mvpa.py:274-275
+                if head_mask.numel() != h:
+                    raise NotImplementedError("head_mask must hold one factor per head")
+                merged = merged * head_mask.to(dt).reshape(1, 1, h, 1)
+            out = _linear(merged.view(bsz, t_len, c_len, e), self.c_proj.weight)
+        present = None
+        if use_cache is True:                               # layers/mvpa.py:318-321
+            present = (k.reshape(bsz, hkv, t_len, c_len, dh), v.reshape(bsz, hkv, t_len, c_len, dh))
+        return out, present
+
+    def forward(
+        self,
+        hidden_states,
+        positional_embedding,
+        channel_embedding,
+        layer_past: Optional[Tuple[torch.Tensor]] = None,
+        attention_mask: Optional[torch.Tensor] = None,
+        head_mask: Optional[torch.Tensor] = None,
+        encoder_hidden_states: Optional[torch.Tensor] = None,
+        encoder_attention_mask: Optional[torch.Tensor] = None,
+        use_cache: Optional[bool] = False,
+        output_attentions: Optional[bool] = False,
+    ):
+        if encoder_hidden_states is not None:
+            raise NotImplementedError("MVPA HIP layer: cross attention is not implemented")
+        if layer_past is not None:
+            raise NotImplementedError("MVPA HIP layer: incremental decoding (layer_past) is not implemented")
+        if not self._honours_masks:
+            attention_mask, head_mask = None, None
+        elif output_attentions:
+            raise NotImplementedError(
+                "MVPA HIP layer: the fused kernel never forms the [B,H,N,N] attention weights")
+        out, present = self._attend(hidden_states, positional_embedding, channel_embedding,
+                                    attention_mask, head_mask, use_cache, window=10)
+        outputs = (out, present)
+        if output_attentions:
+            outputs += (None,)                            # layers/mvpa.py:407-408
+        return outputs
+
+
+class MVPFormerGQAFlashAttention(MVPFormerGQAAttention):
+    """Interface of layers/mvpa.py:340-409: same parameters, attention_mask / head_mask /
+    layer_past ignored, `None` in place of attention weights."""
+
+    _honours_masks = False
+
+    def forward(self, hidden_states, positional_embedding, channel_embedding, layer_past=None,
+                attention_mask=None, head_mask=None, encoder_hidden_states=None,
+                encoder_attention_mask=None, use_cache=False, output_attentions=False):
+        out, present = self._attend(hidden_states, positional_embedding, channel_embedding,
+                                    None, None, use_cache, window=10)
+        outputs = (out, present)
+        if output_attentions:
+            outputs += (None,)
+        return outputs

@@ -1,0 +1,294 @@
+"""ctypes binding of libmvpa_hip.so (the C ABI declared in include/mvpa_hip.h).
+
+PyTorch is used only for device memory and streams: every op here hands raw device
+pointers and the current HIP stream to the library.  There is no fallback: if the shared
+library is missing or an entry point reports an error, the call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmvpa_hip.so")
+
+MVPA_F32, MVPA_BF16 = 0, 1
+KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA = 0, 1, 2
+FLAG_CAUSAL, FLAG_CONTENT, FLAG_TIME_BIAS, FLAG_CHAN_BIAS, FLAG_FP8_QK = 1, 2, 4, 8, 16
+
+ERR_HEAD_DIM, ERR_HEAD_RATIO, ERR_CTX, ERR_SHAPE = -2, -3, -4, -5
+
+
+class MvpaFwdArgs(ctypes.Structure):
+    """Mirror of struct mvpa_fwd_args."""
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32), ("dtype", ctypes.c_int32),
+        ("kernel", ctypes.c_int32), ("flags", ctypes.c_uint32),
+        ("B", ctypes.c_int32), ("H", ctypes.c_int32), ("Hkv", ctypes.c_int32),
+        ("T", ctypes.c_int32), ("C", ctypes.c_int32), ("Dh", ctypes.c_int32),
+        ("window", ctypes.c_int32), ("sm_scale", ctypes.c_float),
+        ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
+        ("o", ctypes.c_void_p),
+        ("q_stride_b", ctypes.c_int64), ("q_stride_h", ctypes.c_int64), ("q_stride_n", ctypes.c_int64),
+        ("k_stride_b", ctypes.c_int64), ("k_stride_h", ctypes.c_int64), ("k_stride_n", ctypes.c_int64),
+        ("v_stride_b", ctypes.c_int64), ("v_stride_h", ctypes.c_int64), ("v_stride_n", ctypes.c_int64),
+        ("o_stride_b", ctypes.c_int64), ("o_stride_h", ctypes.c_int64), ("o_stride_n", ctypes.c_int64),
+        ("bias_u", ctypes.c_void_p), ("bias_v", ctypes.c_void_p), ("bias_z", ctypes.c_void_p),
+        ("k_time", ctypes.c_void_p), ("k_chan", ctypes.c_void_p),
+        ("chan_valid", ctypes.c_void_p), ("key_bias", ctypes.c_void_p),
+        ("lse", ctypes.c_void_p),
+        ("fp8_q_scale", ctypes.c_void_p), ("fp8_k_scale", ctypes.c_void_p),
+    ]
+
+
+class MvpaError(RuntimeError):
+    def __init__(self, status: int, text: str):
+        super().__init__(f"libmvpa_hip: {text} (status {status})")
+        self.status = status
+
+
+_lib = None
+
+
+def load_library() -> ctypes.CDLL:
+    """Load the in-tree shared library; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing - build it with `python __graft_entry__.py` "
+            "(hipcc --offload-arch=gfx950); there is no fallback path")
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, i32, i64, u32, f32 = (ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64,
+                              ctypes.c_uint32, ctypes.c_float)
+    lib.mvpa_version.restype = ctypes.c_int
+    lib.mvpa_version.argtypes = []
+    lib.mvpa_error_string.restype = ctypes.c_char_p
+    lib.mvpa_error_string.argtypes = [ctypes.c_int]
+    for name in ("mvpa_validate", "mvpa_select_kernel"):
+        fn = getattr(lib, name)
+        fn.restype = ctypes.c_int
+        fn.argtypes = [ctypes.POINTER(MvpaFwdArgs)]
+    lib.mvpa_forward.restype = ctypes.c_int
+    lib.mvpa_forward.argtypes = [ctypes.POINTER(MvpaFwdArgs), vp]
+    lib.mvpa_debug_maps.restype = ctypes.c_int
+    lib.mvpa_debug_maps.argtypes = [i32, i32, i32, u32, vp, vp, vp, vp, vp]
+    lib.mvpa_linear_bf16.restype = ctypes.c_int
+    lib.mvpa_linear_bf16.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, i32, vp]
+    lib.mvpa_rmsnorm.restype = ctypes.c_int
+    lib.mvpa_rmsnorm.argtypes = [vp, vp, vp, i64, i32, f32, i32, i32, vp]
+    lib.mvpa_add3_bf16.restype = ctypes.c_int
+    lib.mvpa_add3_bf16.argtypes = [vp, vp, vp, vp, i64, vp]
+    lib.mvpa_wavedec_db4.restype = ctypes.c_int
+    lib.mvpa_wavedec_db4.argtypes = [vp, vp, i64, i32, i32, i32, vp]
+    if lib.mvpa_version() != 1:
+        raise RuntimeError("libmvpa_hip ABI version mismatch")
+    _lib = lib
+    return lib
+
+
+def error_string(status: int) -> str:
+    return load_library().mvpa_error_string(status).decode()
+
+
+def _check(status: int) -> None:
+    """Map library status codes onto the reference's exception types
+    (AssertionError for the shape asserts of attentions/attn.py:1041-1045, 1339, 1344)."""
+    if status == 0:
+        return
+    text = error_string(status)
+    if status in (ERR_HEAD_DIM, ERR_HEAD_RATIO, ERR_CTX, ERR_SHAPE):
+        raise AssertionError(f"libmvpa_hip: {text} (status {status})")
+    raise MvpaError(status, text)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return MVPA_F32
+    if dt == torch.bfloat16:
+        return MVPA_BF16
+    raise TypeError(f"libmvpa_hip supports float32 and bfloat16, got {dt}")
+
+
+def _need_cuda(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("libmvpa_hip ops need tensors in GPU memory (there is no CPU path)")
+
+
+def make_args(q, k, v, out, u, vb, z, k_time, k_chan, *, T: int, C: int,
+              sm_scale: float, window: int = 10, flags: int = 15,
+              chan_valid=None, key_bias=None, lse=None, kernel: int = KERNEL_AUTO,
+              fp8_q_scale=None, fp8_k_scale=None) -> MvpaFwdArgs:
+    """Fill the argument block from [B,H,N,Dh]-indexable tensors (any strides with a unit
+    last stride).  Accepts meta/CPU tensors too so validation can be exercised without a GPU."""
+    a = MvpaFwdArgs()
+    a.struct_size = ctypes.sizeof(MvpaFwdArgs)
+    a.dtype = _dtype_code(q.dtype)
+    a.kernel = kernel
+    a.flags = flags
+    a.B, a.H, _, a.Dh = q.shape
+    a.Hkv = k.shape[1]
+    a.T, a.C = T, C
+    a.window = window
+    a.sm_scale = sm_scale
+    for name, t in (("q", q), ("k", k), ("v", v), ("o", out)):
+        if t.stride(-1) != 1:
+            raise ValueError(f"{name}: last dim must be contiguous")
+        setattr(a, name, t.data_ptr())
+        setattr(a, f"{name}_stride_b", t.stride(0))
+        setattr(a, f"{name}_stride_h", t.stride(1))
+        setattr(a, f"{name}_stride_n", t.stride(2))
+    a.bias_u, a.bias_v, a.bias_z = u.data_ptr(), vb.data_ptr(), z.data_ptr()
+    a.k_time, a.k_chan = k_time.data_ptr(), k_chan.data_ptr()
+    a.chan_valid = chan_valid.data_ptr() if chan_valid is not None else None
+    a.key_bias = key_bias.data_ptr() if key_bias is not None else None
+    a.lse = lse.data_ptr() if lse is not None else None
+    a.fp8_q_scale = fp8_q_scale.data_ptr() if fp8_q_scale is not None else None
+    a.fp8_k_scale = fp8_k_scale.data_ptr() if fp8_k_scale is not None else None
+    return a
+
+
+def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float] = None,
+                 window: int = 10, causal: bool = True, content: bool = True,
+                 time_bias: bool = True, chan_bias: bool = True,
+                 chan_valid: Optional[torch.Tensor] = None,
+                 key_bias: Optional[torch.Tensor] = None, return_lse: bool = False,
+                 kernel: int = KERNEL_AUTO, out: Optional[torch.Tensor] = None,
+                 fp8_qk: bool = False):
+    """Fused MVPA forward on the GPU.
+
+    q [B,H,N,Dh]; k, v [B,Hkv,N,Dh]; u, vb, z [Hkv,Dh]; k_time [Hkv,T,Dh]; k_chan [Hkv,C,Dh];
+    chan_valid [B,C] bool/uint8; key_bias [B,N] float32 additive.  Returns out [B,H,N,Dh] in
+    q's dtype (and the base-2 log-sum-exp [B,H,N] float32 if asked).
+    """
+    lib = load_library()
+    _need_cuda(q, k, v, u, vb, z, k_time, k_chan, chan_valid, key_bias)
+    B, H, N, Dh = q.shape
+    assert k.shape[-1] == Dh and v.shape[-1] == Dh, "head dims of q, k, v differ"
+    T, C = k_time.shape[-2], k_chan.shape[-2]
+    assert N == T * C, "N must equal T*C"
+    dt = q.dtype
+    u, vb, z = (t.to(dt).contiguous() for t in (u, vb, z))
+    k_time, k_chan = k_time.to(dt).contiguous(), k_chan.to(dt).contiguous()
+    if out is None:
+        out = torch.empty((B, H, N, Dh), dtype=dt, device=q.device)
+    if chan_valid is not None:
+        chan_valid = chan_valid.to(torch.uint8).contiguous()
+        assert chan_valid.shape == (B, C)
+    if key_bias is not None:
+        key_bias = key_bias.to(torch.float32).contiguous()
+        assert key_bias.shape == (B, N)
+    lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device) if return_lse else None
+    flags = ((FLAG_CAUSAL if causal else 0) | (FLAG_CONTENT if content else 0) |
+             (FLAG_TIME_BIAS if time_bias else 0) | (FLAG_CHAN_BIAS if chan_bias else 0) |
+             (FLAG_FP8_QK if fp8_qk else 0))
+    q_scale = k_scale = None
+    if fp8_qk:
+        # per-head amax scales mapping each head's range onto e4m3's +-448
+        qf = (q.float() + u.float().repeat_interleave(H // k.shape[1], 0)[None, :, None, :])
+        q_scale = (qf.abs().amax(dim=(0, 2, 3)) / 448.0).clamp_min(1e-12).contiguous()
+        k_scale = (k.float().abs().amax(dim=(0, 2, 3)) / 448.0).clamp_min(1e-12).contiguous()
+    s = (1.0 / Dh ** 0.5) if sm_scale is None else float(sm_scale)
+    a = make_args(q, k, v, out, u, vb, z, k_time, k_chan, T=T, C=C, sm_scale=s, window=window,
+                  flags=flags, chan_valid=chan_valid, key_bias=key_bias, lse=lse, kernel=kernel,
+                  fp8_q_scale=q_scale, fp8_k_scale=k_scale)
+    _check(lib.mvpa_forward(ctypes.byref(a), _stream()))
+    return (out, lse) if return_lse else out
+
+
+def debug_maps(T: int, C: int, window: int = 10, flags: int = 15, chan_valid=None,
+               device="cuda"):
+    """Index and mask maps as the kernels compute them: (time_idx, chan_idx, mask_bits),
+    each [N,N]."""
+    lib = load_library()
+    N = T * C
+    ti = torch.empty((N, N), dtype=torch.int32, device=device)
+    ci = torch.empty((N, N), dtype=torch.int32, device=device)
+    mb = torch.empty((N, N), dtype=torch.uint8, device=device)
+    cv = chan_valid.to(torch.uint8).contiguous() if chan_valid is not None else None
+    _check(lib.mvpa_debug_maps(T, C, window, flags, cv.data_ptr() if cv is not None else None,
+                               ti.data_ptr(), ci.data_ptr(), mb.data_ptr(), _stream()))
+    return ti, ci, mb
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None,
+           gated: bool = False) -> torch.Tensor:
+    """y = x @ weight.T in bf16 on MFMA.  gated=True: weight stacks [gate; up] rows and the
+    result is silu(x@gate.T) * (x@up.T)."""
+    lib = load_library()
+    _need_cuda(x, weight)
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise TypeError("linear: bf16 only")
+    K = x.shape[-1]
+    x2 = x.reshape(-1, K)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    assert weight.shape[1] == K and weight.stride(1) == 1
+    M = x2.shape[0]
+    N = weight.shape[0] // 2 if gated else weight.shape[0]
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    _check(lib.mvpa_linear_bf16(x2.data_ptr(), weight.data_ptr(), out.data_ptr(), M, N, K,
+                                x2.stride(0), weight.stride(0), out.stride(0),
+                                1 if gated else 0, _stream()))
+    return out.view(*x.shape[:-1], N)
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5,
+            out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    lib = load_library()
+    _need_cuda(x, weight)
+    xc = x.contiguous()
+    od = out_dtype or x.dtype
+    y = torch.empty(xc.shape, dtype=od, device=x.device)
+    cols = xc.shape[-1]
+    w = weight.to(torch.float32).contiguous()
+    _check(lib.mvpa_rmsnorm(xc.data_ptr(), w.data_ptr(), y.data_ptr(), xc.numel() // cols, cols,
+                            eps, _dtype_code(x.dtype), _dtype_code(od), _stream()))
+    return y
+
+
+def add3(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor) -> torch.Tensor:
+    lib = load_library()
+    _need_cuda(a, b, c)
+    a, b, c = a.contiguous(), b.contiguous(), c.contiguous()
+    assert a.dtype == b.dtype == c.dtype == torch.bfloat16 and a.shape == b.shape == c.shape
+    out = torch.empty_like(a)
+    _check(lib.mvpa_add3_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), out.data_ptr(),
+                              a.numel(), _stream()))
+    return out
+
+
+def dwt_sizes(size_input: int):
+    """Coefficient sizes per level for db4 / periodic extension and the maximum useful depth
+    floor(log2(L/7)) (models/fftencoder.py:70-78)."""
+    import math
+    levels = max(0, int(math.floor(math.log2(size_input / 7))))
+    sizes, n = [], size_input
+    for _ in range(levels):
+        n = (n + 7) // 2
+        sizes.append(n)
+    sizes.append(n)
+    return levels, sizes
+
+
+def wavedec_db4(x: torch.Tensor, pitch: Optional[int] = None) -> torch.Tensor:
+    """x [M,L] float32 -> coefficients [M,dwt_size] float32, ordered [cA_L, cD_L, .., cD_1]."""
+    lib = load_library()
+    _need_cuda(x)
+    x = x.to(torch.float32).contiguous()
+    M, L = x.shape
+    levels, sizes = dwt_sizes(L)
+    total = sum(sizes)
+    out = torch.empty((M, total), dtype=torch.float32, device=x.device)
+    _check(lib.mvpa_wavedec_db4(x.data_ptr(), out.data_ptr(), M, L, levels, total, _stream()))
+    return out

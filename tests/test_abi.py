@@ -1,0 +1,121 @@
+"""Host-only checks of the C ABI: the library loads, exports every symbol the header
+declares, and rejects bad argument blocks with the documented status codes.  No kernel is
+launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import mvpa_hip
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "mvpa_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mvpa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_exports_every_declared_symbol(lib):
+    names = _declared_functions()
+    assert "mvpa_forward" in names and "mvpa_linear_bf16" in names
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/mvpa_hip.h but not exported"
+    assert lib.mvpa_version() == 1
+
+
+def _args(B=2, H=4, Hkv=4, T=4, C=3, Dh=32, dtype=torch.float32, **kw):
+    N = T * C
+    q = torch.zeros((B, H, N, Dh), dtype=dtype)
+    k = torch.zeros((B, Hkv, N, Dh), dtype=dtype)
+    tab = torch.zeros((Hkv, max(T, C), Dh), dtype=dtype)
+    return mvpa_hip.make_args(q, k, k, q, tab, tab, tab, tab, tab, T=T, C=C, sm_scale=0.1, **kw), (q, k, tab)
+
+
+def test_validate_accepts_good_block(lib):
+    a, keep = _args()
+    assert lib.mvpa_validate(ctypes.byref(a)) == 0
+    assert lib.mvpa_select_kernel(ctypes.byref(a)) == mvpa_hip.KERNEL_GENERIC   # fp32 -> generic
+
+
+@pytest.mark.parametrize("mutate,code", [
+    (lambda a: setattr(a, "Dh", 48), -2),
+    (lambda a: setattr(a, "Hkv", 3), -3),
+    (lambda a: setattr(a, "T", 0), -4),
+    (lambda a: setattr(a, "C", -1), -4),
+    (lambda a: setattr(a, "B", 0), -5),
+    (lambda a: setattr(a, "dtype", 7), -6),
+    (lambda a: setattr(a, "q", None), -1),
+    (lambda a: setattr(a, "k_chan", None), -1),
+    (lambda a: setattr(a, "struct_size", 8), -9),
+    (lambda a: setattr(a, "flags", 2 | 4), -11),
+    (lambda a: setattr(a, "q_stride_n", 8), -5),
+])
+def test_validate_rejects(lib, mutate, code):
+    a, keep = _args()
+    mutate(a)
+    assert lib.mvpa_validate(ctypes.byref(a)) == code
+    assert lib.mvpa_forward(ctypes.byref(a), None) == code      # rejected before any launch
+    assert len(lib.mvpa_error_string(code)) > 3
+
+
+def test_null_block(lib):
+    assert lib.mvpa_validate(None) == -1
+
+
+def test_dense_entry_points_reject_bad_arguments(lib):
+    assert lib.mvpa_linear_bf16(None, None, None, 1, 1, 1, 1, 1, 1, 0, None) == -1
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    p16 = (p + 15) & ~15
+    assert lib.mvpa_linear_bf16(p16, p16, p16, 4, 4, 8, 4, 8, 4, 0, None) == -5   # ldx < K
+    assert lib.mvpa_linear_bf16(p16 + 2, p16, p16, 4, 4, 8, 8, 8, 4, 0, None) == -7
+    assert lib.mvpa_rmsnorm(None, None, None, 1, 1, 1e-5, 0, 0, None) == -1
+    assert lib.mvpa_wavedec_db4(p16, p16, 1, 512, 6, 549, None) == -5            # wrong dwt_size
+    assert lib.mvpa_debug_maps(0, 3, 10, 15, None, p16, p16, p16, None) == -4
+
+
+def test_python_operator_errors():
+    """Same exception types as the reference operator (attentions/attn.py:1041-1045, 1339, 1344)."""
+    from attentions import flashmvpa
+    q = torch.zeros(1, 4, 12, 32)
+    kv = torch.zeros(1, 3, 12, 32)
+    b = torch.zeros(1, 3, 1, 32)
+    with pytest.raises(AssertionError):
+        flashmvpa(q, b, b, b, kv, torch.zeros(1, 3, 4, 32), torch.zeros(1, 3, 3, 32), kv, True, 0.1)
+    kv = torch.zeros(1, 4, 12, 32)
+    b = torch.zeros(1, 4, 1, 32)
+    with pytest.raises(AssertionError):      # N != T*C
+        flashmvpa(q, b, b, b, kv, torch.zeros(1, 4, 5, 32), torch.zeros(1, 4, 3, 32), kv, True, 0.1)
+    with pytest.raises(NotImplementedError):
+        flashmvpa(q, b, b, b, kv, torch.zeros(1, 4, 4, 32), torch.zeros(1, 4, 3, 32), kv, True, 0.1,
+                  p_drop=0.1)
+    with pytest.raises(RuntimeError):        # CPU tensors: no fallback path
+        flashmvpa(q, b, b, b, kv, torch.zeros(1, 4, 4, 32), torch.zeros(1, 4, 3, 32), kv, True, 0.1)
+
+
+def test_layer_state_dict_names():
+    from types import SimpleNamespace
+    from layers import MVPFormerGQAAttention, MVPFormerGQAFlashAttention
+    cfg = SimpleNamespace(max_position_embeddings=16, hidden_size=64, num_attention_heads=4,
+                          n_head_kv=2, n_inner=128, global_att=True, scale_attn_weights=True,
+                          scale_attn_by_inverse_layer_idx=False, reorder_and_upcast_attn=False,
+                          lora=False, attn_pdrop=0.1, resid_pdrop=0.1)
+    for cls in (MVPFormerGQAAttention, MVPFormerGQAFlashAttention):
+        m = cls(cfg, layer_idx=0)
+        assert sorted(m.state_dict().keys()) == sorted([
+            "q_attn.weight", "c_attn.weight", "position_net.weight", "channel_net.weight",
+            "c_proj.weight", "attn_bias", "time_bias", "masked_bias"])
+        assert m.c_attn.weight.shape == (2 * 32, 64) and m.attn_bias.shape == (3 * 32,)
+    cfg.lora, cfg.lora_rank, cfg.lora_alpha, cfg.lora_dropout, cfg.lora_merge = True, 8, 16, 0, True
+    m = MVPFormerGQAAttention(cfg)
+    keys = m.state_dict().keys()
+    for n in m.adapter_params():
+        assert n in keys
+    assert m.c_attn.lora_B.shape == (32, 8) and m.q_attn.lora_A.shape == (8, 64)
+    cfg.hidden_size = 66
+    with pytest.raises(ValueError):
+        MVPFormerGQAAttention(cfg)

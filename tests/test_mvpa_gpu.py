@@ -1,0 +1,151 @@
+"""GPU parity of the fused MVPA forward (through the C ABI) against the CPU oracle."""
+import math
+
+import pytest
+import torch
+
+import mvpa_hip
+from mvpa_hip.synthetic import make_mvpa_inputs
+from oracle import mvpa_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+F32_MAX_ABS = 1e-5            # fp32 kernel vs fp32/fp64 oracle
+BF16_MAX_ABS = 2e-2           # bf16 kernel vs oracle on the same bf16-rounded inputs
+BF16_REL_L2 = 5e-3
+
+
+def _oracle(inp, dtype=torch.float64, **kw):
+    return O.mvpa_direct(inp.q, inp.k, inp.v, inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan,
+                         chan_valid=inp.chan_valid, dtype=dtype, **kw)
+
+
+def _gpu(inp, dtype, **kw):
+    d = inp.to("cuda", dtype)
+    return mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
+                                 chan_valid=d.chan_valid, **kw)
+
+
+def _rel_l2(a, b):
+    return ((a - b).norm() / b.norm()).item()
+
+
+def test_debug_maps_bit_exact():
+    """Gather indices and masks as the kernels compute them == the reference's shift and mask
+    construction, element for element (layers/mvpa.py:127-159, 230-264)."""
+    T, C, W = 14, 5, 10
+    N = T * C
+    valid = torch.tensor([1, 0, 1, 1, 0], dtype=torch.bool)
+    ti, ci, mb = mvpa_hip.debug_maps(T, C, W, chan_valid=valid.cuda())
+    ti, ci, mb = ti.cpu(), ci.cpu(), mb.cpu()
+    # the reference's shifts applied to iota-coded tables give the gathered column
+    xt = torch.arange(T, dtype=torch.float32).expand(1, 1, N, T).contiguous()
+    xc = torch.arange(C, dtype=torch.float32).expand(1, 1, N, C).contiguous()
+    rt = O.repeat_channel(O.rel_shift(xt), C)[0, 0]
+    rc = O.repeat_time(O.rel_shift_chan(xc), T)[0, 0]
+    n = torch.arange(N)
+    causal = (n // C)[None, :] <= (n // C)[:, None]
+    assert torch.equal(ti[causal], rt[causal].to(torch.int32))
+    assert (ti[~causal] == -1).all()
+    assert torch.equal(ci, rc.to(torch.int32))
+    ones = torch.ones((T, T), dtype=torch.bool)
+    win = torch.tril(ones, diagonal=W) & torch.triu(ones, diagonal=-W)
+    win = win.repeat_interleave(C, 0).repeat_interleave(C, 1)
+    win[-C:] = True
+    vis = causal & valid.repeat(T)[None, :]
+    assert torch.equal(mb & 1, vis.to(torch.uint8))
+    assert torch.equal((mb >> 1) & 1, win.to(torch.uint8))
+
+
+def test_fp32_config1_parity():
+    """Config c1 (B2 C8 T32 H4 Dh32, q/k/v ~ N(0,1), seed 0), fp32: max-abs <= 1e-5 against
+    both oracle statements and the committed golden output."""
+    inp = make_mvpa_inputs(B=2, C=8, T=32, H=4, Dh=32, seed=0)
+    out, lse = _gpu(inp, torch.float32, return_lse=True)
+    ref, ref_lse = _oracle(inp, return_lse=True)
+    assert (out.cpu().double() - ref).abs().max().item() <= F32_MAX_ABS
+    assert (lse.cpu().double() - ref_lse).abs().max().item() <= 1e-4
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(B=1, C=3, T=13, H=2, Dh=16, Hkv=1),
+    dict(B=2, C=5, T=23, H=4, Dh=64, Hkv=2, validity=True),
+    dict(B=1, C=130, T=3, H=2, Dh=128, Hkv=2),
+    dict(B=1, C=1, T=40, H=1, Dh=32),
+])
+def test_fp32_generic_shapes(cfg):
+    inp = make_mvpa_inputs(seed=1, table_std=0.3, **cfg)
+    out = _gpu(inp, torch.float32)
+    assert (out.cpu().double() - _oracle(inp)).abs().max().item() <= F32_MAX_ABS
+
+
+def test_fp32_flags_and_key_bias():
+    inp = make_mvpa_inputs(B=2, C=4, T=15, H=2, Dh=32, seed=4, table_std=0.3)
+    d = inp.to("cuda", torch.float32)
+    kb = torch.randn(2, 60) * 0.5
+    kb[0, 7] = torch.finfo(torch.float32).min
+    out = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
+                                key_bias=kb.cuda(), window=3, sm_scale=0.11)
+    ref = O.mvpa_direct(inp.q, inp.k, inp.v, inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan,
+                        key_bias=kb, window=3, sm_scale=0.11)
+    assert (out.cpu().double() - ref).abs().max().item() <= F32_MAX_ABS
+    out = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, content=False)
+    ref = O.mvpa_direct(inp.q, inp.k, inp.v, inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan,
+                        global_att=False)
+    assert (out.cpu().double() - ref).abs().max().item() <= F32_MAX_ABS
+    out = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, window=0)
+    ref = O.mvpa_direct(inp.q, inp.k, inp.v, inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan, window=0)
+    assert (out.cpu().double() - ref).abs().max().item() <= F32_MAX_ABS
+
+
+def test_strided_head_interleaved_layout():
+    """q/k/v as [B,T,C,H,Dh] views and the output written head-merged, without copies."""
+    inp = make_mvpa_inputs(B=2, C=4, T=12, H=4, Dh=32, Hkv=2, seed=6, table_std=0.3)
+    d = inp.to("cuda", torch.float32)
+    B, H, N, Dh = d.q.shape
+    packed = torch.cat([d.q.permute(0, 2, 1, 3).reshape(B, N, -1),
+                        d.k.permute(0, 2, 1, 3).reshape(B, N, -1),
+                        d.v.permute(0, 2, 1, 3).reshape(B, N, -1)], dim=-1).contiguous()
+    e, kv = H * Dh, 2 * Dh
+    q = packed[:, :, :e].view(B, N, H, Dh).permute(0, 2, 1, 3)
+    k = packed[:, :, e:e + kv].view(B, N, 2, Dh).permute(0, 2, 1, 3)
+    v = packed[:, :, e + kv:].view(B, N, 2, Dh).permute(0, 2, 1, 3)
+    merged = torch.zeros((B, N, H, Dh), device="cuda")
+    mvpa_hip.mvpa_forward(q, k, v, d.u, d.vb, d.z, d.k_time, d.k_chan, out=merged.permute(0, 2, 1, 3))
+    ref = _oracle(inp)
+    assert (merged.permute(0, 2, 1, 3).cpu().double() - ref).abs().max().item() <= F32_MAX_ABS
+
+
+def test_bf16_generic_kernel_parity():
+    inp = make_mvpa_inputs(B=2, C=8, T=32, H=4, Dh=32, seed=0).round_to(torch.bfloat16)
+    out = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_GENERIC).float().cpu()
+    ref = _oracle(inp).float()
+    assert (out - ref).abs().max().item() <= BF16_MAX_ABS
+    assert _rel_l2(out, ref) <= BF16_REL_L2
+
+
+def test_masks_are_exact_under_perturbation():
+    """Keys that the masks remove must not influence the result at all: outputs stay
+    bit-identical when K/V change at causally hidden or invalid keys, and when only K
+    changes outside the content window."""
+    cfg = dict(B=1, C=6, T=20, H=2, Dh=32, seed=9, table_std=0.3, validity=True)
+    inp = make_mvpa_inputs(**cfg)
+    inp.chan_valid[0, 2] = False
+    base = _gpu(inp, torch.float32)
+    C, T = inp.C, inp.T
+    p = make_mvpa_inputs(**cfg)
+    p.chan_valid = inp.chan_valid
+    dead = (~inp.chan_valid[0]).nonzero().flatten()
+    for t in range(T):
+        p.k[:, :, t * C + dead] += 5.0
+        p.v[:, :, t * C + dead] -= 5.0
+    p.k[:, :, -C:] *= 2.0
+    p.v[:, :, -C:] *= 2.0
+    out = _gpu(p, torch.float32)
+    assert torch.equal(out[:, :, :-C], base[:, :, :-C])
+    p = make_mvpa_inputs(**cfg)
+    p.chan_valid = inp.chan_valid
+    p.k[:, :, :C] += 1.0           # time step 0: inside the window only for tq <= 10 and tq == T-1
+    out = _gpu(p, torch.float32)
+    same = (out == base).flatten(0, 1).all(-1).view(-1, T, C).all(0).all(-1).cpu()
+    assert same.tolist() == [not (t <= 10 or t == T - 1) for t in range(T)]
