@@ -1,0 +1,162 @@
+#!/usr/bin/env python3
+"""Benchmark of the MVPA forward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3] [--no-cpu] [--no-model]
+
+A step is one fused MVPA forward (one kernel launch) over one batch of synthetic inputs that
+are already resident in HBM.  The default workload is the configuration the headline metric
+is quoted on: B=4, C=64, T=128, H=16, Dh=64, bf16, time-causal, window 10.  Prints ONE JSON
+line with the metric, the roofline of the attention kernel (achieved = algorithmic flops per
+launch / HIP-event time per launch) and a bounded CPU baseline (the oracle's op-by-op
+restatement of the reference PyTorch path on this box's host cores).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(ROOT, "multi-variate-parallel-transformer_amd")
+for _p in (PKG, ROOT):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+BF16_DENSE_PEAK_TFLOPS = 2500.0       # MI355X published dense bf16 MFMA peak
+
+WORKLOADS = {
+    "c2": dict(B=4, C=64, T=128, H=16, Hkv=16, Dh=64, validity=False),
+    "c3": dict(B=8, C=117, T=256, H=16, Hkv=16, Dh=64, validity=True),
+}
+
+
+def algorithmic_flops(B, H, T, C, Dh, window=10):
+    """Flops the operator needs: PV for every causally visible pair, QK^T only where the content
+    term is kept (|tq-tk| <= window, plus the whole last time row), and the two bias-table
+    contractions N*(T+C)."""
+    n = T * C
+    p_causal = C * C * T * (T + 1) // 2
+    if window > 0 and T > window + 1:
+        w1 = window + 1
+        p_window = C * C * (w1 * (w1 + 1) // 2 - w1 + w1 * (T - w1) + T)
+    else:
+        p_window = p_causal
+    return B * H * 2 * Dh * (p_causal + p_window + n * (T + C))
+
+
+def cpu_baseline(cfg, budget_s=12.0):
+    """Oracle restatement of the reference PyTorch MVPA (same op sequence, same N^2 traffic) on
+    the host CPU for a bounded sample: whole (b, h) slices of the workload, fp32."""
+    import torch
+    from mvpa_hip.synthetic import make_mvpa_inputs
+    from oracle import mvpa_oracle as O
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    T, C, Dh = cfg["T"], cfg["C"], cfg["Dh"]
+    # one (b, h) slice at a time; c3 is cut to a prefix of its time steps to bound memory
+    Ts = min(T, 128)
+    inp = make_mvpa_inputs(B=1, C=C, T=Ts, H=1, Dh=Dh, seed=1, qkv_unit=True)
+    q = inp.q.view(1, 1, Ts, C, Dh)
+    k = inp.k.view(1, 1, Ts, C, Dh)
+    v = inp.v.view(1, 1, Ts, C, Dh)
+    tk = inp.k_time.view(1, 1, Ts, 1, Dh)
+    ck = inp.k_chan.view(1, 1, 1, C, Dh)
+    bias = torch.cat([inp.u.reshape(-1), inp.vb.reshape(-1), inp.z.reshape(-1)])
+    flops = algorithmic_flops(1, 1, Ts, C, Dh)
+    with torch.no_grad():
+        O.rel_attn(q, k, tk, ck, v, bias)                      # warm-up
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            O.rel_attn(q, k, tk, ck, v, bias)
+            reps += 1
+            el = time.perf_counter() - t0
+            if el >= budget_s or reps >= 20:
+                break
+    per = el / reps
+    return {
+        "value": round(flops / per / 1e12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{reps} x one (b,h) slice of the workload (T={Ts}, C={C}, Dh={Dh}, fp32), "
+                  f"{per * 1e3:.0f} ms each; algorithmic flops as for the GPU line",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-model", action="store_true", help="skip the MVPFormer-S forward leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures ONE GPU (the MVPA forward shards over batch and "
+              "heads with no exchange step); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import mvpa_hip
+    from mvpa_hip.synthetic import make_mvpa_inputs
+
+    mvpa_hip.load_library()           # fails loudly if the HIP extension is missing
+    cfg = WORKLOADS[args.workload]
+    B, C, T, H, Hkv, Dh = (cfg[k] for k in ("B", "C", "T", "H", "Hkv", "Dh"))
+    inp = make_mvpa_inputs(B=B, C=C, T=T, H=H, Hkv=Hkv, Dh=Dh, seed=0, qkv_unit=True,
+                           validity=cfg["validity"])
+    d = inp.to("cuda:0", torch.bfloat16)
+    torch.cuda.set_device(0)
+    out = torch.empty_like(d.q)
+
+    def step():
+        mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
+                              chan_valid=d.chan_valid, out=out, kernel=mvpa_hip.KERNEL_MFMA)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()                      # kernels go to torch's current stream, so these events see them
+    for _ in range(args.steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kern_ms = ev0.elapsed_time(ev1) / args.steps
+    flops = algorithmic_flops(B, H, T, C, Dh)
+    tflops = flops / (wall_ms * 1e-3) / 1e12
+    kern_tflops = flops / (kern_ms * 1e-3) / 1e12
+
+    line = {
+        "metric": "MVPA fwd TFLOP/s (algorithmic flops), bf16, 1 GPU",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: MVPA forward B={B} C={C} T={T} H={H} Hkv={Hkv} "
+                               f"Dh={Dh}, window 10, time-causal"
+                               + (", per-sample channel validity" if cfg["validity"] else ""),
+                   "algorithmic_flops": flops},
+        "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 2),
+                     "peak": BF16_DENSE_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(kern_tflops / BF16_DENSE_PEAK_TFLOPS, 4),
+                     "traffic": None, "kernel": "mvpa_mfma_kernel",
+                     "kernel_ms": round(kern_ms, 4)},
+    }
+    if not args.no_model:
+        try:
+            from models.bench_model import mvpformer_s_windows_per_s
+            line["mvpformer_s"] = mvpformer_s_windows_per_s()
+        except ImportError:
+            line["mvpformer_s"] = None
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(cfg)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

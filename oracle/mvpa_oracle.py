@@ -261,6 +261,7 @@ def mvpa_direct(
     dtype: torch.dtype = torch.float64,
     q_block: int = 2048,
     heads: Optional[list] = None,                # subset of (b, h) pairs to evaluate
+    q_ranges: Optional[list] = None,             # subset of query rows: [(n0, n1), ...]
     return_lse: bool = False,
 ):
     """Closed-form MVPA: score = s*[W*(q+u).k + (q+v).r[T-1-(tq-tk)] + (q+z).e[C-1-|cq-ck|]],
@@ -285,8 +286,10 @@ def mvpa_direct(
         vv = v[b, g].to(dtype)
         r = k_time[g].to(dtype)
         e = k_chan[g].to(dtype)
-        for q0 in range(0, n, q_block):
-            q1 = min(n, q0 + q_block)
+        blocks = []
+        for (r0, r1) in (q_ranges if q_ranges is not None else [(0, n)]):
+            blocks += [(x, min(r1, x + q_block)) for x in range(r0, r1, q_block)]
+        for (q0, q1) in blocks:
             qq = q[b, h, q0:q1].to(dtype)
             tq = (n_idx[q0:q1] // c_len)[:, None]
             cq = (n_idx[q0:q1] % c_len)[:, None]

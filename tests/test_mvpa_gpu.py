@@ -149,3 +149,164 @@ def test_masks_are_exact_under_perturbation():
     out = _gpu(p, torch.float32)
     same = (out == base).flatten(0, 1).all(-1).view(-1, T, C).all(0).all(-1).cpu()
     assert same.tolist() == [not (t <= 10 or t == T - 1) for t in range(T)]
+
+
+# ------------------------------------------------------------------------------------------
+# tiled bf16 MFMA kernel
+# ------------------------------------------------------------------------------------------
+
+MFMA_SHAPES = [
+    dict(B=1, C=8, T=32, H=2, Dh=32),                              # c1's grid, padded 8 -> 32
+    dict(B=2, C=64, T=16, H=2, Dh=64),                             # one wave per time step
+    dict(B=1, C=32, T=70, H=2, Dh=64),                             # crosses two 32-step slabs
+    dict(B=2, C=40, T=20, H=4, Dh=64, Hkv=2, validity=True),       # ragged channels, GQA
+    dict(B=1, C=117, T=14, H=2, Dh=64, validity=True),             # c3's channel count
+    dict(B=1, C=128, T=6, H=2, Dh=128, Hkv=1),                     # base-model head size
+    dict(B=1, C=64, T=13, H=2, Dh=128),
+    dict(B=1, C=20, T=37, H=1, Dh=128, validity=True),
+    dict(B=1, C=1, T=45, H=2, Dh=32),
+    dict(B=3, C=33, T=5, H=3, Dh=32),                              # B*H not a multiple of 8
+]
+
+
+def _check_bf16(out, ref):
+    out, ref = out.float().cpu(), ref.float()
+    err = (out - ref).abs().max().item()
+    rel = _rel_l2(out, ref)
+    assert err <= BF16_MAX_ABS and rel <= BF16_REL_L2, f"max-abs {err:.3e}, rel-L2 {rel:.3e}"
+
+
+@pytest.mark.parametrize("cfg", MFMA_SHAPES)
+def test_bf16_mfma_shapes(cfg):
+    inp = make_mvpa_inputs(seed=21, table_std=0.3, qkv_unit=True, **cfg).round_to(torch.bfloat16)
+    out, lse = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA, return_lse=True)
+    ref, ref_lse = _oracle(inp, return_lse=True)
+    _check_bf16(out, ref)
+    assert (lse.cpu().double() - ref_lse).abs().max().item() <= 3e-2
+
+
+@pytest.mark.parametrize("kw", [dict(window=3), dict(window=0), dict(content=False),
+                                dict(time_bias=False), dict(chan_bias=False), dict(sm_scale=0.05)])
+def test_bf16_mfma_flags(kw):
+    inp = make_mvpa_inputs(B=1, C=24, T=40, H=2, Dh=64, seed=22, table_std=0.3,
+                           qkv_unit=True).round_to(torch.bfloat16)
+    out = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA, **kw)
+    okw = dict(kw)
+    if "content" in okw:
+        okw["global_att"] = okw.pop("content")
+    tb, cb = okw.pop("time_bias", True), okw.pop("chan_bias", True)
+    ref_in = inp
+    if not tb or not cb:
+        import copy
+        ref_in = copy.copy(inp)
+        if not tb:
+            ref_in.k_time = torch.zeros_like(inp.k_time)
+        if not cb:
+            ref_in.k_chan = torch.zeros_like(inp.k_chan)
+    _check_bf16(out, _oracle(ref_in, **okw))
+
+
+def test_bf16_mfma_large_logits():
+    """Wide score range (q,k,v ~ N(0,1), tables std 1): running-max bookkeeping of the far and
+    near paths must not overflow or lose rows."""
+    inp = make_mvpa_inputs(B=1, C=16, T=48, H=2, Dh=32, seed=23, table_std=1.0).round_to(torch.bfloat16)
+    out = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA)
+    assert torch.isfinite(out).all()
+    _check_bf16(out, _oracle(inp))
+
+
+def test_bf16_mfma_masks_exact_under_perturbation():
+    cfg = dict(B=1, C=40, T=20, H=2, Dh=64, seed=9, table_std=0.3, qkv_unit=True, validity=True)
+    inp = make_mvpa_inputs(**cfg)
+    inp.chan_valid[0, 2] = False
+    run = lambda i: _gpu(i, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA)
+    base = run(inp)
+    C, T = inp.C, inp.T
+    p = make_mvpa_inputs(**cfg)
+    p.chan_valid = inp.chan_valid
+    dead = (~inp.chan_valid[0]).nonzero().flatten()
+    for t in range(T):
+        p.k[:, :, t * C + dead] += 5.0
+        p.v[:, :, t * C + dead] = float("nan")        # absent channels may hold anything
+    p.k[:, :, -C:] *= 2.0
+    p.v[:, :, -C:] *= 2.0
+    out = run(p)
+    assert torch.equal(out[:, :, :-C], base[:, :, :-C])
+    p = make_mvpa_inputs(**cfg)
+    p.chan_valid = inp.chan_valid
+    p.k[:, :, :C] += 1.0
+    out = run(p)
+    same = (out == base).flatten(0, 1).all(-1).view(-1, T, C).all(0).all(-1).cpu()
+    assert same.tolist() == [not (t <= 10 or t == T - 1) for t in range(T)]
+
+
+def test_bf16_mfma_strided_layout_and_auto_dispatch():
+    inp = make_mvpa_inputs(B=2, C=16, T=12, H=4, Dh=64, Hkv=2, seed=6, table_std=0.3,
+                           qkv_unit=True).round_to(torch.bfloat16)
+    d = inp.to("cuda", torch.bfloat16)
+    B, H, N, Dh = d.q.shape
+    packed = torch.cat([d.q.permute(0, 2, 1, 3).reshape(B, N, -1),
+                        d.k.permute(0, 2, 1, 3).reshape(B, N, -1),
+                        d.v.permute(0, 2, 1, 3).reshape(B, N, -1)], dim=-1).contiguous()
+    e, kv = H * Dh, 2 * Dh
+    q = packed[:, :, :e].view(B, N, H, Dh).permute(0, 2, 1, 3)
+    k = packed[:, :, e:e + kv].view(B, N, 2, Dh).permute(0, 2, 1, 3)
+    v = packed[:, :, e + kv:].view(B, N, 2, Dh).permute(0, 2, 1, 3)
+    merged = torch.zeros((B, N, H, Dh), device="cuda", dtype=torch.bfloat16)
+    import ctypes
+    a = mvpa_hip.make_args(q, k, v, merged.permute(0, 2, 1, 3), d.u, d.vb, d.z, d.k_time, d.k_chan,
+                           T=inp.T, C=inp.C, sm_scale=Dh ** -0.5)
+    assert mvpa_hip.load_library().mvpa_select_kernel(ctypes.byref(a)) == mvpa_hip.KERNEL_MFMA
+    mvpa_hip.mvpa_forward(q, k, v, d.u, d.vb, d.z, d.k_time, d.k_chan, out=merged.permute(0, 2, 1, 3))
+    _check_bf16(merged.permute(0, 2, 1, 3), _oracle(inp))
+
+
+def test_bf16_config2_full_size():
+    """Config c2 (B4 C64 T128 H16 Dh64): two heads against the oracle, the rest through
+    size-independent properties."""
+    inp = make_mvpa_inputs(B=4, C=64, T=128, H=16, Dh=64, seed=0, qkv_unit=True).round_to(torch.bfloat16)
+    d = inp.to("cuda", torch.bfloat16)
+    out = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
+                                kernel=mvpa_hip.KERNEL_MFMA)
+    heads = [(0, 0), (3, 15)]
+    ref = _oracle(inp, dtype=torch.float32, heads=heads, q_block=1024)
+    for (b, h) in heads:
+        _check_bf16(out[b, h], ref[b, h])
+    # V == 1 -> every output is 1 (rows of P sum to one)
+    ones = torch.ones_like(d.v)
+    o1 = mvpa_hip.mvpa_forward(d.q, d.k, ones, d.u, d.vb, d.z, d.k_time, d.k_chan).float()
+    assert (o1 - 1).abs().max().item() <= 1e-2
+    # causality, bit exact: changing the last 16 time steps leaves earlier rows untouched
+    k2, v2 = d.k.clone(), d.v.clone()
+    k2[:, :, -16 * 64:] *= -1.5
+    v2[:, :, -16 * 64:] += 1.0
+    o2 = mvpa_hip.mvpa_forward(d.q, k2, v2, d.u, d.vb, d.z, d.k_time, d.k_chan)
+    assert torch.equal(o2[:, :, :-16 * 64], out[:, :, :-16 * 64])
+    # agreement with the fp32-math generic kernel on every head
+    og = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
+                               kernel=mvpa_hip.KERNEL_GENERIC)
+    _check_bf16(out, og.float().cpu())
+
+
+def test_bf16_config3_irregular_channels():
+    """Config c3 (B8 C117 T256 H16 Dh64, per-sample channel validity): sampled query rows of
+    one head against the oracle, masks through bit-exact perturbation."""
+    inp = make_mvpa_inputs(B=8, C=117, T=256, H=16, Dh=64, seed=0, qkv_unit=True,
+                           validity=True).round_to(torch.bfloat16)
+    d = inp.to("cuda", torch.bfloat16)
+    out = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
+                                chan_valid=d.chan_valid, kernel=mvpa_hip.KERNEL_MFMA)
+    C = 117
+    ranges = [(0, 2 * C), (100 * C, 101 * C), (255 * C, 256 * C)]
+    ref = _oracle(inp, dtype=torch.float32, heads=[(5, 7)], q_ranges=ranges, q_block=256)
+    for (r0, r1) in ranges:
+        _check_bf16(out[5, 7, r0:r1], ref[5, 7, r0:r1])
+    # invalid channels and future keys never matter
+    dead = (~d.chan_valid)[:, None, None, :, None]            # [B,1,1,C,1]
+    seven = torch.tensor(7.0, dtype=torch.bfloat16, device="cuda")
+    nan = torch.tensor(float("nan"), dtype=torch.bfloat16, device="cuda")
+    k2 = torch.where(dead, seven, d.k.view(8, 16, 256, C, 64)).view(8, 16, 256 * C, 64)
+    v2 = torch.where(dead, nan, d.v.view(8, 16, 256, C, 64)).view(8, 16, 256 * C, 64)
+    o2 = mvpa_hip.mvpa_forward(d.q, k2, v2, d.u, d.vb, d.z, d.k_time, d.k_chan,
+                               chan_valid=d.chan_valid)
+    assert torch.equal(o2, out)
