@@ -2,7 +2,7 @@
 //
 // Tokens are a T x C grid (n = t*C + c).  Both queries and keys are tiled BY TIME STEP: a key
 // tile is the C keys of one time step tk (channels padded to CP = 32/64/128), a query block is
-// 32 channels of one time step tq.  With that tiling
+// 32 channels of one time step tq and belongs to one wave.  With that tiling
 //   * the time-causal mask is uniform per (query block, key tile): tile tk is either fully
 //     visible (tk <= tq) or skipped - there is no diagonal tile to mask element-wise;
 //   * the relative-time term (q+v).r[T-1-(tq-tk)] is ONE scalar per query row per key tile;
@@ -12,7 +12,7 @@
 //   * the content window (layers/mvpa.py:231-245) is uniform per (query block, key tile) too.
 //     Outside the window the content term is zeroed, so the score is a SUM of a per-tile scalar
 //     and a per-channel value and its exponential FACTORISES:
-//         p(q, tk, ck) = 2^(st[q,tk] - ..) * 2^(bc[q,ck] - ..)  =  et[q,tk] * Ec[q,ck].
+//         p(q, tk, ck) = et[q,tk] * Ec[q,ck].
 //     Such "far" tiles need no QK^T, no per-element exp and no K load:
 //         acc[q,:] += et[q,tk] * (Ec[q,:] @ V[tk]),   l[q] += et[q,tk] * sum_ck Ec[q,ck],
 //     with Ec resident in registers as the MFMA B operand for the whole kernel.
@@ -21,19 +21,28 @@
 // query (MFMA column): the soft-max statistics are per-lane scalars, the row max is an in-lane
 // reduction plus one exchange between the two half-waves, and P^T leaves the QK^T MFMA already
 // in the layout the PV MFMA wants for its B operand (the contraction index is permuted
-// consistently on the V side instead).  V is stored in LDS in "octet" order: the 8 keys that one
-// lane contracts in one MFMA are adjacent, so the V^T fragment is a single 16-byte LDS read.
+// consistently on the V side instead).
 //
-// One workgroup = 4 waves = 4*QB query blocks; K/V tiles are staged global -> registers -> LDS,
-// double buffered, one barrier per key tile.
+// Data movement: K/V tiles go HBM/L2 -> LDS with direct-to-LDS loads (no staging registers)
+// into a ring of STAGES buffers, several tiles ahead of the compute; rows keep their natural
+// [key][dh] layout with an XOR swizzle of the 16-byte chunks (chosen per lane on the global
+// side, since the LDS side of such a load is lane-linear).  K fragments are plain 16-byte LDS
+// reads; V^T fragments come from the transposing LDS read (ds_read_b64_tr_b16), which turns four
+// keys x 16 dh of row-major V into "4 keys per lane, one dh per lane".
+// One workgroup = NW waves = NW query blocks = NW/NCT consecutive time steps; one barrier per
+// key tile.
 #include "mvpa_common.h"
 
 namespace mvpa {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+#define LDS_PTR(T) __attribute__((address_space(3))) T*
+#define GLOBAL_PTR(T) __attribute__((address_space(1))) T*
 
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -42,6 +51,32 @@ __device__ inline void wave_lds_sync() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() would also drain every
+// outstanding global load (vmcnt 0), which would serialise the tile prefetch ring.
+__device__ inline void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+template <int N>
+__device__ inline void wait_vmcnt_imm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// wait until at most n of this wave's vector-memory operations are outstanding
+__device__ inline void wait_vmcnt(int n) {
+  switch (n) {
+    case 0: wait_vmcnt_imm<0>(); break;
+    case 1: wait_vmcnt_imm<1>(); break;
+    case 2: wait_vmcnt_imm<2>(); break;
+    case 3: wait_vmcnt_imm<3>(); break;
+    case 4: wait_vmcnt_imm<4>(); break;
+    case 5: wait_vmcnt_imm<5>(); break;
+    case 6: wait_vmcnt_imm<6>(); break;
+    case 7: wait_vmcnt_imm<7>(); break;
+    default: wait_vmcnt_imm<8>(); break;      // n >= 8: waiting for <= 8 is only stricter
+  }
 }
 
 __device__ inline float xhalf_max(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
@@ -74,37 +109,45 @@ __device__ inline bf16x8 pack8(const f32x16& v, int base) {
   return out;
 }
 
-template <int DH, int NCT, int QB>
+// XOR swizzles of the 16-byte chunk index within a K / V row, chosen so that the lanes that
+// read LDS together (16 consecutive rows at one chunk for K; 4 consecutive rows x 4 chunks for
+// the transposing V read) spread over all banks.
+template <int DH> __device__ inline int swz_k(int row) {
+  return DH == 64 ? ((row >> 1) & 7) : DH == 128 ? (row & 15) : ((row >> 2) & 3);
+}
+template <int DH> __device__ inline int swz_v(int row) {
+  return DH == 64 ? (((row >> 1) & 1) << 2) : DH == 128 ? ((row & 3) << 2) : 0;
+}
+
+template <int DH, int NCT, int NW, int STAGES>
 struct Cfg {
   static constexpr int CP = NCT * 32;          // padded channels per time step
   static constexpr int KS = DH / 16;           // k-steps of the QK^T contraction
   static constexpr int MT = DH / 32;           // 32-row tiles of O^T
-  static constexpr int WPT = NCT / QB;         // waves per time step
-  static constexpr int TQW = 4 / WPT;          // time steps per workgroup
-  static constexpr int QW = QB * 32;           // queries per wave
-  static constexpr int KPITCH = DH + 8;        // K row pitch (elements): 16 B pad
-  static constexpr int K_ELEMS = CP * KPITCH;
-  static constexpr int V_ELEMS = CP * DH;
-  static constexpr int NV = (CP / 4) * (DH / 8);     // V staging tasks per tile
-  static constexpr int NKC = CP * (DH / 8);          // K staging chunks per tile
-  static constexpr int VPT = (NV + 255) / 256;       // per thread
-  static constexpr int KPT = (NKC + 255) / 256;
-  static constexpr size_t KV_BYTES = 2 * (size_t)(K_ELEMS + V_ELEMS) * 2;
-  static constexpr size_t STB_BYTES = 4 * 32 * (size_t)QW * 4;
-  static constexpr size_t MAIN_BYTES = KV_BYTES + STB_BYTES;
-  static constexpr size_t SETUP_BYTES = 4 * (size_t)CP * QW * 4;
-  static constexpr size_t LDS_BYTES = MAIN_BYTES > SETUP_BYTES ? MAIN_BYTES : SETUP_BYTES;
+  static constexpr int TQW = NW / NCT;         // time steps per workgroup
+  static constexpr int THREADS = NW * 64;
+  static constexpr int ROWB = DH * 2;          // bytes per K/V row
+  static constexpr int CHUNKS = DH / 8;        // 16-byte chunks per row
+  static constexpr int TILE_BYTES = CP * ROWB;
+  static constexpr int WLOADS = TILE_BYTES / 1024;           // 64-lane x 16-byte loads per tile
+  static constexpr int LPW = (WLOADS + NW - 1) / NW;         // ... per wave
+  static constexpr int STAGE_BYTES = 2 * TILE_BYTES;         // K tile then V tile
+  static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
+  static constexpr int STB_BYTES = NW * 32 * 32 * 4;
+  static constexpr int MAIN_BYTES = RING_BYTES + STB_BYTES;
+  static constexpr int SETUP_BYTES = NW * CP * 32 * 4;
+  static constexpr int LDS_BYTES = MAIN_BYTES > SETUP_BYTES ? MAIN_BYTES : SETUP_BYTES;
+  static_assert(NW % NCT == 0, "waves must cover whole time steps");
+  static_assert(TILE_BYTES % 1024 == 0, "tile must be a whole number of wave loads");
 };
 
-template <int DH, int NCT, int QB>
-__global__ __launch_bounds__(256, 1) void mvpa_mfma_kernel(mvpa_fwd_args a) {
-  using G = Cfg<DH, NCT, QB>;
-  constexpr int CP = G::CP, KS = G::KS, MT = G::MT, QW = G::QW, KPITCH = G::KPITCH;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  bf16_t* Ks = (bf16_t*)smem_raw;                               // [2][CP][KPITCH]
-  bf16_t* Vt = Ks + 2 * G::K_ELEMS;                             // [2][CP/8][DH][8]
-  float* Stb_all = (float*)(smem_raw + G::KV_BYTES);            // [4][32][QW]
-  float* setup_all = (float*)smem_raw;                          // [4][CP][QW], aliases the above
+template <int DH, int NCT, int NW, int STAGES>
+__global__ __launch_bounds__(NW * 64) void mvpa_mfma_kernel(mvpa_fwd_args a) {
+  using G = Cfg<DH, NCT, NW, STAGES>;
+  constexpr int CP = G::CP, KS = G::KS, MT = G::MT, ROWB = G::ROWB, CHUNKS = G::CHUNKS;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+  float* Stb_all = (float*)(smem_raw + G::RING_BYTES);          // [NW][32][32]
+  float* setup_all = (float*)smem_raw;                          // [NW][CP][32], aliases the ring
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, hh = lane >> 5;
@@ -135,11 +178,13 @@ __global__ __launch_bounds__(256, 1) void mvpa_mfma_kernel(mvpa_fwd_args a) {
   const int g = h / (a.H / a.Hkv);
   const int tq0 = tile * G::TQW;
   const int tq_hi = min(T_ - 1, tq0 + G::TQW - 1);
-  const int tq = tq0 + wave / G::WPT;
+  const int tq = tq0 + wave / NCT;
   const bool active = tq < T_;
-  const int cb0 = (wave % G::WPT) * QB;            // first 32-channel block of this wave
+  const int cq = (wave % NCT) * 32 + ln;           // this lane's query channel
+  const bool qok = active && cq < C_;
 
-  const bf16_t* qbase = (const bf16_t*)a.q + b * a.q_stride_b + h * a.q_stride_h;
+  const bf16_t* qrow = (const bf16_t*)a.q + b * a.q_stride_b + h * a.q_stride_h +
+                       (int64_t)(qok ? tq * C_ + cq : 0) * a.q_stride_n;
   const bf16_t* kbase = (const bf16_t*)a.k + b * a.k_stride_b + g * a.k_stride_h;
   const bf16_t* vbase = (const bf16_t*)a.v + b * a.v_stride_b + g * a.v_stride_h;
   const bf16_t* ktime = (const bf16_t*)a.k_time + (int64_t)g * T_ * DH;
@@ -150,406 +195,346 @@ __global__ __launch_bounds__(256, 1) void mvpa_mfma_kernel(mvpa_fwd_args a) {
   const uint8_t* valid = a.chan_valid ? a.chan_valid + (int64_t)b * C_ : nullptr;
   const float sc2 = a.sm_scale * kLog2e;           // scores live in the base-2 domain
 
-  // this lane's query rows
-  int cq[QB];
-  bool qok[QB];
-  const bf16_t* qrow[QB];
+  // =========================== setup: Qu, channel bias tile, Ec ===========================
+  bf16x8 Qu[KS];
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    cq[qb] = (cb0 + qb) * 32 + ln;
-    qok[qb] = active && cq[qb] < C_;
-    qrow[qb] = qbase + (int64_t)(qok[qb] ? tq * C_ + cq[qb] : 0) * a.q_stride_n;
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d0 = ks * 16 + hh * 8;
+    u32x4 raw = {0u, 0u, 0u, 0u};
+    if (qok) raw = *(const u32x4*)(qrow + d0);
+    Qu[ks] = make_qfrag(raw, bu + d0, sc2);
   }
 
-  // =========================== setup: Qu, channel bias tile, Ec ===========================
-  bf16x8 Qu[QB][KS];
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int d0 = ks * 16 + hh * 8;
-      u32x4 raw = {0u, 0u, 0u, 0u};
-      if (qok[qb]) raw = *(const u32x4*)(qrow[qb] + d0);
-      Qu[qb][ks] = make_qfrag(raw, bu + d0, sc2);
-    }
-
-  f32x16 Bc[QB][NCT];        // channel-bias tile, [ck][q] in accumulator layout; -inf = masked key
+  f32x16 Bc[NCT];            // channel-bias tile, [ck][q] in accumulator layout; -inf = masked key
   {
-    float* scr = setup_all + wave * (CP * QW);
+    float* scr = setup_all + wave * (CP * 32);
+    f32x16 sct[NCT];
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-      f32x16 sct[NCT];
+    for (int t = 0; t < NCT; ++t)
 #pragma unroll
-      for (int t = 0; t < NCT; ++t)
+      for (int i = 0; i < 16; ++i) sct[t][i] = 0.f;
+    if (has_chan) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) sct[t][i] = 0.f;
-      if (has_chan) {
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d0 = ks * 16 + hh * 8;
+        u32x4 raw = {0u, 0u, 0u, 0u};
+        if (qok) raw = *(const u32x4*)(qrow + d0);
+        const bf16x8 qz = make_qfrag(raw, bz + d0, sc2);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const int d0 = ks * 16 + hh * 8;
-          u32x4 raw = {0u, 0u, 0u, 0u};
-          if (qok[qb]) raw = *(const u32x4*)(qrow[qb] + d0);
-          const bf16x8 qz = make_qfrag(raw, bz + d0, sc2);
-#pragma unroll
-          for (int t = 0; t < NCT; ++t) {
-            const int j = t * 32 + ln;
-            u32x4 er = {0u, 0u, 0u, 0u};
-            if (j < C_) er = *(const u32x4*)(kchan + (int64_t)j * DH + d0);
-            sct[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(er), qz, sct[t], 0, 0, 0);
-          }
+        for (int t = 0; t < NCT; ++t) {
+          const int j = t * 32 + ln;
+          u32x4 er = {0u, 0u, 0u, 0u};
+          if (j < C_) er = *(const u32x4*)(kchan + (int64_t)j * DH + d0);
+          sct[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(er), qz, sct[t], 0, 0, 0);
         }
       }
-#pragma unroll
-      for (int t = 0; t < NCT; ++t)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int j = t * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
-          scr[j * QW + qb * 32 + ln] = sct[t][i];
-        }
     }
+#pragma unroll
+    for (int t = 0; t < NCT; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int j = t * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
+        scr[j * 32 + ln] = sct[t][i];
+      }
     wave_lds_sync();
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb)
+    for (int t = 0; t < NCT; ++t)
 #pragma unroll
-      for (int t = 0; t < NCT; ++t)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int ck = t * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
-          const bool kv = ck < C_ && (!valid || valid[ck] != 0);
-          int j = chan_row(cq[qb], ck, C_);
-          j = j < 0 ? 0 : j;                   // padded query rows: any in-range row will do
-          const float val = scr[j * QW + qb * 32 + ln];
-          Bc[qb][t][i] = kv ? val : -INFINITY;
-        }
+      for (int i = 0; i < 16; ++i) {
+        const int ck = t * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
+        const bool kv = ck < C_ && (!valid || valid[ck] != 0);
+        int j = chan_row(cq, ck, C_);
+        j = j < 0 ? 0 : j;                     // padded query rows: any in-range row will do
+        const float val = scr[j * 32 + ln];
+        Bc[t][i] = kv ? val : -INFINITY;
+      }
   }
 
-  float mc[QB], sumEc[QB];
-  bf16x8 Ec[QB][NCT][2];     // exp2(Bc - mc) as PV B-operand fragments
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
+  float mc, sumEc;
+  bf16x8 Ec[NCT][2];         // exp2(Bc - mc) as PV B-operand fragments
+  {
     float mx = -INFINITY;
 #pragma unroll
     for (int t = 0; t < NCT; ++t)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, Bc[qb][t][i]);
-    mx = xhalf_max(mx);
-    mc[qb] = mx;
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, Bc[t][i]);
+    mc = xhalf_max(mx);
     float se = 0.f;
 #pragma unroll
     for (int t = 0; t < NCT; ++t) {
       f32x16 e;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        e[i] = fast_exp2(Bc[qb][t][i] - mx);
+        e[i] = fast_exp2(Bc[t][i] - mc);
         se += e[i];
       }
-      Ec[qb][t][0] = pack8(e, 0);
-      Ec[qb][t][1] = pack8(e, 8);
+      Ec[t][0] = pack8(e, 0);
+      Ec[t][1] = pack8(e, 8);
     }
-    sumEc[qb] = se;           // partial: this half-wave's keys only
+    sumEc = se;               // partial: this half-wave's keys only
   }
 
-  // running soft-max state, per query (lane); l is a per-half-wave partial sum
-  float m_run[QB], l_run[QB];
-  f32x16 acc[QB][MT];
+  // running soft-max state of this lane's query; l is a per-half-wave partial sum
+  float m_run = -INFINITY, l_run = 0.f;
+  f32x16 acc[MT];
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    m_run[qb] = -INFINITY;
-    l_run[qb] = 0.f;
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int i = 0; i < 16; ++i) acc[mt][i] = 0.f;
+
+  // =========================== tile ring ===========================
+  // Wave-load li of a tile covers bytes [li*1024, li*1024+1024): lane L delivers physical chunk
+  // li*64+L, i.e. row (li*64+L)/CHUNKS; the logical chunk it fetches is un-swizzled here.  Rows of
+  // padded or absent channels are never loaded: the ring is zero-filled once, below.
+  int k_off[G::LPW], v_off[G::LPW];
+  bool ld_ok[G::LPW];
+  int n_issue = 0;                                // wave loads this wave really issues per tile
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[qb][mt][i] = 0.f;
+  for (int i = 0; i < G::LPW; ++i) {
+    const int li = wave + NW * i;
+    const int pc = li * 64 + lane;
+    const int row = pc / CHUNKS, phys = pc % CHUNKS;
+    ld_ok[i] = li < G::WLOADS && row < C_ && (!valid || valid[row] != 0);
+    k_off[i] = (int)(row * a.k_stride_n) + ((phys ^ swz_k<DH>(row)) << 3);
+    v_off[i] = (int)(row * a.v_stride_n) + ((phys ^ swz_v<DH>(row)) << 3);
+    if (__ballot(ld_ok[i]) != 0ull) ++n_issue;
   }
-
-  __syncthreads();           // setup scratch aliases the K/V buffers
-
-  // =========================== K/V staging ===========================
-  u32x4 vreg[G::VPT][4];
-  u32x4 kreg[G::KPT];
   auto need_k = [&](int tk) -> bool {
     return has_content && (W <= 0 || tk >= tq0 - W || tq_hi == T_ - 1);
   };
-  auto load_tile = [&](int tk, bool with_k) {
+  auto issue_tile = [&](int tk, bool with_k) {
+    unsigned char* stage = smem_raw + (tk % STAGES) * G::STAGE_BYTES;
+    const bf16_t* vsrc = vbase + (int64_t)tk * C_ * a.v_stride_n;
+    const bf16_t* ksrc = kbase + (int64_t)tk * C_ * a.k_stride_n;
 #pragma unroll
-    for (int i = 0; i < G::VPT; ++i) {
-      const int task = tid + 256 * i;
-      if (task < G::NV) {
-        const int quad = task / (DH / 8), seg = task % (DH / 8);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int ck = quad * 4 + r;
-          u32x4 x = {0u, 0u, 0u, 0u};
-          if (ck < C_ && (!valid || valid[ck] != 0))
-            x = *(const u32x4*)(vbase + (int64_t)(tk * C_ + ck) * a.v_stride_n + seg * 8);
-          vreg[i][r] = x;
-        }
-      }
+    for (int i = 0; i < G::LPW; ++i) {
+      const int li = wave + NW * i;
+      if (ld_ok[i])
+        __builtin_amdgcn_global_load_lds((const GLOBAL_PTR(void))(vsrc + v_off[i]),
+                                         (LDS_PTR(void))(stage + G::TILE_BYTES + li * 1024), 16, 0, 0);
     }
     if (with_k) {
 #pragma unroll
-      for (int i = 0; i < G::KPT; ++i) {
-        const int c = tid + 256 * i;
-        if (c < G::NKC) {
-          const int ck = c / (DH / 8), seg = c % (DH / 8);
-          u32x4 x = {0u, 0u, 0u, 0u};
-          if (ck < C_ && (!valid || valid[ck] != 0))
-            x = *(const u32x4*)(kbase + (int64_t)(tk * C_ + ck) * a.k_stride_n + seg * 8);
-          kreg[i] = x;
-        }
-      }
-    }
-  };
-  auto store_tile = [&](int buf, bool with_k) {
-    bf16_t* vdst = Vt + buf * G::V_ELEMS;
-#pragma unroll
-    for (int i = 0; i < G::VPT; ++i) {
-      const int task = tid + 256 * i;
-      if (task < G::NV) {
-        const int quad = task / (DH / 8), seg = task % (DH / 8);
-        const int key0 = quad * 4;
-        const int oct = (key0 >> 4) * 2 + ((key0 >> 2) & 1);   // 16-key group, half-wave
-        const int jhalf = (key0 >> 3) & 1;
-        bf16_t* dst = vdst + ((int64_t)oct * DH + seg * 8) * 8 + jhalf * 4;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          const uint32_t x0 = vreg[i][0][w], x1 = vreg[i][1][w], x2 = vreg[i][2][w], x3 = vreg[i][3][w];
-          u32x2 lo, hi;
-          lo.x = __builtin_amdgcn_perm(x1, x0, 0x05040100u);
-          lo.y = __builtin_amdgcn_perm(x3, x2, 0x05040100u);
-          hi.x = __builtin_amdgcn_perm(x1, x0, 0x07060302u);
-          hi.y = __builtin_amdgcn_perm(x3, x2, 0x07060302u);
-          *(u32x2*)(dst + (2 * w) * 8) = lo;
-          *(u32x2*)(dst + (2 * w + 1) * 8) = hi;
-        }
-      }
-    }
-    if (with_k) {
-      bf16_t* kdst = Ks + buf * G::K_ELEMS;
-#pragma unroll
-      for (int i = 0; i < G::KPT; ++i) {
-        const int c = tid + 256 * i;
-        if (c < G::NKC) {
-          const int ck = c / (DH / 8), seg = c % (DH / 8);
-          *(u32x4*)(kdst + ck * KPITCH + seg * 8) = kreg[i];
-        }
+      for (int i = 0; i < G::LPW; ++i) {
+        const int li = wave + NW * i;
+        if (ld_ok[i])
+          __builtin_amdgcn_global_load_lds((const GLOBAL_PTR(void))(ksrc + k_off[i]),
+                                           (LDS_PTR(void))(stage + li * 1024), 16, 0, 0);
       }
     }
   };
 
-  load_tile(0, need_k(0));
-  store_tile(0, need_k(0));
-  __syncthreads();
+  lds_barrier();             // setup scratch aliases the ring
+  {
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    for (int i = tid * 16; i < G::RING_BYTES; i += G::THREADS * 16) *(u32x4*)(smem_raw + i) = zero;
+  }
+  lds_barrier();
 
-  float* Stb = Stb_all + wave * (32 * QW);
+  // prologue: tiles 0 .. STAGES-2 in flight
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s)
+    if (s <= tq_hi) issue_tile(s, need_k(s));
+
+  float* Stb = Stb_all + wave * (32 * 32);
   const bool last_row = tq == T_ - 1;
   auto is_far = [&](int tk) -> bool {
     return !has_content || (W > 0 && !last_row && tq - tk > W);
   };
 
+  // per-lane pieces of the LDS fragment addresses
+  //   K fragment (t, ks): row 32t+ln, logical chunk 2ks+hh
+  //   V^T fragment (t, s, mt), read rd: row 32t+16s+8rd+4hh+e, dh 32mt+16grp+4a  (transposing read)
+  const int tr_e = (ln & 15) >> 2, tr_a = ln & 3, tr_grp = ln >> 4;
+
   // =========================== main loop over key time steps ===========================
   for (int tk = 0; tk <= tq_hi; ++tk) {
-    const int cur = tk & 1;
-    const bool more = tk + 1 <= tq_hi;
-    const bool nk = more && need_k(tk + 1);
-    if (more) load_tile(tk + 1, nk);
+    // tile tk has landed once at most the loads of the younger tiles are still in flight
+    {
+      int younger = 0;
+#pragma unroll
+      for (int s = 1; s <= STAGES - 2; ++s)
+        if (tk + s <= tq_hi) younger += n_issue * (need_k(tk + s) ? 2 : 1);
+      wait_vmcnt(younger);
+    }
+    lds_barrier();            // tile tk visible to all; everyone is done with tile tk-1's buffer
+    if (tk + STAGES - 1 <= tq_hi) issue_tile(tk + STAGES - 1, need_k(tk + STAGES - 1));
 
     // ---- every 32 key steps: time-bias slab St[j][q] for the next 32 steps -> LDS, and one
     //      soft-max rescale that covers all far steps of the slab
     if ((tk & 31) == 0 && active) {
       const int j0 = time_row(tq, tk, T_);
+      f32x16 stc;
 #pragma unroll
-      for (int qb = 0; qb < QB; ++qb) {
-        f32x16 stc;
+      for (int i = 0; i < 16; ++i) stc[i] = 0.f;
+      if (has_time) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) stc[i] = 0.f;
-        if (has_time) {
-#pragma unroll
-          for (int ks = 0; ks < KS; ++ks) {
-            const int d0 = ks * 16 + hh * 8;
-            u32x4 raw = {0u, 0u, 0u, 0u};
-            if (qok[qb]) raw = *(const u32x4*)(qrow[qb] + d0);
-            const bf16x8 qv = make_qfrag(raw, bv + d0, sc2);
-            const int j = j0 + ln;
-            u32x4 rr = {0u, 0u, 0u, 0u};
-            if (j >= 0 && j < T_) rr = *(const u32x4*)(ktime + (int64_t)j * DH + d0);
-            stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(rr), qv, stc, 0, 0, 0);
-          }
+        for (int ks = 0; ks < KS; ++ks) {
+          const int d0 = ks * 16 + hh * 8;
+          u32x4 raw = {0u, 0u, 0u, 0u};
+          if (qok) raw = *(const u32x4*)(qrow + d0);
+          const bf16x8 qv = make_qfrag(raw, bv + d0, sc2);
+          const int j = j0 + ln;
+          u32x4 rr = {0u, 0u, 0u, 0u};
+          if (j >= 0 && j < T_) rr = *(const u32x4*)(ktime + (int64_t)j * DH + d0);
+          stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(rr), qv, stc, 0, 0, 0);
         }
-        float cm = -INFINITY;
+      }
+      float cm = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int jj = (i >> 2) * 8 + hh * 4 + (i & 3);
-          Stb[jj * QW + qb * 32 + ln] = stc[i];
-          const int tkk = tk + jj;
-          if (tkk <= tq && is_far(tkk)) cm = fmaxf(cm, stc[i]);
-        }
-        cm = xhalf_max(cm);
-        if (cm > -INFINITY) {
-          const float m_new = fmaxf(m_run[qb], cm + mc[qb]);
-          const float alpha = fast_exp2(m_run[qb] - m_new);
-          m_run[qb] = m_new;
-          l_run[qb] *= alpha;
+      for (int i = 0; i < 16; ++i) {
+        const int jj = (i >> 2) * 8 + hh * 4 + (i & 3);
+        Stb[jj * 32 + ln] = stc[i];
+        const int tkk = tk + jj;
+        if (tkk <= tq && is_far(tkk)) cm = fmaxf(cm, stc[i]);
+      }
+      cm = xhalf_max(cm);
+      if (cm > -INFINITY) {
+        const float m_new = fmaxf(m_run, cm + mc);
+        const float alpha = fast_exp2(m_run - m_new);
+        m_run = m_new;
+        l_run *= alpha;
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) acc[qb][mt][i] *= alpha;
-        }
+          for (int i = 0; i < 16; ++i) acc[mt][i] *= alpha;
       }
       wave_lds_sync();
     }
 
     if (active && tk <= tq) {
-      const bf16_t* vt = Vt + cur * G::V_ELEMS;
-      float st[QB];
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb) st[qb] = Stb[(tk & 31) * QW + qb * 32 + ln];
+      const unsigned char* stage = smem_raw + (tk % STAGES) * G::STAGE_BYTES;
+      const unsigned char* vt = stage + G::TILE_BYTES;
+      const float st = Stb[(tk & 31) * 32 + ln];
+
+      // V^T fragment: two transposing reads of 4 keys each
+      auto v_frag = [&](int t, int s, int mt) -> bf16x8 {
+        const int chunk = 4 * mt + 2 * tr_grp + (tr_a >> 1);
+        bf16x4 lo, hi;
+        {
+          const int row = 32 * t + 16 * s + 4 * hh + tr_e;
+          const unsigned char* p = vt + row * ROWB + ((chunk ^ swz_v<DH>(row)) << 4) + ((tr_a & 1) << 3);
+          lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((LDS_PTR(bf16x4))p);
+        }
+        {
+          const int row = 32 * t + 16 * s + 8 + 4 * hh + tr_e;
+          const unsigned char* p = vt + row * ROWB + ((chunk ^ swz_v<DH>(row)) << 4) + ((tr_a & 1) << 3);
+          hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((LDS_PTR(bf16x4))p);
+        }
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      };
 
       if (is_far(tk)) {
         // ------------------------------ far tile ------------------------------
-        f32x16 tmp[QB][MT];
+        f32x16 tmp[MT];
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) tmp[qb][mt][i] = 0.f;
+          for (int i = 0; i < 16; ++i) tmp[mt][i] = 0.f;
 #pragma unroll
         for (int t = 0; t < NCT; ++t)
 #pragma unroll
-          for (int s = 0; s < 2; ++s) {
-            const int oct = (t * 2 + s) * 2 + hh;
-            bf16x8 va[MT];
+          for (int s = 0; s < 2; ++s)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
-              va[mt] = *(const bf16x8*)(vt + ((int64_t)oct * DH + mt * 32 + ln) * 8);
+              tmp[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(t, s, mt), Ec[t][s], tmp[mt], 0, 0, 0);
+        const float et = fast_exp2(st + mc - m_run);
+        l_run += et * sumEc;
 #pragma unroll
-            for (int qb = 0; qb < QB; ++qb)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-              for (int mt = 0; mt < MT; ++mt)
-                tmp[qb][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[mt], Ec[qb][t][s], tmp[qb][mt], 0, 0, 0);
-          }
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) {
-          const float et = fast_exp2(st[qb] + mc[qb] - m_run[qb]);
-          l_run[qb] += et * sumEc[qb];
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[qb][mt][i] += et * tmp[qb][mt][i];
-        }
+          for (int i = 0; i < 16; ++i) acc[mt][i] += et * tmp[mt][i];
       } else {
         // ------------------------------ near tile ------------------------------
-        const bf16_t* ks_ = Ks + cur * G::K_ELEMS;
-        f32x16 S[QB][NCT];
+        f32x16 S[NCT];
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-          for (int t = 0; t < NCT; ++t) S[qb][t] = Bc[qb][t];
+        for (int t = 0; t < NCT; ++t) S[t] = Bc[t];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
           for (int t = 0; t < NCT; ++t) {
-            const bf16x8 ka = *(const bf16x8*)(ks_ + (t * 32 + ln) * KPITCH + ks * 16 + hh * 8);
-#pragma unroll
-            for (int qb = 0; qb < QB; ++qb)
-              S[qb][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, Qu[qb][ks], S[qb][t], 0, 0, 0);
+            const int row = t * 32 + ln;
+            const bf16x8 ka = *(const bf16x8*)(stage + row * ROWB + (((2 * ks + hh) ^ swz_k<DH>(row)) << 4));
+            S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, Qu[ks], S[t], 0, 0, 0);
           }
-        bf16x8 P[QB][NCT][2];
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) {
-          float rmax = -INFINITY;
-#pragma unroll
-          for (int t = 0; t < NCT; ++t)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) rmax = fmaxf(rmax, S[qb][t][i]);
-          rmax = xhalf_max(rmax);
-          const float m_new = fmaxf(m_run[qb], rmax + st[qb]);
-          const float alpha = fast_exp2(m_run[qb] - m_new);
-          const float off = st[qb] - m_new;
-          float ls = 0.f;
-#pragma unroll
-          for (int t = 0; t < NCT; ++t) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const float p = fast_exp2(S[qb][t][i] + off);
-              S[qb][t][i] = p;
-              ls += p;
-            }
-            P[qb][t][0] = pack8(S[qb][t], 0);
-            P[qb][t][1] = pack8(S[qb][t], 8);
-          }
-          m_run[qb] = m_new;
-          l_run[qb] = l_run[qb] * alpha + ls;
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[qb][mt][i] *= alpha;
-        }
+        float rmax = -INFINITY;
 #pragma unroll
         for (int t = 0; t < NCT; ++t)
 #pragma unroll
-          for (int s = 0; s < 2; ++s) {
-            const int oct = (t * 2 + s) * 2 + hh;
-            bf16x8 va[MT];
+          for (int i = 0; i < 16; ++i) rmax = fmaxf(rmax, S[t][i]);
+        rmax = xhalf_max(rmax);
+        const float m_new = fmaxf(m_run, rmax + st);
+        const float off = st - m_new;
+        float ls = 0.f;
+        bf16x8 P[NCT][2];
+#pragma unroll
+        for (int t = 0; t < NCT; ++t) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const float p = fast_exp2(S[t][i] + off);
+            S[t][i] = p;
+            ls += p;
+          }
+          P[t][0] = pack8(S[t], 0);
+          P[t][1] = pack8(S[t], 8);
+        }
+        if (__ballot(m_new > m_run) != 0ull) {      // skip the rescale when no lane's max moved
+          const float alpha = fast_exp2(m_run - m_new);
+          l_run *= alpha;
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[mt][i] *= alpha;
+        }
+        m_run = m_new;
+        l_run += ls;
+#pragma unroll
+        for (int t = 0; t < NCT; ++t)
+#pragma unroll
+          for (int s = 0; s < 2; ++s)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
-              va[mt] = *(const bf16x8*)(vt + ((int64_t)oct * DH + mt * 32 + ln) * 8);
-#pragma unroll
-            for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-              for (int mt = 0; mt < MT; ++mt)
-                acc[qb][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[mt], P[qb][t][s], acc[qb][mt], 0, 0, 0);
-          }
+              acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(t, s, mt), P[t][s], acc[mt], 0, 0, 0);
       }
     }
-
-    if (more) store_tile(cur ^ 1, nk);
-    __syncthreads();
   }
 
   // =========================== epilogue ===========================
+  {
+    const float ltot = l_run + __shfl_xor(l_run, 32);
+    if (qok) {
+      const float inv = 1.f / ltot;
+      const int64_t n = (int64_t)tq * C_ + cq;
+      bf16_t* orow = (bf16_t*)a.o + b * a.o_stride_b + h * a.o_stride_h + n * a.o_stride_n;
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    const float ltot = l_run[qb] + __shfl_xor(l_run[qb], 32);
-    if (!qok[qb]) continue;
-    const float inv = 1.f / ltot;
-    const int64_t n = (int64_t)tq * C_ + cq[qb];
-    bf16_t* orow = (bf16_t*)a.o + b * a.o_stride_b + h * a.o_stride_h + n * a.o_stride_n;
+      for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int a4 = 0; a4 < 4; ++a4) {
-        const int d0 = mt * 32 + a4 * 8 + hh * 4;
-        u32x2 w;
-        const float x0 = acc[qb][mt][a4 * 4 + 0] * inv, x1 = acc[qb][mt][a4 * 4 + 1] * inv;
-        const float x2 = acc[qb][mt][a4 * 4 + 2] * inv, x3 = acc[qb][mt][a4 * 4 + 3] * inv;
-        w.x = (uint32_t)f32_to_bf16(x0) | ((uint32_t)f32_to_bf16(x1) << 16);
-        w.y = (uint32_t)f32_to_bf16(x2) | ((uint32_t)f32_to_bf16(x3) << 16);
-        *(u32x2*)(orow + d0) = w;
-      }
-    if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * ((int64_t)T_ * C_) + n] = m_run[qb] + log2f(ltot);
+        for (int a4 = 0; a4 < 4; ++a4) {
+          const int d0 = mt * 32 + a4 * 8 + hh * 4;
+          u32x2 w;
+          const float x0 = acc[mt][a4 * 4 + 0] * inv, x1 = acc[mt][a4 * 4 + 1] * inv;
+          const float x2 = acc[mt][a4 * 4 + 2] * inv, x3 = acc[mt][a4 * 4 + 3] * inv;
+          w.x = (uint32_t)f32_to_bf16(x0) | ((uint32_t)f32_to_bf16(x1) << 16);
+          w.y = (uint32_t)f32_to_bf16(x2) | ((uint32_t)f32_to_bf16(x3) << 16);
+          *(u32x2*)(orow + d0) = w;
+        }
+      if (a.lse && hh == 0)
+        a.lse[((int64_t)b * a.H + h) * ((int64_t)T_ * C_) + n] = m_run + log2f(ltot);
+    }
   }
 }
 
-template <int DH, int NCT, int QB>
+template <int DH, int NCT, int NW, int STAGES>
 static int launch_cfg(const mvpa_fwd_args* a, hipStream_t stream) {
-  using G = Cfg<DH, NCT, QB>;
-  auto kern = mvpa_mfma_kernel<DH, NCT, QB>;
+  using G = Cfg<DH, NCT, NW, STAGES>;
+  static_assert(G::LDS_BYTES <= 160 * 1024, "LDS budget");
+  auto kern = mvpa_mfma_kernel<DH, NCT, NW, STAGES>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)G::LDS_BYTES);
   const int nt = (a->T + G::TQW - 1) / G::TQW;
   dim3 grid((unsigned)(nt * a->B * a->H));
-  hipLaunchKernelGGL(kern, grid, dim3(256), G::LDS_BYTES, stream, *a);
+  hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), G::LDS_BYTES, stream, *a);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
-}
-
-template <int DH>
-static int launch_dh(const mvpa_fwd_args* a, hipStream_t stream) {
-  constexpr int QB2 = DH <= 64 ? 2 : 1;
-  if (a->C <= 32) return launch_cfg<DH, 1, 1>(a, stream);
-  if (a->C <= 64) return launch_cfg<DH, 2, QB2>(a, stream);
-  return launch_cfg<DH, 4, 1>(a, stream);
 }
 
 }  // namespace mvpa
@@ -568,14 +553,28 @@ int mvpa_mfma_supported(const mvpa_fwd_args* a) {
                     a->k_stride_n | a->v_stride_b | a->v_stride_h | a->v_stride_n |
                     a->o_stride_b | a->o_stride_h | a->o_stride_n;
   if ((p & 15) || (s & 7)) return 0;
+  // per-sample element offsets are kept in 32 bits inside the kernel
+  const int64_t n = (int64_t)a->T * a->C;
+  if (n * a->k_stride_n >= ((int64_t)1 << 31) || n * a->v_stride_n >= ((int64_t)1 << 31)) return 0;
   return 1;
 }
 
 int mvpa_launch_mfma(const mvpa_fwd_args* a, hipStream_t stream) {
+  using namespace mvpa;
+  const int nct = a->C <= 32 ? 1 : a->C <= 64 ? 2 : 4;
   switch (a->Dh) {
-    case 32: return mvpa::launch_dh<32>(a, stream);
-    case 64: return mvpa::launch_dh<64>(a, stream);
-    case 128: return mvpa::launch_dh<128>(a, stream);
+    case 32:
+      if (nct == 1) return launch_cfg<32, 1, 8, 4>(a, stream);
+      if (nct == 2) return launch_cfg<32, 2, 8, 4>(a, stream);
+      return launch_cfg<32, 4, 8, 4>(a, stream);
+    case 64:
+      if (nct == 1) return launch_cfg<64, 1, 8, 4>(a, stream);
+      if (nct == 2) return launch_cfg<64, 2, 8, 4>(a, stream);
+      return launch_cfg<64, 4, 4, 3>(a, stream);
+    case 128:
+      if (nct == 1) return launch_cfg<128, 1, 4, 4>(a, stream);
+      if (nct == 2) return launch_cfg<128, 2, 4, 3>(a, stream);
+      return launch_cfg<128, 4, 4, 2>(a, stream);
   }
   return MVPA_ERR_UNSUPPORTED;
 }
