@@ -491,22 +491,64 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma_kernel(mvpa_fwd_args a) {
   // the number of younger loads is a compile-time constant.  The loop is unrolled over the ring so
   // that stage addresses are immediates.  It stops early enough that every tile it issues is
   // still V-only; the generic loop below takes over from there.
+  // Within a step the accumulate acc += et * tmp of the PREVIOUS step is deferred to here, so that
+  // it fills the LDS latency of this step's first fragments instead of trailing the MFMAs.
   int tk = 0;
   {
     // uniform over the workgroup (every wave must reach the same barriers): all of these steps
     // are at or before tq0, hence visible to every query of the workgroup
     const int fast_end = min(tk_near - (STAGES - 1), tq0 + 1);
     const int n_groups = fast_end > 0 ? fast_end / STAGES : 0;
+    f32x16 ptmp[MT];                       // V^T Ec^T of the previous step, not yet accumulated
+    float pet = 0.f;                       // its weight
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) ptmp[mt][i] = 0.f;
+    auto flush = [&]() {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][i] += pet * ptmp[mt][i];
+      pet = 0.f;
+    };
     for (int grp = 0; grp < n_groups; ++grp) {
 #pragma unroll
       for (int s = 0; s < STAGES; ++s, ++tk) {
         wait_vmcnt_imm<(STAGES - 2) * G::LPW>();
         lds_barrier();
         issue_tile(tk + STAGES - 1, (s + STAGES - 1) % STAGES, false);
-        if ((tk & 31) == 0 && active) time_slab(tk);
-        if (active) far_step(smem_raw + s * G::STAGE_BYTES, tk);
+        if ((tk & 31) == 0 && active) {
+          flush();
+          time_slab(tk);
+        }
+        if (active) {
+          const unsigned char* stage = smem_raw + s * G::STAGE_BYTES;
+          const float st = Stb[(tk & 31) * 32 + ln];
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            bf16x8 vf[NCT * 2];
+#pragma unroll
+            for (int t = 0; t < NCT; ++t)
+#pragma unroll
+              for (int s2 = 0; s2 < 2; ++s2) vf[t * 2 + s2] = v_frag(stage, t, s2, mt);
+            // previous step's contribution to this output tile, while the fragments arrive
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[mt][i] += pet * ptmp[mt][i];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) ptmp[mt][i] = 0.f;
+#pragma unroll
+            for (int t = 0; t < NCT; ++t)
+#pragma unroll
+              for (int s2 = 0; s2 < 2; ++s2)
+                ptmp[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[t * 2 + s2], Ec[t][s2], ptmp[mt], 0, 0, 0);
+          }
+          pet = fast_exp2(st + mc - m_run);
+          l_run += pet * sumEc;
+        }
       }
     }
+    flush();
   }
 
   // =========================== generic loop: remaining key steps ===========================
