@@ -148,18 +148,21 @@ int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M, int64_t N
 
 /* RMSNorm over the last dim: y = x * rsqrt(mean(x^2)+eps) * weight
  * (models/mvpformer.py:108,133,167,380; models/fftencoder.py:67,93).
- * in_dtype/out_dtype: MVPA_F32 | MVPA_BF16; weight is fp32. */
+ * in_dtype/out_dtype: MVPA_F32 | MVPA_BF16; weight is fp32; ldx/ldy are row pitches in
+ * elements (>= cols). */
 int mvpa_rmsnorm(const void* x, const float* weight, void* y, int64_t rows, int32_t cols,
-                 float eps, int32_t in_dtype, int32_t out_dtype, void* stream);
+                 int64_t ldx, int64_t ldy, float eps, int32_t in_dtype, int32_t out_dtype,
+                 void* stream);
 
 /* out = a + b + c elementwise, bf16 (models/mvpformer.py:147 residual + mlp + attn). */
 int mvpa_add3_bf16(const void* a, const void* b, const void* c, void* out, int64_t n,
                    void* stream);
 
 /* Multilevel db4 analysis with periodic extension of fp32 rows x[M,L] into
- * coeffs[M,dwt_size] ordered [cA_L, cD_L, ..., cD_1] (models/fftencoder.py:80-88). */
+ * coeffs[M,dwt_size] (row pitch ldc >= dwt_size) ordered [cA_L, cD_L, ..., cD_1]
+ * (models/fftencoder.py:80-88). */
 int mvpa_wavedec_db4(const float* x, float* coeffs, int64_t M, int32_t L, int32_t levels,
-                     int32_t dwt_size, void* stream);
+                     int32_t dwt_size, int64_t ldc, void* stream);
 
 #ifdef __cplusplus
 }

@@ -163,11 +163,12 @@ __global__ __launch_bounds__(256) void linear_bf16_kernel(const bf16_t* __restri
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const TI* __restrict__ x,
                                                       const float* __restrict__ w,
-                                                      TO* __restrict__ y, int cols, float eps) {
+                                                      TO* __restrict__ y, int cols, int64_t ldx,
+                                                      int64_t ldy, float eps) {
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
-  const TI* xr = x + row * cols;
-  TO* yr = y + row * cols;
+  const TI* xr = x + row * ldx;
+  TO* yr = y + row * ldy;
   float ss = 0.f;
   for (int c = threadIdx.x; c < cols; c += 256) {
     const float v = io<TI>::load(xr + c);
@@ -203,7 +204,7 @@ __constant__ float kDb4Lo[8] = {-0.010597401784997278f, 0.032883011666982945f,
 
 __global__ __launch_bounds__(256) void wavedec_db4_kernel(const float* __restrict__ x,
                                                           float* __restrict__ out, int L,
-                                                          int levels, int dwt_size) {
+                                                          int levels, int dwt_size, int64_t ldc) {
   extern __shared__ float buf[];   // 2 * L floats
   float* cur = buf;
   float* nxt = buf + L;
@@ -216,7 +217,7 @@ __global__ __launch_bounds__(256) void wavedec_db4_kernel(const float* __restric
   for (int lv = 1; lv <= levels; ++lv) {
     const int m = (n + 7) >> 1;
     tail -= m;
-    float* det = out + row * dwt_size + tail;
+    float* det = out + row * ldc + tail;
     for (int k = threadIdx.x; k < m; k += 256) {
       float lo = 0.f, hi = 0.f;
 #pragma unroll
@@ -235,7 +236,7 @@ __global__ __launch_bounds__(256) void wavedec_db4_kernel(const float* __restric
     float* t = cur; cur = nxt; nxt = t;
     n = m;
   }
-  for (int k = threadIdx.x; k < n; k += 256) out[row * dwt_size + k] = cur[k];
+  for (int k = threadIdx.x; k < n; k += 256) out[row * ldc + k] = cur[k];
 }
 
 }  // namespace mvpa
@@ -263,20 +264,20 @@ extern "C" int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M
 }
 
 extern "C" int mvpa_rmsnorm(const void* x, const float* weight, void* y, int64_t rows,
-                            int32_t cols, float eps, int32_t in_dtype, int32_t out_dtype,
-                            void* stream) {
+                            int32_t cols, int64_t ldx, int64_t ldy, float eps, int32_t in_dtype,
+                            int32_t out_dtype, void* stream) {
   if (!x || !weight || !y) return MVPA_ERR_NULL;
-  if (rows <= 0 || cols <= 0) return MVPA_ERR_SHAPE;
+  if (rows <= 0 || cols <= 0 || ldx < cols || ldy < cols) return MVPA_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   dim3 grid((unsigned)rows), block(256);
   if (in_dtype == MVPA_F32 && out_dtype == MVPA_F32)
-    hipLaunchKernelGGL((rmsnorm_kernel<float, float>), grid, block, 0, s, (const float*)x, weight, (float*)y, cols, eps);
+    hipLaunchKernelGGL((rmsnorm_kernel<float, float>), grid, block, 0, s, (const float*)x, weight, (float*)y, cols, ldx, ldy, eps);
   else if (in_dtype == MVPA_F32 && out_dtype == MVPA_BF16)
-    hipLaunchKernelGGL((rmsnorm_kernel<float, bf16_t>), grid, block, 0, s, (const float*)x, weight, (bf16_t*)y, cols, eps);
+    hipLaunchKernelGGL((rmsnorm_kernel<float, bf16_t>), grid, block, 0, s, (const float*)x, weight, (bf16_t*)y, cols, ldx, ldy, eps);
   else if (in_dtype == MVPA_BF16 && out_dtype == MVPA_BF16)
-    hipLaunchKernelGGL((rmsnorm_kernel<bf16_t, bf16_t>), grid, block, 0, s, (const bf16_t*)x, weight, (bf16_t*)y, cols, eps);
+    hipLaunchKernelGGL((rmsnorm_kernel<bf16_t, bf16_t>), grid, block, 0, s, (const bf16_t*)x, weight, (bf16_t*)y, cols, ldx, ldy, eps);
   else if (in_dtype == MVPA_BF16 && out_dtype == MVPA_F32)
-    hipLaunchKernelGGL((rmsnorm_kernel<bf16_t, float>), grid, block, 0, s, (const bf16_t*)x, weight, (float*)y, cols, eps);
+    hipLaunchKernelGGL((rmsnorm_kernel<bf16_t, float>), grid, block, 0, s, (const bf16_t*)x, weight, (float*)y, cols, ldx, ldy, eps);
   else
     return MVPA_ERR_DTYPE;
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
@@ -293,14 +294,14 @@ extern "C" int mvpa_add3_bf16(const void* a, const void* b, const void* c, void*
 }
 
 extern "C" int mvpa_wavedec_db4(const float* x, float* coeffs, int64_t M, int32_t L,
-                                int32_t levels, int32_t dwt_size, void* stream) {
+                                int32_t levels, int32_t dwt_size, int64_t ldc, void* stream) {
   if (!x || !coeffs) return MVPA_ERR_NULL;
-  if (M <= 0 || L < 8 || levels < 1 || L > 16384) return MVPA_ERR_SHAPE;
+  if (M <= 0 || L < 8 || levels < 1 || L > 16384 || ldc < dwt_size) return MVPA_ERR_SHAPE;
   int n = L, total = 0;
   for (int lv = 0; lv < levels; ++lv) { n = (n + 7) >> 1; total += n; }
   total += n;
   if (total != dwt_size) return MVPA_ERR_SHAPE;
   hipLaunchKernelGGL(wavedec_db4_kernel, dim3((unsigned)M), dim3(256), 2 * L * sizeof(float),
-                     (hipStream_t)stream, x, coeffs, L, levels, dwt_size);
+                     (hipStream_t)stream, x, coeffs, L, levels, dwt_size, ldc);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }

@@ -1,0 +1,232 @@
+"""MVPFormer stack on the HIP library: config, parallel block, model, head and the inference
+wrapper, with the reference's class names, constructor arguments and state-dict keys
+(models/mvpformer.py:37-152, 155-402, 405-479, 596-607, 979-989) but without the training
+harness (no Lightning, no HF base classes).  Inference / eval only, bf16 on the GPU.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import nn
+
+import mvpa_hip
+from layers import MVPFormerGQAAttention, MVPFormerGQAFlashAttention
+from models import BrainDecider, BrainEncoder, BrainModel
+from models.fftencoder import RMSNorm
+
+
+class MVPFormerConfig:
+    """Same constructor arguments and attribute aliases as models/mvpformer.py:37-101."""
+
+    attribute_map = {
+        "hidden_size": "n_embd",
+        "max_position_embeddings": "n_positions",
+        "max_channel_embeddings": "n_channels",
+        "num_attention_heads": "n_head",
+        "num_hidden_layers": "n_layer",
+        "intermediate_size": "n_inner",
+        "hidden_act": "activation_function",
+    }
+
+    def __init__(self, n_positions=100, n_channels=128, n_embd=768, n_layer=12, n_head=12,
+                 n_inner=2048, n_head_kv=12, global_att=True, activation_function="silu",
+                 resid_pdrop=0.1, embd_pdrop=0.1, attn_pdrop=0.1, layer_norm_epsilon=0.00001,
+                 initializer_range=0.02, scale_attn_weights=True, use_cache=False,
+                 scale_attn_by_inverse_layer_idx=False, reorder_and_upcast_attn=False,
+                 lora=False, lora_alpha=16, lora_rank=8, lora_dropout=0, lora_merge=True):
+        self.n_positions, self.n_channels, self.n_embd = n_positions, n_channels, n_embd
+        self.n_layer, self.n_head, self.n_inner, self.n_head_kv = n_layer, n_head, n_inner, n_head_kv
+        self.global_att = global_att
+        self.activation_function = activation_function
+        self.resid_pdrop, self.embd_pdrop, self.attn_pdrop = resid_pdrop, embd_pdrop, attn_pdrop
+        self.layer_norm_epsilon = layer_norm_epsilon
+        self.initializer_range = initializer_range
+        self.scale_attn_weights = scale_attn_weights
+        self.use_cache = use_cache
+        self.scale_attn_by_inverse_layer_idx = scale_attn_by_inverse_layer_idx
+        self.reorder_and_upcast_attn = reorder_and_upcast_attn
+        self.pretraining_tp = 1
+        self.mlp_bias = False
+        self.lora, self.lora_alpha, self.lora_rank = lora, lora_alpha, lora_rank
+        self.lora_dropout, self.lora_merge = lora_dropout, lora_merge
+        self.add_cross_attention = False
+        self.output_attentions = False
+        self.output_hidden_states = False
+
+    def __getattr__(self, name):
+        amap = type(self).attribute_map
+        if name in amap:
+            return getattr(self, amap[name])
+        raise AttributeError(name)
+
+    @classmethod
+    def from_yaml(cls, path: str) -> "MVPFormerConfig":
+        """Read the gpt_config block of one of the reference's YAML files (configs/*.yaml:49-71)."""
+        import yaml
+        with open(path) as f:
+            doc = yaml.safe_load(f)
+        return cls(**doc["model"]["init_args"]["gpt_config"]["init_args"])
+
+
+class GatedMLP(nn.Module):
+    """down(silu(gate(x)) * up(x)), bias-free: the MLP the reference takes from the Llama family
+    (models/mvpformer.py:114).  gate and up run as ONE GEMM with the SiLU-multiply fused."""
+
+    def __init__(self, config):
+        super().__init__()
+        h, m = config.hidden_size, config.intermediate_size
+        self.gate_proj = nn.Linear(h, m, bias=False)
+        self.up_proj = nn.Linear(h, m, bias=False)
+        self.down_proj = nn.Linear(m, h, bias=False)
+        self._gu = None
+        self._gu_key = None
+
+    def _gate_up(self) -> torch.Tensor:
+        key = (self.gate_proj.weight.data_ptr(), self.gate_proj.weight._version,
+               self.up_proj.weight.data_ptr(), self.up_proj.weight._version)
+        if self._gu_key != key:
+            self._gu = torch.cat([self.gate_proj.weight, self.up_proj.weight], 0).detach().to(torch.bfloat16).contiguous()
+            self._gu_key = key
+        return self._gu
+
+    @torch.no_grad()
+    def forward(self, x):
+        mid = mvpa_hip.linear(x, self._gate_up(), gated=True)
+        return mvpa_hip.linear(mid, self.down_proj.weight.to(torch.bfloat16))
+
+
+class MVPFormerBlock(nn.Module):
+    """Parallel block: x + MLP(ln_1(x)) + Attn(ln_1(x)); ln_2 exists but is unused
+    (models/mvpformer.py:104-152)."""
+
+    def __init__(self, config, layer_idx=None, flash: bool = True):
+        super().__init__()
+        hidden_size = config.hidden_size
+        self.ln_1 = RMSNorm(hidden_size, eps=config.layer_norm_epsilon)
+        cls = MVPFormerGQAFlashAttention if flash else MVPFormerGQAAttention
+        self.attn = cls(config, layer_idx=layer_idx)
+        self.ln_2 = RMSNorm(hidden_size, eps=config.layer_norm_epsilon)
+        self.mlp = GatedMLP(config)
+
+    def forward(self, hidden_states, positional_embedding, channel_embedding, layer_past=None,
+                attention_mask=None, head_mask=None, encoder_hidden_states=None,
+                encoder_attention_mask=None, use_cache=False, output_attentions=False):
+        residual = hidden_states
+        hidden_states = self.ln_1(hidden_states)
+        attn_outputs = self.attn(hidden_states, positional_embedding, channel_embedding,
+                                 layer_past=layer_past, attention_mask=attention_mask,
+                                 head_mask=head_mask, use_cache=use_cache,
+                                 output_attentions=output_attentions)
+        attn_output = attn_outputs[0]
+        outputs = attn_outputs[1:]
+        mlp_output = self.mlp(hidden_states)
+        hidden_states = mvpa_hip.add3(residual, mlp_output, attn_output)
+        if use_cache:
+            outputs = (hidden_states,) + outputs
+        else:
+            outputs = (hidden_states,) + outputs[1:]
+        return outputs
+
+
+class MVPFormerModel(nn.Module):
+    """models/mvpformer.py:155-402 without the HF base class: h, ln_f, positional_embedding,
+    channel_embedding; forward(inputs_embeds=[B,T,C,E]) -> last_hidden_state [B,T,C,E]."""
+
+    def __init__(self, config, gradient_checkpointing=False, flash: bool = True):
+        super().__init__()
+        self.config = config
+        self.embed_dim = config.hidden_size
+        self.num_heads = config.num_attention_heads
+        self.num_kv_heads = config.n_head_kv
+        self.head_dim = self.embed_dim // self.num_heads
+        self.embed_kv_dim = self.head_dim * self.num_kv_heads
+        self.drop = nn.Dropout(config.embd_pdrop)
+        self.h = nn.ModuleList([MVPFormerBlock(config, layer_idx=i, flash=flash)
+                                for i in range(config.num_hidden_layers)])
+        self.ln_f = RMSNorm(self.embed_dim, eps=config.layer_norm_epsilon)
+        self.positional_embedding = nn.Embedding(config.max_position_embeddings, self.embed_dim)
+        self.channel_embedding = nn.Embedding(config.max_channel_embeddings, self.embed_dim)
+        self.gradient_checkpointing = gradient_checkpointing
+        self.apply(self._init_weights)
+
+    def _init_weights(self, module):
+        std = self.config.initializer_range                      # models/mvpformer.py:179-188
+        if isinstance(module, (nn.Linear, nn.Embedding)):
+            module.weight.data.normal_(mean=0.0, std=std)
+
+    @torch.no_grad()
+    def forward(self, input_ids=None, inputs_embeds=None, attention_mask=None, head_mask=None,
+                use_cache=None, output_attentions=None, **unused):
+        if inputs_embeds is None:
+            raise NotImplementedError
+        if self.training:
+            raise NotImplementedError("MVPFormer HIP stack: inference only; call .eval()")
+        bsz, t_len, c_len, _ = inputs_embeds.shape
+        device = inputs_embeds.device
+        position_ids = torch.arange(t_len, dtype=torch.long, device=device).unsqueeze(0)
+        channel_ids = torch.arange(c_len, dtype=torch.long, device=device).unsqueeze(0)
+        if attention_mask is not None:                           # models/mvpformer.py:262-268
+            dt = inputs_embeds.dtype
+            attention_mask = attention_mask.view(bsz, -1)[:, None, None, :].to(dtype=dt)
+            attention_mask = (1.0 - attention_mask) * torch.finfo(dt).min
+        position_embeds = self.positional_embedding(position_ids)
+        channel_embeds = self.channel_embedding(channel_ids)
+        hidden_states = inputs_embeds
+        for block in self.h:
+            hidden_states = block(hidden_states, position_embeds, channel_embeds,
+                                  attention_mask=attention_mask, use_cache=False)[0]
+        hidden_states = self.ln_f(hidden_states)
+        return hidden_states.view(bsz, t_len, c_len, -1)
+
+
+class MVPFormerHead(BrainDecider):
+    def __init__(self, size: int, size_out: Optional[int] = None) -> None:
+        super().__init__()
+        self.head = nn.Linear(size, size_out if size_out is not None else size, bias=False)
+
+    @torch.no_grad()
+    def forward(self, x: torch.Tensor):
+        if x.is_cuda and x.dtype == torch.bfloat16:
+            return mvpa_hip.linear(x, self.head.weight.to(torch.bfloat16))
+        return self.head(x)
+
+
+class HMVPFormer(BrainModel):
+    """Inference part of the reference's harness: encoder -> stack -> head
+    (models/mvpformer.py:405-479, 596-607, 749-764).  Sub-module names match the reference so
+    its `base_model` / `head_model` state dicts load key for key."""
+
+    def __init__(self, gpt_config: MVPFormerConfig, encoder: BrainEncoder, head: BrainDecider,
+                 flash: bool = True) -> None:
+        super().__init__()
+        self.gpt_config = gpt_config
+        self.mvpformer = MVPFormerModel(gpt_config, flash=flash)
+        self.head = head
+        self.encoder = encoder
+        self.seizure_embeddings = nn.Parameter(
+            torch.normal(mean=0, std=1.0 / encoder.size_input, size=(3, encoder.size_input)))
+
+    @torch.no_grad()
+    def _common_forward(self, batch: torch.Tensor, attention_mask=None):
+        """batch [B, n_seg, ch, len] -> (last_hidden_state [B,T,C,E], input_embeds [B,T,C,E])."""
+        bsz, seg_n, ch, seg = batch.shape
+        out_enc = self.encoder(batch.reshape(bsz * seg_n * ch, seg))
+        input_embeds = out_enc.view(bsz, seg_n, ch, -1)
+        out = self.mvpformer(inputs_embeds=input_embeds, attention_mask=attention_mask)
+        return out, input_embeds
+
+    @torch.no_grad()
+    def predict_next_segment(self, batch: torch.Tensor):
+        """Generative scoring of models/mvpformer.py:749-764: cosine similarity between the head's
+        prediction at segment t and the encoding of segment t+1, per channel."""
+        out, enc = self._common_forward(batch)
+        out = self.head(out)
+        return torch.cosine_similarity(enc[:, 1:].float(), out[:, :-1].float(), dim=-1)
+
+    @torch.no_grad()
+    def classify(self, batch: torch.Tensor):
+        """Classification scoring of models/mvpformer.py:947-953: head(mean over channels of the
+        last segment's hidden state)."""
+        out, _ = self._common_forward(batch)
+        return self.head(out[:, -1].float().mean(dim=1).to(out.dtype))

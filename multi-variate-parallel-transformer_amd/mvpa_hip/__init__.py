@@ -80,11 +80,11 @@ def load_library() -> ctypes.CDLL:
     lib.mvpa_linear_bf16.restype = ctypes.c_int
     lib.mvpa_linear_bf16.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, i32, vp]
     lib.mvpa_rmsnorm.restype = ctypes.c_int
-    lib.mvpa_rmsnorm.argtypes = [vp, vp, vp, i64, i32, f32, i32, i32, vp]
+    lib.mvpa_rmsnorm.argtypes = [vp, vp, vp, i64, i32, i64, i64, f32, i32, i32, vp]
     lib.mvpa_add3_bf16.restype = ctypes.c_int
     lib.mvpa_add3_bf16.argtypes = [vp, vp, vp, vp, i64, vp]
     lib.mvpa_wavedec_db4.restype = ctypes.c_int
-    lib.mvpa_wavedec_db4.argtypes = [vp, vp, i64, i32, i32, i32, vp]
+    lib.mvpa_wavedec_db4.argtypes = [vp, vp, i64, i32, i32, i32, i64, vp]
     if lib.mvpa_version() != 1:
         raise RuntimeError("libmvpa_hip ABI version mismatch")
     _lib = lib
@@ -244,16 +244,28 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = 
 
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5,
-            out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+            out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMSNorm over the last dim.  x may be a 2-D row-pitched view (unit last stride); `out`, if
+    given, is a 2-D tensor/view [rows, cols] with unit last stride."""
     lib = load_library()
     _need_cuda(x, weight)
-    xc = x.contiguous()
-    od = out_dtype or x.dtype
-    y = torch.empty(xc.shape, dtype=od, device=x.device)
-    cols = xc.shape[-1]
-    w = weight.to(torch.float32).contiguous()
-    _check(lib.mvpa_rmsnorm(xc.data_ptr(), w.data_ptr(), y.data_ptr(), xc.numel() // cols, cols,
-                            eps, _dtype_code(x.dtype), _dtype_code(od), _stream()))
+    cols = x.shape[-1]
+    if x.dim() == 2 and x.stride(-1) == 1:
+        x2 = x
+    else:
+        x2 = x.contiguous().view(-1, cols)
+    rows = x2.shape[0]
+    od = out_dtype or (out.dtype if out is not None else x.dtype)
+    if out is None:
+        y = torch.empty(x.shape, dtype=od, device=x.device)
+        y2 = y.view(-1, cols)
+    else:
+        y = y2 = out
+        assert out.dim() == 2 and out.shape == (rows, cols) and out.stride(-1) == 1
+    w = weight if weight.dtype == torch.float32 else weight.to(torch.float32)
+    _check(lib.mvpa_rmsnorm(x2.data_ptr(), w.contiguous().data_ptr(), y2.data_ptr(), rows, cols,
+                            x2.stride(0), y2.stride(0), eps, _dtype_code(x.dtype), _dtype_code(od),
+                            _stream()))
     return y
 
 
@@ -282,13 +294,15 @@ def dwt_sizes(size_input: int):
 
 
 def wavedec_db4(x: torch.Tensor, pitch: Optional[int] = None) -> torch.Tensor:
-    """x [M,L] float32 -> coefficients [M,dwt_size] float32, ordered [cA_L, cD_L, .., cD_1]."""
+    """x [M,L] float32 -> coefficients [M,dwt_size] float32, ordered [cA_L, cD_L, .., cD_1].
+    With `pitch` the result is a [M,dwt_size] view of a zero-filled [M,pitch] buffer."""
     lib = load_library()
     _need_cuda(x)
     x = x.to(torch.float32).contiguous()
     M, L = x.shape
     levels, sizes = dwt_sizes(L)
     total = sum(sizes)
-    out = torch.empty((M, total), dtype=torch.float32, device=x.device)
-    _check(lib.mvpa_wavedec_db4(x.data_ptr(), out.data_ptr(), M, L, levels, total, _stream()))
-    return out
+    ldc = total if pitch is None else pitch
+    buf = (torch.empty if ldc == total else torch.zeros)((M, ldc), dtype=torch.float32, device=x.device)
+    _check(lib.mvpa_wavedec_db4(x.data_ptr(), buf.data_ptr(), M, L, levels, total, ldc, _stream()))
+    return buf[:, :total]

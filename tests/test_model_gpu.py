@@ -1,0 +1,107 @@
+"""GPU checks of the attention layers and of the MVPFormer stack against the CPU oracle."""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from layers import MVPFormerGQAAttention, MVPFormerGQAFlashAttention
+from mvpa_hip.synthetic import make_ieeg
+from oracle import mvpa_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _cfg(**kw):
+    base = dict(max_position_embeddings=32, hidden_size=128, num_attention_heads=4, n_head_kv=2,
+                n_inner=256, global_att=True, scale_attn_weights=True,
+                scale_attn_by_inverse_layer_idx=False, reorder_and_upcast_attn=False,
+                lora=False, attn_pdrop=0.1, resid_pdrop=0.1)
+    base.update(kw)
+    return SimpleNamespace(**base)
+
+
+def _layer_io(T=14, C=6, E=128, B=2, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    h = torch.randn(B, T, C, E, generator=g)
+    pos = torch.randn(1, T, E, generator=g) * 0.5
+    chan = torch.randn(1, C, E, generator=g) * 0.5
+    return h, pos, chan
+
+
+def _oracle_layer(layer, h, pos, chan, heads, kv, **kw):
+    w = {k: v.detach().float().cpu() for k, v in layer.state_dict().items()}
+    return O.attention_layer_forward(h, pos, chan, w, heads, kv, **kw)
+
+
+def test_layer_fp32_matches_oracle():
+    """MVPFormerGQAAttention in fp32 (generic kernel + BLAS projections), with the additive
+    attention_mask the model builds from a 0/1 mask."""
+    torch.manual_seed(0)
+    layer = MVPFormerGQAAttention(_cfg(), layer_idx=0).eval()
+    for p in layer.parameters():
+        p.data.mul_(4.0)            # lift the logits off zero so masks and biases matter
+    h, pos, chan = _layer_io()
+    B, T, C, _ = h.shape
+    keep = (torch.rand(B, T * C, generator=torch.Generator().manual_seed(1)) > 0.2).float()
+    am = ((1.0 - keep) * torch.finfo(torch.float32).min)[:, None, None, :]
+    ref = _oracle_layer(layer, h, pos, chan, 4, 2, attention_mask=am)
+    lg = layer.cuda()
+    out, present = lg(h.cuda(), pos.cuda(), chan.cuda(), attention_mask=am.cuda())
+    assert present is None
+    assert (out.cpu() - ref).abs().max().item() <= 2e-4
+    out2 = lg(h.cuda(), pos.cuda(), chan.cuda(), attention_mask=am.cuda(), use_cache=True)
+    assert out2[1][0].shape == (B, 2, T, C, 32)
+    with pytest.raises(NotImplementedError):
+        lg(h.cuda(), pos.cuda(), chan.cuda(), output_attentions=True)
+
+
+def test_flash_layer_bf16_matches_oracle_and_ignores_mask():
+    torch.manual_seed(1)
+    layer = MVPFormerGQAFlashAttention(_cfg(lora=True, lora_rank=8, lora_alpha=16, lora_dropout=0,
+                                            lora_merge=True), layer_idx=0).eval()
+    for p in layer.parameters():
+        p.data.mul_(3.0)
+    layer.c_attn.lora_B.data.normal_(0, 0.05)          # make the adapter path matter
+    layer = layer.to(torch.bfloat16)
+    h, pos, chan = _layer_io(T=20, C=40, seed=3)
+    hb, pb, cb = h.bfloat16(), pos.bfloat16(), chan.bfloat16()
+    w = {k: v.detach().float() for k, v in layer.state_dict().items()}
+    w["q_attn.weight"] = layer.q_attn.effective_weight().detach().float()
+    w["c_attn.weight"] = layer.c_attn.effective_weight().detach().float()
+    ref = O.attention_layer_forward(hb.float(), pb.float(), cb.float(), w, 4, 2)
+    lg = layer.cuda()
+    out = lg(hb.cuda(), pb.cuda(), cb.cuda(), attention_mask=torch.full((2, 1, 1, 800), -1e30).cuda())
+    assert len(out) == 2 and out[1] is None
+    o = out[0].float().cpu()
+    rel = ((o - ref).norm() / ref.norm()).item()
+    assert rel <= 2e-2, rel
+    out3 = lg(hb.cuda(), pb.cuda(), cb.cuda(), output_attentions=True)
+    assert len(out3) == 3 and out3[2] is None
+
+
+def test_mvpformer_forward_matches_oracle():
+    """Encoder -> two parallel blocks -> final norm -> head, bf16 on the GPU against the fp32
+    oracle stack on the same (bf16-rounded) parameters."""
+    from models.fftencoder import WaveEncoder
+    from models.mvpformer import HMVPFormer, MVPFormerConfig, MVPFormerHead
+    torch.manual_seed(2)
+    cfg = MVPFormerConfig(n_positions=16, n_channels=16, n_embd=128, n_layer=2, n_head=4,
+                          n_head_kv=2, n_inner=256)
+    model = HMVPFormer(cfg, WaveEncoder(512, 128), MVPFormerHead(128, 128)).to(torch.bfloat16).eval()
+    for name, p in model.named_parameters():
+        if "attn" in name or "embedding" in name:
+            p.data.mul_(3.0)
+    sd = model.state_dict()
+    assert "mvpformer.h.1.attn.c_attn.weight" in sd and "mvpformer.h.0.ln_2.weight" in sd
+    assert "mvpformer.h.0.mlp.gate_proj.weight" in sd and "encoder.proj.weight" in sd
+    assert "head.head.weight" in sd and "seizure_embeddings" in sd and sd["encoder.proj.weight"].shape == (128, 550)
+    x = make_ieeg(2, 8, 6, 512, seed=5)
+    params = {k: v.float() for k, v in sd.items()}
+    ref, ref_emb = O.mvpformer_forward(x, params, dict(n_layer=2, n_head=4, n_head_kv=2))
+    out, emb = model.cuda()._common_forward(x.cuda())
+    rel_e = ((emb.float().cpu() - ref_emb).norm() / ref_emb.norm()).item()
+    rel_o = ((out.float().cpu() - ref).norm() / ref.norm()).item()
+    assert rel_e <= 1e-2, rel_e
+    assert rel_o <= 3e-2, rel_o
+    score = model.predict_next_segment(x.cuda())
+    assert score.shape == (2, 5, 8) and torch.isfinite(score).all()
