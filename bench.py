@@ -26,6 +26,10 @@ for _p in (PKG, ROOT):
 
 BF16_DENSE_PEAK_TFLOPS = 2500.0       # MI355X published dense bf16 MFMA peak
 
+# HBM bytes per launch of the attention kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by
+# what the same counters read for a plain 256 MiB copy (profiles/mvpa_mfma_kernel_c2.md).
+MEASURED_TRAFFIC_BYTES = {"c2": 345.1e6}
+
 WORKLOADS = {
     "c2": dict(B=4, C=64, T=128, H=16, Hkv=16, Dh=64, validity=False),
     "c3": dict(B=8, C=117, T=256, H=16, Hkv=16, Dh=64, validity=True),
@@ -92,6 +96,8 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-model", action="store_true", help="skip the MVPFormer-S forward leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain 256 MiB device copy (calibrates HBM traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures ONE GPU (the MVPA forward shards over batch and "
@@ -115,6 +121,12 @@ def main():
         mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
                               chan_valid=d.chan_valid, out=out, kernel=mvpa_hip.KERNEL_MFMA)
 
+    if args.copy_probe:
+        src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -144,7 +156,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 2),
                      "peak": BF16_DENSE_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(kern_tflops / BF16_DENSE_PEAK_TFLOPS, 4),
-                     "traffic": None, "kernel": "mvpa_mfma_kernel",
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "kernel": "mvpa_mfma_kernel",
                      "kernel_ms": round(kern_ms, 4)},
     }
     if not args.no_model:
