@@ -65,6 +65,10 @@ def test_fp32_config1_parity():
     ref, ref_lse = _oracle(inp, return_lse=True)
     assert (out.cpu().double() - ref).abs().max().item() <= F32_MAX_ABS
     assert (lse.cpu().double() - ref_lse).abs().max().item() <= 1e-4
+    import os
+    import numpy as np
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "c1_seed0.npz"))
+    assert np.abs(out.cpu().numpy() - g["out"]).max() <= F32_MAX_ABS
 
 
 @pytest.mark.parametrize("cfg", [

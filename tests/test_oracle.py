@@ -188,3 +188,15 @@ def test_db4_filter_bank_properties():
     assert torch.allclose(a[:, n2:], a[:, : a.shape[1] - n2]) and torch.allclose(d[:, n2:], d[:, : d.shape[1] - n2])
     energy = (a[:, :n2] ** 2).sum(-1) + (d[:, :n2] ** 2).sum(-1)
     assert torch.allclose(energy, (x ** 2).sum(-1))
+
+
+def test_golden_c1_fixture():
+    """Oracle and input generator against the committed vector (tests/golden/c1_seed0.npz)."""
+    import os
+    import numpy as np
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "c1_seed0.npz"))
+    inp = make_mvpa_inputs(B=2, C=8, T=32, H=4, Dh=32, seed=0)
+    assert np.array_equal(inp.q[0, 0, :4].numpy(), g["q_probe"])
+    assert np.array_equal(inp.k_time[0, :2].numpy(), g["k_time_probe"])
+    out, _ = _rel_attn(inp)
+    assert np.abs(out.numpy() - g["out"]).max() <= 5e-6
