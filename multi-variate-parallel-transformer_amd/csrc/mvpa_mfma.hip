@@ -30,7 +30,8 @@
 // reads; V^T fragments come from the transposing LDS read (ds_read_b64_tr_b16), which turns four
 // keys x 16 dh of row-major V into "4 keys per lane, one dh per lane".
 // One workgroup = NW waves = NW query blocks = NW/NCT consecutive time steps; one barrier per
-// key tile.
+// key tile.  Where registers allow, two 4-wave workgroups share a CU so that one computes while
+// the other sits at its barrier.
 #include "mvpa_common.h"
 
 namespace mvpa {
@@ -151,8 +152,8 @@ struct Cfg {
   static_assert(WLOADS % NW == 0 || WLOADS < NW, "every loading wave issues the same number of loads");
 };
 
-template <int DH, int NCT, int NW, int STAGES>
-__global__ __launch_bounds__(NW * 64) void mvpa_mfma_kernel(mvpa_fwd_args a) {
+template <int DH, int NCT, int NW, int STAGES, int MINB>
+__global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args a) {
   using G = Cfg<DH, NCT, NW, STAGES>;
   constexpr int CP = G::CP, KS = G::KS, MT = G::MT, ROWB = G::ROWB, CHUNKS = G::CHUNKS;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
@@ -602,11 +603,11 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma_kernel(mvpa_fwd_args a) {
   }
 }
 
-template <int DH, int NCT, int NW, int STAGES>
+template <int DH, int NCT, int NW, int STAGES, int MINB = 1>
 static int launch_cfg(const mvpa_fwd_args* a, hipStream_t stream) {
   using G = Cfg<DH, NCT, NW, STAGES>;
   static_assert(G::LDS_BYTES <= 160 * 1024, "LDS budget");
-  auto kern = mvpa_mfma_kernel<DH, NCT, NW, STAGES>;
+  auto kern = mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)G::LDS_BYTES);
   const int nt = (a->T + G::TQW - 1) / G::TQW;
@@ -647,7 +648,7 @@ int mvpa_launch_mfma(const mvpa_fwd_args* a, hipStream_t stream) {
       return launch_cfg<32, 4, 4, 4>(a, stream);
     case 64:
       if (nct == 1) return launch_cfg<64, 1, 8, 4>(a, stream);
-      if (nct == 2) return launch_cfg<64, 2, 8, 4>(a, stream);
+      if (nct == 2) return launch_cfg<64, 2, 4, 3, 2>(a, stream);   // two workgroups per CU
       return launch_cfg<64, 4, 4, 3>(a, stream);
     case 128:
       if (nct == 1) return launch_cfg<128, 1, 4, 4>(a, stream);
