@@ -8,7 +8,9 @@ from oracle import mvpa_oracle as O
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 200, 72), (1000, 768, 550), (64, 2304, 768), (17, 33, 8)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 200, 72), (1000, 768, 550), (64, 2304, 768), (17, 33, 8),
+                                   (2048, 768, 768), (1024, 1280, 768), (600, 130, 72), (4100, 2048, 552),
+                                   (16384, 768, 1728)])
 def test_linear_bf16(M, N, K):
     g = torch.Generator().manual_seed(M + N + K)
     ldk = (K + 7) // 8 * 8
@@ -24,9 +26,9 @@ def test_linear_bf16(M, N, K):
     assert (y.double() - ref).abs().max().item() <= 2 ** -8 * ref.abs().max().item() + 1e-6
 
 
-def test_linear_gated():
+@pytest.mark.parametrize("M,N,K", [(200, 96, 64), (1024, 1728, 768), (700, 200, 136), (4096, 64, 768)])
+def test_linear_gated(M, N, K):
     g = torch.Generator().manual_seed(3)
-    M, N, K = 200, 96, 64
     x = torch.randn(M, K, generator=g).bfloat16()
     w = (torch.randn(2 * N, K, generator=g) * 0.2).bfloat16()
     y = mvpa_hip.linear(x.cuda(), w.cuda(), gated=True).float().cpu()
