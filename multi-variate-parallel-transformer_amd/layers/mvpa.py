@@ -122,6 +122,8 @@ class MVPFormerGQAAttention(torch.nn.Module):
         self.resid_dropout = torch.nn.Dropout(config.resid_pdrop)
         self._fused_w = None
         self._fused_key = None
+        self._tables = None
+        self._tables_key = None
 
     def adapter_params(self):
         return ["q_attn.lora_A", "q_attn.lora_B", "c_attn.lora_A", "c_attn.lora_B"]
@@ -138,6 +140,49 @@ class MVPFormerGQAAttention(torch.nn.Module):
             self._fused_w = torch.cat([_weight_of(self.q_attn), _weight_of(self.c_attn)], 0).to(dtype).contiguous()
             self._fused_key = key
         return self._fused_w
+
+    def _key_tables(self, positional_embedding, channel_embedding):
+        """position_net(positional_embedding) -> [Hkv,T,Dh] and channel_net(channel_embedding) ->
+        [Hkv,C,Dh] (layers/mvpa.py:307-313).  Both depend only on parameters and on the embedding
+        rows, so they are computed once and reused until one of those tensors changes."""
+        hkv, dh = self.num_kv_heads, self.head_dim
+        t_len, c_len = positional_embedding.shape[-2], channel_embedding.shape[-2]
+
+        def compute():
+            k_time = _linear(positional_embedding, self.position_net.weight)
+            k_chan = _linear(channel_embedding, self.channel_net.weight)
+            return (k_time.view(t_len, hkv, dh).permute(1, 0, 2).contiguous(),
+                    k_chan.view(c_len, hkv, dh).permute(1, 0, 2).contiguous())
+
+        # only views of parameters can be recognised safely from one call to the next (their
+        # version counter follows every in-place update); anything else is recomputed
+        def ident(t):
+            base = t._base if t._base is not None else t
+            if not isinstance(base, torch.nn.Parameter):
+                return None
+            return (base.data_ptr(), base._version, t.storage_offset(), tuple(t.shape), tuple(t.stride()), t.dtype)
+
+        ids = tuple(ident(t) for t in (positional_embedding, channel_embedding,
+                                       self.position_net.weight, self.channel_net.weight))
+        if any(i is None for i in ids):
+            return compute()
+        if self._tables_key != ids:
+            self._tables, self._tables_key = compute(), ids
+        return self._tables
+
+    @staticmethod
+    def _as_channel_validity(attention_mask, bsz, t_len, c_len):
+        """An additive key mask built from a 0/1 mask (models/mvpformer.py:262-268: zeros and
+        finfo.min) that is the same at every time step is a per-channel validity mask, which the
+        bf16 MFMA kernel applies exactly.  Returns [B,C] bool, or None if the mask is anything else
+        (then it is passed on as an additive key bias)."""
+        m = attention_mask.reshape(bsz, t_len, c_len)
+        first = m[:, 0]
+        binary = ((first == 0) | (first <= -1e30)).all()
+        same = (m == first[:, None]).all()
+        if bool(binary & same):          # one device sync per call, only when a mask is given
+            return first == 0
+        return None
 
     def _scale(self) -> float:
         s = 1.0
@@ -166,14 +211,13 @@ class MVPFormerGQAAttention(torch.nn.Module):
             q = qkv[:, :, :e].view(bsz, n, h, dh).permute(0, 2, 1, 3)        # views, no copy
             k = qkv[:, :, e:e + kv].view(bsz, n, hkv, dh).permute(0, 2, 1, 3)
             v = qkv[:, :, e + kv:].view(bsz, n, hkv, dh).permute(0, 2, 1, 3)
-            k_time = _linear(positional_embedding, self.position_net.weight)  # [1,T,kvE]
-            k_chan = _linear(channel_embedding, self.channel_net.weight)      # [1,C,kvE]
-            k_time = k_time.view(t_len, hkv, dh).permute(1, 0, 2).contiguous()
-            k_chan = k_chan.view(c_len, hkv, dh).permute(1, 0, 2).contiguous()
+            k_time, k_chan = self._key_tables(positional_embedding, channel_embedding)
             u, vb, z = (b.view(hkv, dh) for b in self.attn_bias.split(kv, dim=0))
             chan_valid, key_bias = None, None
             if attention_mask is not None:
-                key_bias = attention_mask.reshape(bsz, n).to(torch.float32)
+                chan_valid = self._as_channel_validity(attention_mask, bsz, t_len, c_len)
+                if chan_valid is None:
+                    key_bias = attention_mask.reshape(bsz, n).to(torch.float32)
             merged = torch.empty((bsz, n, h, dh), dtype=dt, device=hidden_states.device)
             mvpa_hip.mvpa_forward(
                 q, k, v, u, vb, z, k_time, k_chan, sm_scale=self._scale(), window=window,

@@ -163,15 +163,16 @@ class MVPFormerModel(nn.Module):
         if self.training:
             raise NotImplementedError("MVPFormer HIP stack: inference only; call .eval()")
         bsz, t_len, c_len, _ = inputs_embeds.shape
-        device = inputs_embeds.device
-        position_ids = torch.arange(t_len, dtype=torch.long, device=device).unsqueeze(0)
-        channel_ids = torch.arange(c_len, dtype=torch.long, device=device).unsqueeze(0)
         if attention_mask is not None:                           # models/mvpformer.py:262-268
             dt = inputs_embeds.dtype
             attention_mask = attention_mask.view(bsz, -1)[:, None, None, :].to(dtype=dt)
             attention_mask = (1.0 - attention_mask) * torch.finfo(dt).min
-        position_embeds = self.positional_embedding(position_ids)
-        channel_embeds = self.channel_embedding(channel_ids)
+        # ids are arange(T) / arange(C) (models/mvpformer.py:246-261), so the lookups
+        # (models/mvpformer.py:282-283) are leading slices of the embedding tables
+        if t_len > self.positional_embedding.num_embeddings or c_len > self.channel_embedding.num_embeddings:
+            raise IndexError("more time steps / channels than embedding rows (n_positions / n_channels)")
+        position_embeds = self.positional_embedding.weight[:t_len][None]
+        channel_embeds = self.channel_embedding.weight[:c_len][None]
         hidden_states = inputs_embeds
         for block in self.h:
             hidden_states = block(hidden_states, position_embeds, channel_embeds,

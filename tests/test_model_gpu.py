@@ -53,6 +53,14 @@ def test_layer_fp32_matches_oracle():
     assert out2[1][0].shape == (B, 2, T, C, 32)
     with pytest.raises(NotImplementedError):
         lg(h.cuda(), pos.cuda(), chan.cuda(), output_attentions=True)
+    # a mask that is constant over time is recognised as channel validity (same result)
+    keep_c = torch.tensor([[1, 1, 0, 1, 1, 0], [0, 1, 1, 1, 1, 1]], dtype=torch.float32)
+    am2 = ((1.0 - keep_c[:, None, :].expand(B, T, C).reshape(B, T * C)) * torch.finfo(torch.float32).min)[:, None, None, :]
+    assert lg._as_channel_validity(am2.cuda(), B, T, C) is not None
+    assert lg._as_channel_validity(am.cuda(), B, T, C) is None
+    ref2 = _oracle_layer(layer.cpu(), h, pos, chan, 4, 2, attention_mask=am2)
+    out3 = layer.cuda()(h.cuda(), pos.cuda(), chan.cuda(), attention_mask=am2.cuda())[0]
+    assert (out3.cpu() - ref2).abs().max().item() <= 2e-4
 
 
 def test_flash_layer_bf16_matches_oracle_and_ignores_mask():
