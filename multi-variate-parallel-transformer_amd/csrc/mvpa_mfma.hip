@@ -106,6 +106,40 @@ __device__ inline bf16x8 make_qfrag(u32x4 raw, const bf16_t* __restrict__ bias, 
   return out;
 }
 
+// 8 floats -> 8 fp8 (e4m3) packed in 64 bits, the operand of the 32x32x16 fp8 MFMA
+__device__ inline long pack_fp8(const float (&f)[8]) {
+  int lo = 0, hi = 0;
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], hi, false);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
+  return (long)(((unsigned long)(unsigned)hi << 32) | (unsigned)lo);
+}
+
+// (q + bias) * scale as an fp8 fragment
+__device__ inline long make_qfrag_fp8(u32x4 raw, const bf16_t* __restrict__ bias, float scale) {
+  const u32x4 braw = *(const u32x4*)bias;
+  float f[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t w = raw[i], bw = braw[i];
+    f[2 * i] = (__uint_as_float(w << 16) + __uint_as_float(bw << 16)) * scale;
+    f[2 * i + 1] = (__uint_as_float(w & 0xffff0000u) + __uint_as_float(bw & 0xffff0000u)) * scale;
+  }
+  return pack_fp8(f);
+}
+
+// a bf16 K fragment, scaled, as an fp8 fragment
+__device__ inline long kfrag_fp8(u32x4 raw, float scale) {
+  float f[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = __uint_as_float(raw[i] << 16) * scale;
+    f[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u) * scale;
+  }
+  return pack_fp8(f);
+}
+
 __device__ inline bf16x8 as_bf16x8(u32x4 v) {
   union { u32x4 u; bf16x8 b; } c;
   c.u = v;
@@ -152,7 +186,7 @@ struct Cfg {
   static_assert(WLOADS % NW == 0 || WLOADS < NW, "every loading wave issues the same number of loads");
 };
 
-template <int DH, int NCT, int NW, int STAGES, int MINB>
+template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8>
 __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args a) {
   using G = Cfg<DH, NCT, NW, STAGES>;
   constexpr int CP = G::CP, KS = G::KS, MT = G::MT, ROWB = G::ROWB, CHUNKS = G::CHUNKS;
@@ -213,6 +247,16 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 
   // =========================== setup: Qu, Qv, channel bias tile, Ec ===========================
   bf16x8 Qu[KS], Qv[KS];     // (q+u), (q+v) * scale as QK^T / time-slab B operands
+  // fp8 content term: q' = (q+u)*scale/sq and k' = k/sk are rounded to e4m3 with the per-head
+  // amax scales sq, sk chosen by the caller; the MFMA accumulates in units of 1/(sq*sk), the
+  // channel-bias tile is pre-divided accordingly and the product sq*sk returns inside the exp2 fma
+  long Qu8[KS];
+  float fp8_d = 1.f, fp8_inv_sk = 1.f;
+  if (FP8) {
+    const float sq = a.fp8_q_scale[h], sk = a.fp8_k_scale[g];
+    fp8_d = sq * sk;
+    fp8_inv_sk = 1.f / sk;
+  }
   f32x16 Bc[NCT];            // channel-bias tile, [ck][q] in accumulator layout; -inf = masked key
   {
     u32x4 raw[KS];
@@ -227,6 +271,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     for (int ks = 0; ks < KS; ++ks) {
       const int d0 = ks * 16 + hh * 8;
       Qu[ks] = make_qfrag(raw[ks], bu + d0, sc2);
+      if (FP8) Qu8[ks] = make_qfrag_fp8(raw[ks], bu + d0, sc2 / a.fp8_q_scale[h]);
       Qv[ks] = make_qfrag(raw[ks], bv + d0, sc2);
       const bf16x8 qz = make_qfrag(raw[ks], bz + d0, sc2);
 #pragma unroll
@@ -288,6 +333,13 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
       Ec[t][1] = pack8(e, 8);
     }
     sumEc = se;               // partial: this half-wave's keys only
+  }
+  if (FP8) {
+    const float inv_d = 1.f / fp8_d;
+#pragma unroll
+    for (int t = 0; t < NCT; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) Bc[t][i] *= inv_d;
   }
 
   // running soft-max state of this lane's query; l is a per-half-wave partial sum
@@ -439,8 +491,13 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
       for (int t = 0; t < NCT; ++t) {
-        const bf16x8 ka = *(const bf16x8*)(stage + k_lane[ks] + t * 32 * ROWB);
-        S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, Qu[ks], S[t], 0, 0, 0);
+        if (FP8) {
+          const u32x4 kr = *(const u32x4*)(stage + k_lane[ks] + t * 32 * ROWB);
+          S[t] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(kfrag_fp8(kr, fp8_inv_sk), Qu8[ks], S[t], 0, 0, 0);
+        } else {
+          const bf16x8 ka = *(const bf16x8*)(stage + k_lane[ks] + t * 32 * ROWB);
+          S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, Qu[ks], S[t], 0, 0, 0);
+        }
       }
     float rmax = -INFINITY;
 #pragma unroll
@@ -448,6 +505,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 #pragma unroll
       for (int i = 0; i < 16; ++i) rmax = fmaxf(rmax, S[t][i]);
     rmax = xhalf_max(rmax);
+    if (FP8) rmax *= fp8_d;
     // Lazy running max: the reference point only moves when some query's row max outgrew it by
     // more than 2^8; until then probabilities are formed against the old reference (at most 256
     // times larger, harmless in fp32/bf16) and the accumulator rescale is skipped altogether.
@@ -461,7 +519,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     for (int t = 0; t < NCT; ++t) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const float p = fast_exp2(S[t][i] + off);
+        const float p = FP8 ? fast_exp2(__builtin_fmaf(S[t][i], fp8_d, off)) : fast_exp2(S[t][i] + off);
         S[t][i] = p;
         ls += p;
       }
@@ -603,11 +661,11 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   }
 }
 
-template <int DH, int NCT, int NW, int STAGES, int MINB = 1>
-static int launch_cfg(const mvpa_fwd_args* a, hipStream_t stream) {
+template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8>
+static int launch_one(const mvpa_fwd_args* a, hipStream_t stream) {
   using G = Cfg<DH, NCT, NW, STAGES>;
   static_assert(G::LDS_BYTES <= 160 * 1024, "LDS budget");
-  auto kern = mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB>;
+  auto kern = mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)G::LDS_BYTES);
   const int nt = (a->T + G::TQW - 1) / G::TQW;
@@ -616,12 +674,17 @@ static int launch_cfg(const mvpa_fwd_args* a, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 
+template <int DH, int NCT, int NW, int STAGES, int MINB = 1>
+static int launch_cfg(const mvpa_fwd_args* a, hipStream_t stream) {
+  if (a->flags & MVPA_FLAG_FP8_QK) return launch_one<DH, NCT, NW, STAGES, MINB, true>(a, stream);
+  return launch_one<DH, NCT, NW, STAGES, MINB, false>(a, stream);
+}
+
 }  // namespace mvpa
 
 int mvpa_mfma_supported(const mvpa_fwd_args* a) {
   if (a->dtype != MVPA_BF16) return 0;
   if (!(a->flags & MVPA_FLAG_CAUSAL)) return 0;
-  if (a->flags & MVPA_FLAG_FP8_QK) return 0;
   if (a->key_bias) return 0;
   if (a->C > 128) return 0;
   if (a->Dh != 32 && a->Dh != 64 && a->Dh != 128) return 0;

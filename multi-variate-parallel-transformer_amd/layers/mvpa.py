@@ -105,6 +105,8 @@ class MVPFormerGQAAttention(torch.nn.Module):
         self.scale_attn_by_inverse_layer_idx = config.scale_attn_by_inverse_layer_idx
         self.layer_idx = layer_idx
         self.reorder_and_upcast_attn = config.reorder_and_upcast_attn
+        # extension: content-term QK^T in fp8 e4m3 with per-head amax scales (bf16 GPU path only)
+        self.fp8_qk = bool(getattr(config, "fp8_qk", False))
         e, kv = self.embed_dim, self.embed_kv_dim
         if getattr(config, "lora", False):
             self.q_attn = _LoRALinear(e, e, config.lora_rank, config.lora_alpha, enable=(True,))
@@ -222,7 +224,8 @@ class MVPFormerGQAAttention(torch.nn.Module):
             mvpa_hip.mvpa_forward(
                 q, k, v, u, vb, z, k_time, k_chan, sm_scale=self._scale(), window=window,
                 causal=True, content=bool(self.global_att), chan_valid=chan_valid,
-                key_bias=key_bias, out=merged.permute(0, 2, 1, 3))
+                key_bias=key_bias, out=merged.permute(0, 2, 1, 3),
+                fp8_qk=self.fp8_qk and dt == torch.bfloat16 and key_bias is None)
             if head_mask is not None:                       # layers/mvpa.py:274-275
                 if head_mask.numel() != h:
                     raise NotImplementedError("head_mask must hold one factor per head")

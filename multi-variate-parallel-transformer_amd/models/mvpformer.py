@@ -34,7 +34,8 @@ class MVPFormerConfig:
                  resid_pdrop=0.1, embd_pdrop=0.1, attn_pdrop=0.1, layer_norm_epsilon=0.00001,
                  initializer_range=0.02, scale_attn_weights=True, use_cache=False,
                  scale_attn_by_inverse_layer_idx=False, reorder_and_upcast_attn=False,
-                 lora=False, lora_alpha=16, lora_rank=8, lora_dropout=0, lora_merge=True):
+                 lora=False, lora_alpha=16, lora_rank=8, lora_dropout=0, lora_merge=True,
+                 fp8_qk=False):
         self.n_positions, self.n_channels, self.n_embd = n_positions, n_channels, n_embd
         self.n_layer, self.n_head, self.n_inner, self.n_head_kv = n_layer, n_head, n_inner, n_head_kv
         self.global_att = global_att
@@ -50,6 +51,7 @@ class MVPFormerConfig:
         self.mlp_bias = False
         self.lora, self.lora_alpha, self.lora_rank = lora, lora_alpha, lora_rank
         self.lora_dropout, self.lora_merge = lora_dropout, lora_merge
+        self.fp8_qk = fp8_qk            # extension: fp8 e4m3 QK^T of the content term
         self.add_cross_attention = False
         self.output_attentions = False
         self.output_hidden_states = False

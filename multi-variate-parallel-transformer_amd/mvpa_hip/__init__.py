@@ -191,13 +191,15 @@ def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float]
     flags = ((FLAG_CAUSAL if causal else 0) | (FLAG_CONTENT if content else 0) |
              (FLAG_TIME_BIAS if time_bias else 0) | (FLAG_CHAN_BIAS if chan_bias else 0) |
              (FLAG_FP8_QK if fp8_qk else 0))
+    s = (1.0 / Dh ** 0.5) if sm_scale is None else float(sm_scale)
     q_scale = k_scale = None
     if fp8_qk:
-        # per-head amax scales mapping each head's range onto e4m3's +-448
-        qf = (q.float() + u.float().repeat_interleave(H // k.shape[1], 0)[None, :, None, :])
-        q_scale = (qf.abs().amax(dim=(0, 2, 3)) / 448.0).clamp_min(1e-12).contiguous()
-        k_scale = (k.float().abs().amax(dim=(0, 2, 3)) / 448.0).clamp_min(1e-12).contiguous()
-    s = (1.0 / Dh ** 0.5) if sm_scale is None else float(sm_scale)
+        # per-head amax scales: the kernel rounds (q+u)*s*log2(e)/q_scale and k/k_scale to e4m3;
+        # 224 keeps the largest magnitude inside the range of either e4m3 flavour
+        grp = H // k.shape[1]
+        qf = q.float() + u.float().repeat_interleave(grp, 0)[None, :, None, :]
+        q_scale = (qf.abs().amax(dim=(0, 2, 3)) * (s * 1.4426950408889634 / 224.0)).clamp_min(1e-20).contiguous()
+        k_scale = (k.float().abs().amax(dim=(0, 2, 3)) / 224.0).clamp_min(1e-20).contiguous()
     a = make_args(q, k, v, out, u, vb, z, k_time, k_chan, T=T, C=C, sm_scale=s, window=window,
                   flags=flags, chan_valid=chan_valid, key_bias=key_bias, lse=lse, kernel=kernel,
                   fp8_q_scale=q_scale, fp8_k_scale=k_scale)

@@ -113,3 +113,33 @@ def test_mvpformer_forward_matches_oracle():
     assert rel_o <= 3e-2, rel_o
     score = model.predict_next_segment(x.cuda())
     assert score.shape == (2, 5, 8) and torch.isfinite(score).all()
+
+
+def test_base_classification_bf16_then_fp8():
+    """Base-size dims (E2048 H16 Hkv8 Dh128 n_inner5632, C=128) cut to two layers and 12 segments:
+    binary-head logits in bf16 and with fp8 QK^T against the fp32 oracle stack.  Tolerances are
+    this build's statement: logits within 3e-2 (bf16) and 6e-2 (fp8) of the fp32 reference in
+    units of the logit spread."""
+    from models.configs import MVPFORMER_BASE
+    from models.fftencoder import WaveEncoder
+    from models.mvpformer import HMVPFormer, MVPFormerConfig, MVPFormerHead
+    dims = dict(MVPFORMER_BASE, n_layer=2)
+    x = make_ieeg(1, 128, 12, 512, seed=7)
+    logits = {}
+    for fp8 in (False, True):
+        torch.manual_seed(3)
+        cfg = MVPFormerConfig(**dims, fp8_qk=fp8)
+        model = HMVPFormer(cfg, WaveEncoder(512, cfg.n_embd), MVPFormerHead(cfg.n_embd, 2)).to(torch.bfloat16).eval()
+        for name, p in model.named_parameters():
+            if "attn" in name or "embedding" in name:
+                p.data.mul_(2.0)
+        if not fp8:
+            params = {k: v.float() for k, v in model.state_dict().items()}
+            h, _ = O.mvpformer_forward(x, params, dict(n_layer=2, n_head=16, n_head_kv=8))
+            ref = torch.nn.functional.linear(h[:, -1].mean(dim=1), params["head.head.weight"])
+        logits[fp8] = model.cuda().classify(x.cuda()).float().cpu()
+    spread = ref.abs().max().item() + 1e-6
+    e16 = (logits[False] - ref).abs().max().item() / spread
+    e8 = (logits[True] - ref).abs().max().item() / spread
+    print(f"base-size logits: ref {ref.flatten().tolist()}, bf16 err {e16:.3e}, fp8 err {e8:.3e} (relative to spread)")
+    assert e16 <= 3e-2 and e8 <= 6e-2

@@ -314,3 +314,37 @@ def test_bf16_config3_irregular_channels():
     o2 = mvpa_hip.mvpa_forward(d.q, k2, v2, d.u, d.vb, d.z, d.k_time, d.k_chan,
                                chan_valid=d.chan_valid)
     assert torch.equal(o2, out)
+
+
+# fp8 (e4m3) content term: 3 mantissa bits on q' and k.  Rounding both factors to e4m3 perturbs a
+# content score by about 2.5 % of the score's own spread, so the stated tolerance scales with how
+# wide the content logits are: unit-variance logits (q, k ~ N(0,1), Dh = 64) versus the narrow
+# logits of the benchmark distribution (q, k ~ N(0,1)/sqrt(Dh)).
+FP8_TOL = {False: dict(max_abs=1.2e-1, rel_l2=6e-2), True: dict(max_abs=2e-2, rel_l2=6e-3)}
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(B=2, C=64, T=24, H=4, Dh=64, Hkv=2, qkv_unit=False, table_std=0.3),
+    dict(B=1, C=117, T=14, H=2, Dh=64, qkv_unit=True, table_std=0.3, validity=True),
+    dict(B=1, C=128, T=13, H=2, Dh=128, Hkv=1, qkv_unit=False, table_std=0.3),
+])
+def test_fp8_qk_within_stated_tolerance(cfg):
+    """QK^T of the content term in fp8 e4m3 with per-head amax scales (biases, soft-max and PV
+    unchanged).  The reference has no fp8 path; the tolerance against the fp64 oracle is this
+    build's own statement."""
+    inp = make_mvpa_inputs(seed=31, **cfg).round_to(torch.bfloat16)
+    ref = _oracle(inp).float()
+    o8 = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA, fp8_qk=True).float().cpu()
+    o16 = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA).float().cpu()
+    assert not torch.equal(o8, o16)                     # the fp8 path really ran
+    err, rel = (o8 - ref).abs().max().item(), _rel_l2(o8, ref)
+    tol = FP8_TOL[cfg["qkv_unit"]]
+    print(f"fp8 QK^T: max-abs {err:.3e} rel-L2 {rel:.3e} (bf16: {(o16 - ref).abs().max().item():.3e}, {_rel_l2(o16, ref):.3e})")
+    assert err <= tol["max_abs"] and rel <= tol["rel_l2"], f"max-abs {err:.3e}, rel-L2 {rel:.3e}"
+
+
+def test_fp8_needs_mfma_kernel():
+    inp = make_mvpa_inputs(B=1, C=4, T=6, H=1, Dh=32, seed=1)
+    d = inp.to("cuda", torch.float32)
+    with pytest.raises(mvpa_hip.MvpaError):
+        mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, fp8_qk=True)
