@@ -89,7 +89,12 @@ __device__ inline void wait_vmcnt(int n) {
   }
 }
 
-__device__ inline float xhalf_max(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
+// max over a lane and its partner in the other half-wave (lane ^ 32): one register swap between
+// the halves instead of a round trip through the LDS crossbar
+__device__ inline float xhalf_max(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
 
 // 8 bf16 (one 16-byte chunk of a q row) + bias, scaled, back to a bf16 MFMA fragment
 __device__ inline bf16x8 make_qfrag(u32x4 raw, const bf16_t* __restrict__ bias, float scale) {
@@ -206,21 +211,46 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 
   // ---- block -> (b*H + h, time tile).  Workgroups are dealt round-robin to the 8 XCDs, so
   // ids that are equal mod 8 share an L2: give them the same (b, h) so its K/V stay in that L2.
-  // Within a (b, h) the latest (= longest) time tiles are issued first.
+  // The LAST time tile of every (b, h) goes out first: its final row keeps the content term for
+  // every key step (no far steps at all), which makes it several times longer than any other
+  // workgroup, and it must not be what the rest of the grid ends up waiting for.  After those,
+  // within a (b, h) the latest (= longest) time tiles are issued first.
   const int nt = (T_ + G::TQW - 1) / G::TQW;
   const int nbh = a.B * a.H;
+  constexpr int PASSES = 1;
   int bh, tile;
   {
     const int L = blockIdx.x;
-    if ((nbh & 7) == 0) {
-      const int xcd = L & 7, s = L >> 3;
-      bh = xcd + 8 * (s / nt);
-      tile = s % nt;
+    if ((nbh & 7) == 0 && nt > 1) {
+      if (L < nbh) {
+        bh = L;                          // L & 7 is the XCD, the same one as below for this (b, h)
+        tile = nt - 1;
+      } else {
+        // The other nt-1 tiles go out in PASSES passes over the (b, h) of an XCD, heavy tiles in
+        // the first pass and light ones in the last, so that what is left to run at the very
+        // end of the grid is short.
+        const int L2 = L - nbh;
+        const int xcd = L2 & 7, per_xcd = nbh >> 3;
+        int s = L2 >> 3, hi = nt - 1;
+        bh = xcd;
+        tile = 0;
+#pragma unroll 1
+        for (int p = 0; p < PASSES; ++p) {
+          const int lo = ((nt - 1) * (PASSES - 1 - p)) / PASSES;
+          const int cnt = (hi - lo) * per_xcd;
+          if (s < cnt || p == PASSES - 1) {
+            bh = xcd + 8 * (s / (hi - lo));
+            tile = hi - 1 - s % (hi - lo);
+            break;
+          }
+          s -= cnt;
+          hi = lo;
+        }
+      }
     } else {
       bh = L / nt;
-      tile = L % nt;
+      tile = nt - 1 - L % nt;
     }
-    tile = nt - 1 - tile;
   }
   const int b = bh / a.H, h = bh % a.H;
   const int g = h / (a.H / a.Hkv);
@@ -487,18 +517,28 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     f32x16 S[NCT];
 #pragma unroll
     for (int t = 0; t < NCT; ++t) S[t] = Bc[t];
+    if (FP8) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
+      for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-      for (int t = 0; t < NCT; ++t) {
-        if (FP8) {
+        for (int t = 0; t < NCT; ++t) {
           const u32x4 kr = *(const u32x4*)(stage + k_lane[ks] + t * 32 * ROWB);
           S[t] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(kfrag_fp8(kr, fp8_inv_sk), Qu8[ks], S[t], 0, 0, 0);
-        } else {
-          const bf16x8 ka = *(const bf16x8*)(stage + k_lane[ks] + t * 32 * ROWB);
-          S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, Qu[ks], S[t], 0, 0, 0);
         }
-      }
+    } else {
+      // every K fragment of the tile is requested before the first MFMA waits for one
+      bf16x8 ka[KS][NCT];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int t = 0; t < NCT; ++t) ka[ks][t] = *(const bf16x8*)(stage + k_lane[ks] + t * 32 * ROWB);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int t = 0; t < NCT; ++t)
+          S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][t], Qu[ks], S[t], 0, 0, 0);
+    }
     float rmax = -INFINITY;
 #pragma unroll
     for (int t = 0; t < NCT; ++t)
