@@ -217,7 +217,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   // within a (b, h) the latest (= longest) time tiles are issued first.
   const int nt = (T_ + G::TQW - 1) / G::TQW;
   const int nbh = a.B * a.H;
-  constexpr int PASSES = 1;
+  constexpr int TAIL_MERGE = 2;
   int bh, tile;
   {
     const int L = blockIdx.x;
@@ -226,25 +226,20 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
         bh = L;                          // L & 7 is the XCD, the same one as below for this (b, h)
         tile = nt - 1;
       } else {
-        // The other nt-1 tiles go out in PASSES passes over the (b, h) of an XCD, heavy tiles in
-        // the first pass and light ones in the last, so that what is left to run at the very
-        // end of the grid is short.
+        // the other nt-1 tiles: one (b, h) of the XCD after the other, long tiles first; the
+        // last TAIL_MERGE (b, h) of the XCD are interleaved tile by tile so that the grid does
+        // not end on the long tiles of a single (b, h)
         const int L2 = L - nbh;
-        const int xcd = L2 & 7, per_xcd = nbh >> 3;
-        int s = L2 >> 3, hi = nt - 1;
-        bh = xcd;
-        tile = 0;
-#pragma unroll 1
-        for (int p = 0; p < PASSES; ++p) {
-          const int lo = ((nt - 1) * (PASSES - 1 - p)) / PASSES;
-          const int cnt = (hi - lo) * per_xcd;
-          if (s < cnt || p == PASSES - 1) {
-            bh = xcd + 8 * (s / (hi - lo));
-            tile = hi - 1 - s % (hi - lo);
-            break;
-          }
-          s -= cnt;
-          hi = lo;
+        const int xcd = L2 & 7, per_xcd = nbh >> 3, s = L2 >> 3;
+        const int merged = per_xcd < TAIL_MERGE ? per_xcd : TAIL_MERGE;
+        const int plain = (per_xcd - merged) * (nt - 1);
+        if (s < plain) {
+          bh = xcd + 8 * (s / (nt - 1));
+          tile = nt - 2 - s % (nt - 1);
+        } else {
+          const int r = s - plain;
+          bh = xcd + 8 * (per_xcd - merged + r % merged);
+          tile = nt - 2 - r / merged;
         }
       }
     } else {
