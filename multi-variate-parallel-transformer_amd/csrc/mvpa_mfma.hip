@@ -38,6 +38,7 @@ namespace mvpa {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
@@ -46,6 +47,8 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 #define GLOBAL_PTR(T) __attribute__((address_space(1))) T*
 
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+#define kOnes2 (bf16x2{(__bf16)1.0f, (__bf16)1.0f})
 
 // order LDS traffic between the lanes of ONE wave (no workgroup barrier needed)
 __device__ inline void wave_lds_sync() {
@@ -314,24 +317,37 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
         const int j = t * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
         scr[j * 32 + ln] = has_chan ? sct[t][i] : 0.f;
       }
-    // key-channel mask as two 64-bit words: bit ck set = channel exists and is present
-    uint64_t kmask[2];
+    // key-channel mask: bit ck set = channel exists and is present.  Each lane keeps the bits of
+    // its own 32 keys (8(i/4) + 4hh + i%4 within key tile t) shifted down by 4hh, so that the bit
+    // of element i sits at the compile-time position 8(i/4) + i%4.
+    uint32_t kbits[NCT];
+    {
+      uint64_t kmask[2];
 #pragma unroll
-    for (int w = 0; w < 2; ++w) {
-      const int ck = w * 64 + lane;
-      bool ok = ck < C_;
-      if (valid) ok = ok && valid[min(ck, C_ - 1)] != 0;
-      kmask[w] = __ballot(ok);
+      for (int w = 0; w < 2; ++w) {
+        const int ck = w * 64 + lane;
+        bool ok = ck < C_;
+        if (valid) ok = ok && valid[min(ck, C_ - 1)] != 0;
+        kmask[w] = __ballot(ok);
+      }
+#pragma unroll
+      for (int t = 0; t < NCT; ++t) kbits[t] = (uint32_t)(kmask[t >> 1] >> ((t & 1) * 32 + 4 * hh));
     }
     wave_lds_sync();
+    // Bc[ck][q] = scr[C-1-|cq-ck|][q].  With ck = c_i + 4hh (c_i a compile-time constant) the
+    // distance is |(cq - 4hh + 4) - (c_i + 4)| on unsigned operands; distances past C-1 only occur
+    // for padded queries or keys, whose values are never used, and are clamped into the scratch.
+    const uint32_t cq4 = (uint32_t)(cq - 4 * hh + 4);
+    const int gbase = ((C_ - 1) * 32 + ln) * 4;
+    const unsigned char* scr_b = (const unsigned char*)scr;
 #pragma unroll
     for (int t = 0; t < NCT; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int ck = t * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
-        const bool kv = (kmask[t >> 1] >> (ck & 63)) & 1;
-        const int j = max(chan_row(cq, ck, C_), 0);   // padded rows/keys: any in-range row will do
-        const float val = scr[j * 32 + ln];
+        const uint32_t ci4 = (uint32_t)(t * 32 + (i >> 2) * 8 + (i & 3) + 4);
+        const uint32_t dist = min(max(cq4, ci4) - min(cq4, ci4), (uint32_t)(C_ - 1));
+        const float val = *(const float*)(scr_b + (gbase - (int)(dist * 128u)));
+        const bool kv = (kbits[t] >> ((i >> 2) * 8 + (i & 3))) & 1u;
         Bc[t][i] = kv ? val : -INFINITY;
       }
   }
@@ -553,13 +569,19 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 #pragma unroll
     for (int t = 0; t < NCT; ++t) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float p = FP8 ? fast_exp2(__builtin_fmaf(S[t][i], fp8_d, off)) : fast_exp2(S[t][i] + off);
-        S[t][i] = p;
-        ls += p;
-      }
+      for (int i = 0; i < 16; ++i)
+        S[t][i] = FP8 ? fast_exp2(__builtin_fmaf(S[t][i], fp8_d, off)) : fast_exp2(S[t][i] + off);
       P[t][0] = pack8(S[t], 0);
       P[t][1] = pack8(S[t], 8);
+      // the row sum is taken over the bf16 probabilities the PV product uses, two per
+      // instruction (v_dot2c_f32_bf16 against a pair of ones), accumulated in fp32
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        union { bf16x8 v; bf16x2 q[4]; } u;
+        u.v = P[t][s];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ls = __builtin_amdgcn_fdot2_f32_bf16(u.q[j], kOnes2, ls, false);
+      }
     }
     if (grow) {
       const float alpha = fast_exp2(m_run - m_new);
