@@ -158,6 +158,15 @@ int mvpa_rmsnorm(const void* x, const float* weight, void* y, int64_t rows, int3
 int mvpa_add3_bf16(const void* a, const void* b, const void* c, void* out, int64_t n,
                    void* stream);
 
+/* sum = a + b + c (bf16, one rounding) and norm = RMSNorm(sum) * weight in one pass: the residual
+ * update of a block (models/mvpformer.py:147) fused with the input norm of the next block
+ * (models/mvpformer.py:133) or with ln_f (models/mvpformer.py:380).  Rows are contiguous
+ * ([rows, cols]); cols % 8 == 0 and 16-byte aligned pointers, else MVPA_ERR_ALIGN.  The norm is
+ * taken over the rounded sum: identical to mvpa_add3_bf16 followed by mvpa_rmsnorm. */
+int mvpa_add3_rmsnorm_bf16(const void* a, const void* b, const void* c, const float* weight,
+                           void* sum, void* norm, int64_t rows, int32_t cols, float eps,
+                           void* stream);
+
 /* Multilevel db4 analysis with periodic extension of fp32 rows x[M,L] into
  * coeffs[M,dwt_size] (row pitch ldc >= dwt_size) ordered [cA_L, cD_L, ..., cD_1]
  * (models/fftencoder.py:80-88). */

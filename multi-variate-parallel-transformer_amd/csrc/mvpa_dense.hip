@@ -379,6 +379,123 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const TI* __restrict__ x,
     io<TO>::store(yr + c, io<TI>::load(xr + c) * inv * w[c]);
 }
 
+// ---- 8 elements per lane and access (16 bytes of bf16, 32 bytes of fp32) --------------------
+template <typename T> struct vec8;
+template <> struct vec8<float> {
+  __device__ static inline void load(const float* p, float (&v)[8]) {
+    const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  __device__ static inline void store(float* p, const float (&v)[8]) {
+    *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+    *(float4*)(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+};
+template <> struct vec8<bf16_t> {
+  __device__ static inline void load(const bf16_t* p, float (&v)[8]) {
+    const uint4 r = *(const uint4*)p;
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(w[i] << 16);
+      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+  __device__ static inline void store(bf16_t* p, const float (&v)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      w[i] = (uint32_t)f32_to_bf16(v[2 * i]) | ((uint32_t)f32_to_bf16(v[2 * i + 1]) << 16);
+    *(uint4*)p = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+};
+
+__device__ inline float wave_sum(float x) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off);
+  return x;
+}
+
+// One wave per row, 8 elements per lane and access; needs cols % 8 == 0 and 16-byte aligned rows.
+// The second pass re-reads the row, which is still in the CU's cache.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const TI* __restrict__ x,
+                                                           const float* __restrict__ w,
+                                                           TO* __restrict__ y, int64_t rows, int cols,
+                                                           int64_t ldx, int64_t ldy, float eps) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const TI* xr = x + row * ldx;
+  TO* yr = y + row * ldy;
+  float ss = 0.f;
+  for (int c = lane * 8; c < cols; c += 512) {
+    float v[8];
+    vec8<TI>::load(xr + c, v);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss += v[i] * v[i];
+  }
+  const float inv = rsqrtf(wave_sum(ss) / (float)cols + eps);
+  for (int c = lane * 8; c < cols; c += 512) {
+    float v[8], g[8];
+    vec8<TI>::load(xr + c, v);
+    vec8<float>::load(w + c, g);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = v[i] * inv * g[i];
+    vec8<TO>::store(yr + c, v);
+  }
+}
+
+// sum = bf16(a + b + c) and norm = RMSNorm(sum) * w in one pass over the three inputs: the
+// residual update of one block fused with the input norm of the next.  The norm is taken over
+// the ROUNDED sum, so the result equals the two separate kernels bit for bit.
+__global__ __launch_bounds__(256) void add3_rmsnorm_bf16_kernel(
+    const bf16_t* __restrict__ a, const bf16_t* __restrict__ b, const bf16_t* __restrict__ c,
+    const float* __restrict__ w, bf16_t* __restrict__ sum, bf16_t* __restrict__ norm, int64_t rows,
+    int cols, float eps) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t base = row * cols;
+  float ss = 0.f;
+  for (int col = lane * 8; col < cols; col += 512) {
+    float va[8], vb[8], vc[8];
+    vec8<bf16_t>::load(a + base + col, va);
+    vec8<bf16_t>::load(b + base + col, vb);
+    vec8<bf16_t>::load(c + base + col, vc);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      va[i] = bf16_to_f32(f32_to_bf16(va[i] + vb[i] + vc[i]));
+      ss += va[i] * va[i];
+    }
+    vec8<bf16_t>::store(sum + base + col, va);
+  }
+  const float inv = rsqrtf(wave_sum(ss) / (float)cols + eps);
+  for (int col = lane * 8; col < cols; col += 512) {
+    float v[8], g[8];
+    vec8<bf16_t>::load(sum + base + col, v);      // this lane's own stores, read back
+    vec8<float>::load(w + col, g);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = v[i] * inv * g[i];
+    vec8<bf16_t>::store(norm + base + col, v);
+  }
+}
+
+__global__ __launch_bounds__(256) void add3_bf16_vec_kernel(const bf16_t* __restrict__ a,
+                                                            const bf16_t* __restrict__ b,
+                                                            const bf16_t* __restrict__ c,
+                                                            bf16_t* __restrict__ o, int64_t n8) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n8) return;
+  float va[8], vb[8], vc[8];
+  vec8<bf16_t>::load(a + i * 8, va);
+  vec8<bf16_t>::load(b + i * 8, vb);
+  vec8<bf16_t>::load(c + i * 8, vc);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) va[k] += vb[k] + vc[k];
+  vec8<bf16_t>::store(o + i * 8, va);
+}
+
 __global__ __launch_bounds__(256) void add3_bf16_kernel(const bf16_t* __restrict__ a,
                                                         const bf16_t* __restrict__ b,
                                                         const bf16_t* __restrict__ c,
@@ -482,6 +599,23 @@ extern "C" int mvpa_rmsnorm(const void* x, const float* weight, void* y, int64_t
   if (rows <= 0 || cols <= 0 || ldx < cols || ldy < cols) return MVPA_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   dim3 grid((unsigned)rows), block(256);
+  const int in_b = in_dtype == MVPA_F32 ? 4 : 2, out_b = out_dtype == MVPA_F32 ? 4 : 2;
+  const bool vec_ok = (in_dtype == MVPA_F32 || in_dtype == MVPA_BF16) &&
+                      (out_dtype == MVPA_F32 || out_dtype == MVPA_BF16) && cols % 8 == 0 &&
+                      (((uintptr_t)x | (uintptr_t)y | (uintptr_t)weight) & 15) == 0 &&
+                      (ldx * in_b) % 16 == 0 && (ldy * out_b) % 16 == 0;
+  if (vec_ok) {
+    dim3 vgrid((unsigned)((rows + 3) / 4));
+    if (in_dtype == MVPA_F32 && out_dtype == MVPA_F32)
+      hipLaunchKernelGGL((rmsnorm_rows_kernel<float, float>), vgrid, block, 0, s, (const float*)x, weight, (float*)y, rows, cols, ldx, ldy, eps);
+    else if (in_dtype == MVPA_F32)
+      hipLaunchKernelGGL((rmsnorm_rows_kernel<float, bf16_t>), vgrid, block, 0, s, (const float*)x, weight, (bf16_t*)y, rows, cols, ldx, ldy, eps);
+    else if (out_dtype == MVPA_BF16)
+      hipLaunchKernelGGL((rmsnorm_rows_kernel<bf16_t, bf16_t>), vgrid, block, 0, s, (const bf16_t*)x, weight, (bf16_t*)y, rows, cols, ldx, ldy, eps);
+    else
+      hipLaunchKernelGGL((rmsnorm_rows_kernel<bf16_t, float>), vgrid, block, 0, s, (const bf16_t*)x, weight, (float*)y, rows, cols, ldx, ldy, eps);
+    return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  }
   if (in_dtype == MVPA_F32 && out_dtype == MVPA_F32)
     hipLaunchKernelGGL((rmsnorm_kernel<float, float>), grid, block, 0, s, (const float*)x, weight, (float*)y, cols, ldx, ldy, eps);
   else if (in_dtype == MVPA_F32 && out_dtype == MVPA_BF16)
@@ -499,9 +633,30 @@ extern "C" int mvpa_add3_bf16(const void* a, const void* b, const void* c, void*
                               void* stream) {
   if (!a || !b || !c || !out) return MVPA_ERR_NULL;
   if (n <= 0) return MVPA_ERR_SHAPE;
+  if (n % 8 == 0 && (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)out) & 15) == 0) {
+    const int64_t n8 = n / 8;
+    hipLaunchKernelGGL(add3_bf16_vec_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)c,
+                       (bf16_t*)out, n8);
+    return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  }
   hipLaunchKernelGGL(add3_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)c,
                      (bf16_t*)out, n);
+  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+}
+
+extern "C" int mvpa_add3_rmsnorm_bf16(const void* a, const void* b, const void* c,
+                                      const float* weight, void* sum, void* norm, int64_t rows,
+                                      int32_t cols, float eps, void* stream) {
+  if (!a || !b || !c || !weight || !sum || !norm) return MVPA_ERR_NULL;
+  if (rows <= 0 || cols <= 0) return MVPA_ERR_SHAPE;
+  if (cols % 8 != 0 || (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)sum |
+                         (uintptr_t)norm | (uintptr_t)weight) & 15) != 0)
+    return MVPA_ERR_ALIGN;
+  hipLaunchKernelGGL(add3_rmsnorm_bf16_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                     (hipStream_t)stream, (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)c,
+                     weight, (bf16_t*)sum, (bf16_t*)norm, rows, cols, eps);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 

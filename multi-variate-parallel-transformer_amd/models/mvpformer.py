@@ -114,21 +114,42 @@ class MVPFormerBlock(nn.Module):
     def forward(self, hidden_states, positional_embedding, channel_embedding, layer_past=None,
                 attention_mask=None, head_mask=None, encoder_hidden_states=None,
                 encoder_attention_mask=None, use_cache=False, output_attentions=False):
+        outputs, _ = self.forward_fused(hidden_states, None, None, positional_embedding,
+                                        channel_embedding, layer_past=layer_past,
+                                        attention_mask=attention_mask, head_mask=head_mask,
+                                        use_cache=use_cache, output_attentions=output_attentions)
+        return outputs
+
+    def forward_fused(self, hidden_states, normed, next_norm, positional_embedding,
+                      channel_embedding, layer_past=None, attention_mask=None, head_mask=None,
+                      use_cache=False, output_attentions=False):
+        """The block with its norms at the seams: `normed` is ln_1(hidden_states) when the caller
+        already has it, `next_norm` the RMSNorm that will consume this block's output (the next
+        block's ln_1, or ln_f).  Returns (outputs, next_norm(output) or None); the residual sum and
+        that norm come out of one kernel."""
         residual = hidden_states
-        hidden_states = self.ln_1(hidden_states)
-        attn_outputs = self.attn(hidden_states, positional_embedding, channel_embedding,
+        if normed is None:
+            normed = self.ln_1(hidden_states)
+        attn_outputs = self.attn(normed, positional_embedding, channel_embedding,
                                  layer_past=layer_past, attention_mask=attention_mask,
                                  head_mask=head_mask, use_cache=use_cache,
                                  output_attentions=output_attentions)
         attn_output = attn_outputs[0]
         outputs = attn_outputs[1:]
-        mlp_output = self.mlp(hidden_states)
-        hidden_states = mvpa_hip.add3(residual, mlp_output, attn_output)
+        mlp_output = self.mlp(normed)
+        next_normed = None
+        if next_norm is not None and residual.dtype == torch.bfloat16:
+            hidden_states, next_normed = mvpa_hip.add3_rmsnorm(residual, mlp_output, attn_output,
+                                                               next_norm.weight, next_norm.eps)
+        else:
+            hidden_states = mvpa_hip.add3(residual, mlp_output, attn_output)
+            if next_norm is not None:
+                next_normed = next_norm(hidden_states)
         if use_cache:
             outputs = (hidden_states,) + outputs
         else:
             outputs = (hidden_states,) + outputs[1:]
-        return outputs
+        return outputs, next_normed
 
 
 class MVPFormerModel(nn.Module):
@@ -175,12 +196,17 @@ class MVPFormerModel(nn.Module):
             raise IndexError("more time steps / channels than embedding rows (n_positions / n_channels)")
         position_embeds = self.positional_embedding.weight[:t_len][None]
         channel_embeds = self.channel_embedding.weight[:c_len][None]
-        hidden_states = inputs_embeds
-        for block in self.h:
-            hidden_states = block(hidden_states, position_embeds, channel_embeds,
-                                  attention_mask=attention_mask, use_cache=False)[0]
-        hidden_states = self.ln_f(hidden_states)
-        return hidden_states.view(bsz, t_len, c_len, -1)
+        hidden_states, normed = inputs_embeds, None
+        n_layers = len(self.h)
+        for i, block in enumerate(self.h):
+            next_norm = self.h[i + 1].ln_1 if i + 1 < n_layers else self.ln_f
+            outputs, normed = block.forward_fused(hidden_states, normed, next_norm, position_embeds,
+                                                  channel_embeds, attention_mask=attention_mask,
+                                                  use_cache=False)
+            hidden_states = outputs[0]
+        if normed is None:                                       # no blocks
+            normed = self.ln_f(hidden_states)
+        return normed.view(bsz, t_len, c_len, -1)
 
 
 class MVPFormerHead(BrainDecider):

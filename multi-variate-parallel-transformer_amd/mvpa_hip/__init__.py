@@ -83,6 +83,8 @@ def load_library() -> ctypes.CDLL:
     lib.mvpa_rmsnorm.argtypes = [vp, vp, vp, i64, i32, i64, i64, f32, i32, i32, vp]
     lib.mvpa_add3_bf16.restype = ctypes.c_int
     lib.mvpa_add3_bf16.argtypes = [vp, vp, vp, vp, i64, vp]
+    lib.mvpa_add3_rmsnorm_bf16.restype = ctypes.c_int
+    lib.mvpa_add3_rmsnorm_bf16.argtypes = [vp, vp, vp, vp, vp, vp, i64, i32, f32, vp]
     lib.mvpa_wavedec_db4.restype = ctypes.c_int
     lib.mvpa_wavedec_db4.argtypes = [vp, vp, i64, i32, i32, i32, i64, vp]
     if lib.mvpa_version() != 1:
@@ -280,6 +282,26 @@ def add3(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor) -> torch.Tensor:
     _check(lib.mvpa_add3_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), out.data_ptr(),
                               a.numel(), _stream()))
     return out
+
+
+def add3_rmsnorm(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, weight: torch.Tensor,
+                 eps: float):
+    """(a + b + c, RMSNorm(a + b + c) * weight) in one pass; bit-identical to add3 followed by
+    rmsnorm.  Falls back to the two separate kernels when the row length is not a multiple of 8."""
+    lib = load_library()
+    _need_cuda(a, b, c, weight)
+    a, b, c = a.contiguous(), b.contiguous(), c.contiguous()
+    assert a.dtype == b.dtype == c.dtype == torch.bfloat16 and a.shape == b.shape == c.shape
+    cols = a.shape[-1]
+    if cols % 8 != 0:
+        total = add3(a, b, c)
+        return total, rmsnorm(total, weight, eps)
+    w = weight.detach().float().contiguous()
+    total, normed = torch.empty_like(a), torch.empty_like(a)
+    _check(lib.mvpa_add3_rmsnorm_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), w.data_ptr(),
+                                      total.data_ptr(), normed.data_ptr(), a.numel() // cols, cols,
+                                      float(eps), _stream()))
+    return total, normed
 
 
 def dwt_sizes(size_input: int):

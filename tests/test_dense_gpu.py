@@ -49,6 +49,36 @@ def test_rmsnorm(dtype):
     assert (y - ref).abs().max().item() <= tol
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,cols", [(37, 768), (5, 552), (130, 1536)])
+def test_rmsnorm_row_vector_path(dtype, rows, cols):
+    """Row lengths that are multiples of 8 take the one-wave-per-row kernel."""
+    g = torch.Generator().manual_seed(rows)
+    x = torch.randn(rows, cols, generator=g).to(dtype)
+    w = torch.rand(cols, generator=g) + 0.5
+    y = mvpa_hip.rmsnorm(x.cuda(), w.cuda(), 1e-5).float().cpu()
+    ref = O.rmsnorm(x.float(), w, 1e-5)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert (y - ref).abs().max().item() <= tol
+
+
+@pytest.mark.parametrize("rows,cols", [(37, 768), (3, 8), (129, 2048), (6, 1000)])
+def test_add3_rmsnorm_equals_separate_kernels(rows, cols):
+    """The fused residual-sum + norm is bit-identical to add3 followed by rmsnorm, and both
+    agree with the fp32 statement of the two operations."""
+    g = torch.Generator().manual_seed(cols)
+    a, b, c = (torch.randn(rows, cols, generator=g).bfloat16().cuda() for _ in range(3))
+    w = (torch.rand(cols, generator=g) + 0.5).cuda()
+    total, normed = mvpa_hip.add3_rmsnorm(a, b, c, w, 1e-5)
+    total2 = mvpa_hip.add3(a, b, c)
+    normed2 = mvpa_hip.rmsnorm(total2, w, 1e-5)
+    assert torch.equal(total, total2) and torch.equal(normed, normed2)
+    ref_sum = (a.float() + b.float() + c.float()).bfloat16()
+    assert torch.equal(total, ref_sum)
+    ref = O.rmsnorm(ref_sum.float().cpu(), w.cpu(), 1e-5)
+    assert (normed.float().cpu() - ref).abs().max().item() <= 2e-2
+
+
 def test_add3():
     g = torch.Generator().manual_seed(2)
     a, b, c = (torch.randn(5, 1000, generator=g).bfloat16() for _ in range(3))
