@@ -117,6 +117,53 @@ int mvpa_validate(const mvpa_fwd_args* args);
  * layers/mvpa.py:173-278.  Validates, then enqueues on `stream`. */
 int mvpa_forward(const mvpa_fwd_args* args, void* stream);
 
+/* ---- backward ------------------------------------------------------------------------------
+ * Argument block of mvpa_backward: the boundary of FlashMVPA.backward
+ * (attentions/attn.py:1140-1302).  Inputs as in mvpa_fwd_args plus the forward output o, the
+ * incoming gradient d_o and the forward's base-2 log-sum-exp.  Every gradient and workspace
+ * buffer is fp32, contiguous and caller-allocated; none needs to be cleared. */
+typedef struct mvpa_bwd_args {
+  uint32_t struct_size;      /* = sizeof(mvpa_bwd_args)                                       */
+  int32_t dtype;             /* dtype of q, k, v, o, d_o, biases and tables                   */
+  uint32_t flags;            /* MVPA_FLAG_CAUSAL | CONTENT | TIME_BIAS | CHAN_BIAS            */
+  int32_t B, H, Hkv, T, C, Dh;
+  int32_t window;
+  float sm_scale;
+  const void* q;             /* [B,H,N,Dh]-indexable, element strides below                   */
+  const void* k;             /* [B,Hkv,N,Dh]                                                  */
+  const void* v;
+  const void* o;             /* forward output                                                */
+  const void* d_o;           /* gradient of the loss with respect to o                        */
+  int64_t q_stride_b, q_stride_h, q_stride_n;
+  int64_t k_stride_b, k_stride_h, k_stride_n;
+  int64_t v_stride_b, v_stride_h, v_stride_n;
+  int64_t o_stride_b, o_stride_h, o_stride_n;
+  int64_t do_stride_b, do_stride_h, do_stride_n;
+  const void* bias_u;        /* [Hkv,Dh]                                                      */
+  const void* bias_v;
+  const void* bias_z;
+  const void* k_time;        /* [Hkv,T,Dh]                                                    */
+  const void* k_chan;        /* [Hkv,C,Dh]                                                    */
+  const uint8_t* chan_valid; /* nullable [B,C]                                                */
+  const float* key_bias;     /* nullable [B,N]                                                */
+  const float* lse;          /* [B*H,N] from the forward                                      */
+  float* dq;                 /* [B,H,N,Dh]   content-term share of dq (the reference's dq);
+                                its sum over batch, group and rows is dq_bias               */
+  float* dk;                 /* [B,Hkv,N,Dh] summed over the query heads of a group           */
+  float* dv;                 /* [B,Hkv,N,Dh]                                                  */
+  float* dbias_time;         /* [B,H,N,T] gradient of the table (q+v).k_time^T, by table column */
+  float* dbias_chan;         /* [B,H,N,C] gradient of the table (q+z).k_chan^T, by table column */
+  float* ws_delta;           /* workspace [B*H,N]                                             */
+  float* ws_time;            /* workspace [B,H,N,T]                                           */
+  float* ws_chan;            /* workspace [B,H,N,C]                                           */
+} mvpa_bwd_args;
+
+/* Backward of the fused forward; replaces FlashMVPA.backward and its _bwd_kernel
+ * (attentions/attn.py:350-1010, 1140-1302).  The gradients of q_btime, q_bchan, k_time and
+ * k_chan, and the bias-term share of dq, follow from dbias_time / dbias_chan by the matrix
+ * products that autograd applies to attentions/attn.py:1305-1314. */
+int mvpa_backward(const mvpa_bwd_args* args, void* stream);
+
 /* Which kernel mvpa_forward would run for these arguments: MVPA_KERNEL_GENERIC or
  * MVPA_KERNEL_MFMA (or a negative status). */
 int mvpa_select_kernel(const mvpa_fwd_args* args);

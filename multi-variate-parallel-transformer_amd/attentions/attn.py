@@ -6,14 +6,61 @@ layers/mvpa.py.  Differences in mechanism only: the relative-bias tables [B,H,N,
 [B,H,N,C] that the reference materialises in HBM (attentions/attn.py:1305-1314) are never
 built - the kernel contracts the query with the small key tables itself.
 
-Forward only: dropout (p_drop > 0), a torch.Generator and autograd are not implemented and
-raise NotImplementedError.
+Autograd: when an input requires grad the call goes through `FlashMVPA`, whose backward runs
+`mvpa_backward` (the boundary of the reference's FlashMVPA.backward, attentions/attn.py:1140-1302)
+and finishes the bias-table gradients with the matrix products that autograd applies to
+attentions/attn.py:1305-1314.  Dropout (p_drop > 0) and a torch.Generator are not implemented
+and raise NotImplementedError.
 """
 from __future__ import annotations
 
 import torch
 
 import mvpa_hip
+
+
+class FlashMVPA(torch.autograd.Function):
+    """Differentiable fused MVPA.  forward saves o and the base-2 log-sum-exp (the reference
+    saves o and L, attentions/attn.py:1124-1137); nothing of size N x N is kept."""
+
+    @staticmethod
+    def forward(ctx, q, u, vb, z, k, k_time, k_chan, v, causal, sm_scale, window, time_bias,
+                chan_bias, chan_valid):
+        out, lse = mvpa_hip.mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, sm_scale=sm_scale,
+                                         window=window, causal=causal, content=True,
+                                         time_bias=time_bias, chan_bias=chan_bias,
+                                         chan_valid=chan_valid, return_lse=True)
+        ctx.save_for_backward(q, u, vb, z, k, k_time, k_chan, v, out, lse)
+        ctx.conf = (causal, sm_scale, window, time_bias, chan_bias, chan_valid)
+        return out
+
+    @staticmethod
+    def backward(ctx, d_out):
+        q, u, vb, z, k, k_time, k_chan, v, out, lse = ctx.saved_tensors
+        causal, sm_scale, window, time_bias, chan_bias, chan_valid = ctx.conf
+        dq_c, dk, dv, dbt, dbc = mvpa_hip.mvpa_backward(
+            q, k, v, out, d_out.contiguous(), lse, u, vb, z, k_time, k_chan, sm_scale=sm_scale,
+            window=window, causal=causal, content=True, time_bias=time_bias, chan_bias=chan_bias,
+            chan_valid=chan_valid)
+        B, H, N, Dh = q.shape
+        Hkv = k.shape[1]
+        grp = H // Hkv
+        qf = q.float().view(B, Hkv, grp, N, Dh)
+        # time table (q+vb) @ k_time^T and channel table (q+z) @ k_chan^T, per kv head g
+        dbt = dbt.view(B, Hkv, grp, N, -1)
+        dbc = dbc.view(B, Hkv, grp, N, -1)
+        rt, ec = k_time.float(), k_chan.float()                    # [Hkv,T,Dh], [Hkv,C,Dh]
+        dq_t = torch.einsum("bgrnj,gjd->bgrnd", dbt, rt)
+        dq_ch = torch.einsum("bgrnj,gjd->bgrnd", dbc, ec)
+        dq = dq_c.view(B, Hkv, grp, N, Dh) + dq_t + dq_ch
+        du = dq_c.view(B, Hkv, grp, N, Dh).sum(dim=(0, 2, 3))
+        dvb = dq_t.sum(dim=(0, 2, 3))
+        dz = dq_ch.sum(dim=(0, 2, 3))
+        dk_time = torch.einsum("bgrnj,bgrnd->gjd", dbt, qf + vb.float()[None, :, None, None, :])
+        dk_chan = torch.einsum("bgrnj,bgrnd->gjd", dbc, qf + z.float()[None, :, None, None, :])
+        return (dq.view(B, H, N, Dh).to(q.dtype), du.to(u.dtype), dvb.to(vb.dtype), dz.to(z.dtype),
+                dk.to(k.dtype), dk_time.to(k_time.dtype), dk_chan.to(k_chan.dtype), dv.to(v.dtype),
+                None, None, None, None, None, None)
 
 
 def flash_mvpa(
@@ -55,12 +102,18 @@ def flash_mvpa(
         raise NotImplementedError(
             "flash_mvpa: a content window without relative biases (masking instead of zeroing) "
             "is not implemented")
-    if torch.is_grad_enabled() and any(
-            t.requires_grad for t in (q, q_bias, q_btime, q_bchan, k_glob, k_time, k_chan, v)):
-        raise NotImplementedError("flash_mvpa: backward is not implemented; call under torch.no_grad()")
     if not q.is_cuda:
         raise RuntimeError("flash_mvpa needs GPU tensors (there is no CPU path)")
     dh = q.shape[-1]
+    if torch.is_grad_enabled() and any(
+            t.requires_grad for t in (q, q_bias, q_btime, q_bchan, k_glob, k_time, k_chan, v)):
+        if out is not None:
+            raise NotImplementedError("flash_mvpa: a preallocated output cannot be used with autograd")
+        return FlashMVPA.apply(
+            q, q_bias.reshape(kv_heads, dh), q_btime.reshape(kv_heads, dh),
+            q_bchan.reshape(kv_heads, dh), k_glob, k_time.reshape(kv_heads, time_ctx, dh),
+            k_chan.reshape(kv_heads, chan_ctx, dh), v, bool(causal), sm_scale, int(window_size),
+            bool(rel_bias_time), bool(rel_bias_chan), chan_valid)
     return mvpa_hip.mvpa_forward(
         q, k_glob, v,
         q_bias.reshape(kv_heads, dh), q_btime.reshape(kv_heads, dh), q_bchan.reshape(kv_heads, dh),

@@ -44,6 +44,21 @@ class MvpaFwdArgs(ctypes.Structure):
     ]
 
 
+class MvpaBwdArgs(ctypes.Structure):
+    """Mirror of struct mvpa_bwd_args."""
+    _fields_ = (
+        [("struct_size", ctypes.c_uint32), ("dtype", ctypes.c_int32), ("flags", ctypes.c_uint32),
+         ("B", ctypes.c_int32), ("H", ctypes.c_int32), ("Hkv", ctypes.c_int32),
+         ("T", ctypes.c_int32), ("C", ctypes.c_int32), ("Dh", ctypes.c_int32),
+         ("window", ctypes.c_int32), ("sm_scale", ctypes.c_float)]
+        + [(n, ctypes.c_void_p) for n in ("q", "k", "v", "o", "d_o")]
+        + [(f"{t}_stride_{ax}", ctypes.c_int64) for t in ("q", "k", "v", "o", "do") for ax in "bhn"]
+        + [(n, ctypes.c_void_p) for n in (
+            "bias_u", "bias_v", "bias_z", "k_time", "k_chan", "chan_valid", "key_bias", "lse",
+            "dq", "dk", "dv", "dbias_time", "dbias_chan", "ws_delta", "ws_time", "ws_chan")]
+    )
+
+
 class MvpaError(RuntimeError):
     def __init__(self, status: int, text: str):
         super().__init__(f"libmvpa_hip: {text} (status {status})")
@@ -75,6 +90,8 @@ def load_library() -> ctypes.CDLL:
         fn.argtypes = [ctypes.POINTER(MvpaFwdArgs)]
     lib.mvpa_forward.restype = ctypes.c_int
     lib.mvpa_forward.argtypes = [ctypes.POINTER(MvpaFwdArgs), vp]
+    lib.mvpa_backward.restype = ctypes.c_int
+    lib.mvpa_backward.argtypes = [ctypes.POINTER(MvpaBwdArgs), vp]
     lib.mvpa_debug_maps.restype = ctypes.c_int
     lib.mvpa_debug_maps.argtypes = [i32, i32, i32, u32, vp, vp, vp, vp, vp]
     lib.mvpa_linear_bf16.restype = ctypes.c_int
@@ -207,6 +224,65 @@ def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float]
                   fp8_q_scale=q_scale, fp8_k_scale=k_scale)
     _check(lib.mvpa_forward(ctypes.byref(a), _stream()))
     return (out, lse) if return_lse else out
+
+
+def mvpa_backward(q, k, v, o, d_o, lse, u, vb, z, k_time, k_chan, *,
+                  sm_scale: Optional[float] = None, window: int = 10, causal: bool = True,
+                  content: bool = True, time_bias: bool = True, chan_bias: bool = True,
+                  chan_valid: Optional[torch.Tensor] = None,
+                  key_bias: Optional[torch.Tensor] = None):
+    """Backward of mvpa_forward at the boundary of the reference's FlashMVPA.backward
+    (attentions/attn.py:1140-1302).  Shapes as in mvpa_forward; o, lse are the forward's results.
+    Returns fp32 tensors (dq_content [B,H,N,Dh], dk [B,Hkv,N,Dh], dv [B,Hkv,N,Dh],
+    dbias_time [B,H,N,T], dbias_chan [B,H,N,C])."""
+    lib = load_library()
+    _need_cuda(q, k, v, o, d_o, lse, u, vb, z, k_time, k_chan, chan_valid, key_bias)
+    B, H, N, Dh = q.shape
+    Hkv = k.shape[1]
+    T, C = k_time.shape[-2], k_chan.shape[-2]
+    assert N == T * C, "N must equal T*C"
+    dt = q.dtype
+    u, vb, z = (t.to(dt).contiguous() for t in (u, vb, z))
+    k_time, k_chan = k_time.to(dt).contiguous(), k_chan.to(dt).contiguous()
+    o, d_o = o.to(dt), d_o.to(dt)
+    lse = lse.to(torch.float32).contiguous()
+    if chan_valid is not None:
+        chan_valid = chan_valid.to(torch.uint8).contiguous()
+    if key_bias is not None:
+        key_bias = key_bias.to(torch.float32).contiguous()
+    f32 = dict(dtype=torch.float32, device=q.device)
+    dq = torch.empty((B, H, N, Dh), **f32)
+    dk = torch.empty((B, Hkv, N, Dh), **f32)
+    dv = torch.empty((B, Hkv, N, Dh), **f32)
+    dbt = torch.empty((B, H, N, T), **f32)
+    dbc = torch.empty((B, H, N, C), **f32)
+    ws_delta = torch.empty((B, H, N), **f32)
+    ws_time = torch.empty((B, H, N, T), **f32)
+    ws_chan = torch.empty((B, H, N, C), **f32)
+    a = MvpaBwdArgs()
+    a.struct_size = ctypes.sizeof(MvpaBwdArgs)
+    a.dtype = _dtype_code(dt)
+    a.flags = ((FLAG_CAUSAL if causal else 0) | (FLAG_CONTENT if content else 0) |
+               (FLAG_TIME_BIAS if time_bias else 0) | (FLAG_CHAN_BIAS if chan_bias else 0))
+    a.B, a.H, a.Hkv, a.T, a.C, a.Dh = B, H, Hkv, T, C, Dh
+    a.window = window
+    a.sm_scale = (1.0 / Dh ** 0.5) if sm_scale is None else float(sm_scale)
+    for name, t in (("q", q), ("k", k), ("v", v), ("o", o), ("do", d_o)):
+        if t.stride(-1) != 1:
+            raise ValueError(f"{name}: last dim must be contiguous")
+        setattr(a, "d_o" if name == "do" else name, t.data_ptr())
+        for ax, st in zip("bhn", t.stride()[:3]):
+            setattr(a, f"{name}_stride_{ax}", st)
+    a.bias_u, a.bias_v, a.bias_z = u.data_ptr(), vb.data_ptr(), z.data_ptr()
+    a.k_time, a.k_chan = k_time.data_ptr(), k_chan.data_ptr()
+    a.chan_valid = chan_valid.data_ptr() if chan_valid is not None else None
+    a.key_bias = key_bias.data_ptr() if key_bias is not None else None
+    a.lse = lse.data_ptr()
+    a.dq, a.dk, a.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    a.dbias_time, a.dbias_chan = dbt.data_ptr(), dbc.data_ptr()
+    a.ws_delta, a.ws_time, a.ws_chan = ws_delta.data_ptr(), ws_time.data_ptr(), ws_chan.data_ptr()
+    _check(lib.mvpa_backward(ctypes.byref(a), _stream()))
+    return dq, dk, dv, dbt, dbc
 
 
 def debug_maps(T: int, C: int, window: int = 10, flags: int = 15, chan_valid=None,

@@ -1,0 +1,115 @@
+"""Parity of the HIP backward (mvpa_backward through the FlashMVPA autograd function) with
+reverse-mode differentiation of the oracle's closed-form MVPA in float64.
+
+The oracle forward is pinned in tests/test_oracle.py; its gradient is what torch.autograd derives
+from it (and tests/test_oracle.py::test_direct_gradcheck checks that derivation against finite
+differences).  Tolerances: fp32 inputs max-abs <= 2e-5 + 1e-4 * max|ref| per gradient; bf16
+inputs rel-L2 <= 2e-2 per gradient (inputs rounded to bf16 on both sides, gradients returned in
+bf16)."""
+import math
+import os
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for p in (os.path.join(ROOT, "multi-variate-parallel-transformer_amd"), ROOT):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+from oracle import mvpa_oracle as O  # noqa: E402
+from mvpa_hip.synthetic import make_mvpa_inputs  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ("q", "u", "vb", "z", "k", "k_time", "k_chan", "v")
+
+
+def _oracle_grads(inp, d_out, window, chan_valid=None, time_bias=True, chan_bias=True):
+    leaves = {n: getattr(inp, n).double().clone().requires_grad_(True) for n in NAMES}
+    k_time = leaves["k_time"] if time_bias else leaves["k_time"] * 0
+    k_chan = leaves["k_chan"] if chan_bias else leaves["k_chan"] * 0
+    vb = leaves["vb"] if time_bias else leaves["vb"] * 0
+    z = leaves["z"] if chan_bias else leaves["z"] * 0
+    out = O.mvpa_direct(leaves["q"], leaves["k"], leaves["v"], leaves["u"], vb, z, k_time, k_chan,
+                        window=window, chan_valid=chan_valid)
+    grads = torch.autograd.grad((out * d_out.double()).sum(), [leaves[n] for n in NAMES],
+                                allow_unused=True)
+    return out.detach(), {n: (g if g is not None else torch.zeros_like(leaves[n])) for n, g in zip(NAMES, grads)}
+
+
+def _gpu_grads(inp, d_out, window, dtype, chan_valid=None, time_bias=True, chan_bias=True):
+    from attentions import flashmvpa
+    hkv, dh = inp.u.shape
+    t_len, c_len = inp.k_time.shape[1], inp.k_chan.shape[1]
+    leaves = {n: getattr(inp, n).to(dtype).cuda().requires_grad_(True) for n in NAMES}
+    out = flashmvpa(leaves["q"], leaves["u"].view(1, hkv, 1, dh), leaves["vb"].view(1, hkv, 1, dh),
+                    leaves["z"].view(1, hkv, 1, dh), leaves["k"],
+                    leaves["k_time"].view(1, hkv, t_len, dh), leaves["k_chan"].view(1, hkv, c_len, dh),
+                    leaves["v"], True, 1.0 / math.sqrt(dh), window_size=window,
+                    rel_bias_time=time_bias, rel_bias_chan=chan_bias,
+                    chan_valid=chan_valid.cuda() if chan_valid is not None else None)
+    out.backward(d_out.to(dtype).cuda())
+    return out.detach().float().cpu(), {n: (leaves[n].grad.float().cpu() if leaves[n].grad is not None
+                                            else torch.zeros_like(getattr(inp, n))) for n in NAMES}
+
+
+CASES = [
+    dict(B=2, C=8, T=32, H=4, Hkv=4, Dh=32, window=10),     # the reference's CPU-runnable size
+    dict(B=1, C=3, T=13, H=4, Hkv=2, Dh=16, window=10),     # GQA, window active
+    dict(B=2, C=5, T=7, H=2, Hkv=1, Dh=64, window=10),      # window vacuous, ragged C
+    dict(B=1, C=4, T=14, H=2, Hkv=2, Dh=32, window=3),      # narrow window
+    dict(B=1, C=6, T=9, H=2, Hkv=2, Dh=128, window=0),      # content everywhere
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "B{B}C{C}T{T}H{H}g{Hkv}D{Dh}w{window}".format(**c))
+def test_backward_fp32_matches_oracle_autograd(case):
+    cfg = dict(case)
+    window = cfg.pop("window")
+    inp = make_mvpa_inputs(seed=3, qkv_unit=True, **cfg)
+    g = torch.Generator().manual_seed(11)
+    d_out = torch.randn(inp.q.shape, generator=g)
+    ref_out, ref = _oracle_grads(inp, d_out, window)
+    out, got = _gpu_grads(inp, d_out, window, torch.float32)
+    assert (out.double() - ref_out).abs().max().item() <= 1e-5
+    for n in NAMES:
+        err = (got[n].double() - ref[n]).abs().max().item()
+        assert err <= 2e-5 + 1e-4 * ref[n].abs().max().item(), (n, err)
+
+
+def test_backward_with_channel_validity():
+    inp = make_mvpa_inputs(B=2, C=6, T=12, H=2, Hkv=2, Dh=32, seed=5, qkv_unit=True)
+    valid = torch.tensor([[1, 1, 0, 1, 1, 0], [0, 1, 1, 1, 1, 1]], dtype=torch.bool)
+    d_out = torch.randn(inp.q.shape, generator=torch.Generator().manual_seed(2))
+    _, ref = _oracle_grads(inp, d_out, 10, chan_valid=valid)
+    _, got = _gpu_grads(inp, d_out, 10, torch.float32, chan_valid=valid)
+    for n in NAMES:
+        err = (got[n].double() - ref[n]).abs().max().item()
+        assert err <= 2e-5 + 1e-4 * ref[n].abs().max().item(), (n, err)
+    # keys of absent channels receive no gradient at all
+    absent = (~valid)[:, None, None, :].expand(2, 2, 12, 6).reshape(2, 2, 72)
+    assert got["k"][absent].abs().max().item() == 0.0
+    assert got["v"][absent].abs().max().item() == 0.0
+
+
+def test_backward_bf16_within_tolerance():
+    inp = make_mvpa_inputs(B=1, C=16, T=24, H=4, Hkv=2, Dh=64, seed=9, qkv_unit=True).round_to(torch.bfloat16)
+    d_out = torch.randn(inp.q.shape, generator=torch.Generator().manual_seed(4)).bfloat16().float()
+    _, ref = _oracle_grads(inp, d_out, 10)
+    _, got = _gpu_grads(inp, d_out, 10, torch.bfloat16)
+    for n in NAMES:
+        rel = (got[n].double() - ref[n]).norm().item() / max(ref[n].norm().item(), 1e-30)
+        assert rel <= 2e-2, (n, rel)
+
+
+def test_backward_rows_are_causal():
+    """do confined to the first time steps must leave dk/dv of later keys exactly zero."""
+    inp = make_mvpa_inputs(B=1, C=4, T=10, H=2, Hkv=2, Dh=32, seed=1, qkv_unit=True)
+    d_out = torch.zeros(inp.q.shape)
+    d_out[:, :, : 3 * 4] = torch.randn(1, 2, 12, 32, generator=torch.Generator().manual_seed(8))
+    _, got = _gpu_grads(inp, d_out, 10, torch.float32)
+    assert got["k"][:, :, 3 * 4:].abs().max().item() == 0.0
+    assert got["v"][:, :, 3 * 4:].abs().max().item() == 0.0
+    assert got["q"][:, :, 3 * 4:].abs().max().item() == 0.0

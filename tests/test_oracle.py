@@ -200,3 +200,16 @@ def test_golden_c1_fixture():
     assert np.array_equal(inp.k_time[0, :2].numpy(), g["k_time_probe"])
     out, _ = _rel_attn(inp)
     assert np.abs(out.numpy() - g["out"]).max() <= 5e-6
+
+
+def test_direct_gradcheck():
+    """The closed-form oracle is differentiable and its reverse-mode gradient agrees with finite
+    differences (float64, windowed, GQA): the reference for the backward parity tests."""
+    torch.manual_seed(0)
+    B, H, Hkv, T, C, Dh = 1, 2, 1, 5, 2, 4
+    mk = lambda *s: (torch.randn(*s, dtype=torch.float64) * 0.5).requires_grad_(True)  # noqa: E731
+    q, k, v = mk(B, H, T * C, Dh), mk(B, Hkv, T * C, Dh), mk(B, Hkv, T * C, Dh)
+    u, vb, z = mk(Hkv, Dh), mk(Hkv, Dh), mk(Hkv, Dh)
+    kt, kc = mk(Hkv, T, Dh), mk(Hkv, C, Dh)
+    assert torch.autograd.gradcheck(lambda *a: O.mvpa_direct(*a, window=2),
+                                    (q, k, v, u, vb, z, kt, kc), eps=1e-6, atol=1e-6)
