@@ -189,6 +189,8 @@ struct Cfg {
   static constexpr int MAIN_BYTES = RING_BYTES + STB_BYTES;
   static constexpr int SETUP_BYTES = NW * CP * 32 * 4;
   static constexpr int LDS_BYTES = MAIN_BYTES > SETUP_BYTES ? MAIN_BYTES : SETUP_BYTES;
+  // the set-up scratch fits behind the stages of the prologue tiles
+  static constexpr bool EARLY = STAGES >= 2 && SETUP_BYTES <= STAGE_BYTES + STB_BYTES;
   static_assert(NW % NCT == 0, "waves must cover whole time steps");
   static_assert(TILE_BYTES % 1024 == 0, "tile must be a whole number of wave loads");
   static_assert(WLOADS % NW == 0 || WLOADS < NW, "every loading wave issues the same number of loads");
@@ -200,7 +202,8 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   constexpr int CP = G::CP, KS = G::KS, MT = G::MT, ROWB = G::ROWB, CHUNKS = G::CHUNKS;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   float* Stb_all = (float*)(smem_raw + G::RING_BYTES);          // [NW][32][32]
-  float* setup_all = (float*)smem_raw;                          // [NW][CP][32], aliases the ring
+  // [NW][CP][32] set-up scratch; aliases the ring (and the slabs), see EARLY
+  float* setup_all = (float*)(smem_raw + (G::EARLY ? (STAGES - 1) * G::STAGE_BYTES : 0));
 
   const int tid = threadIdx.x, lane = tid & 63;
   // the wave index is uniform by construction; reading it through a scalar register lets the
@@ -272,6 +275,54 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   const bf16_t* bz = (const bf16_t*)a.bias_z + g * DH;
   const uint8_t* valid = a.chan_valid ? a.chan_valid + (int64_t)b * C_ : nullptr;
   const float sc2 = a.sm_scale * kLog2e;           // scores live in the base-2 domain
+
+  // =========================== tile ring ===========================
+  // Wave-load li of a tile covers bytes [li*1024, li*1024+1024): lane L delivers physical chunk
+  // li*64+L, i.e. row (li*64+L)/CHUNKS; the logical chunk it fetches is un-swizzled here.  Rows of
+  // padded channels fetch the last real channel instead; whatever lands in rows of padded or
+  // absent channels is neutralised by Ec = 0 / Bc = -inf.
+  int k_off[G::LPW], v_off[G::LPW];
+#pragma unroll
+  for (int i = 0; i < G::LPW; ++i) {
+    const int pc = (wave + NW * i) * 64 + lane;
+    const int row = pc / CHUNKS, phys = pc % CHUNKS;
+    const int rowc = min(row, C_ - 1);
+    k_off[i] = (int)(rowc * a.k_stride_n) + ((phys ^ swz_k<DH>(row)) << 3);
+    v_off[i] = (int)(rowc * a.v_stride_n) + ((phys ^ swz_v<DH>(row)) << 3);
+  }
+  // first key step that needs K: the band of the earliest query step of this workgroup
+  const int tk_near = !has_content ? tq_hi + 1 : (W <= 0 || tq_hi == T_ - 1) ? 0 : max(0, tq0 - W);
+  const uint32_t ring_lds = (uint32_t)(uintptr_t)(LDS_PTR(unsigned char))smem_raw;
+  auto issue_tile = [&](int tk, int stage_idx, bool with_k) {
+    const uint32_t stage = ring_lds + stage_idx * G::STAGE_BYTES;
+    const bf16_t* vsrc = vbase + (int64_t)tk * C_ * a.v_stride_n;
+#pragma unroll
+    for (int i = 0; i < G::LPW; ++i) {
+      const int li = wave + NW * i;
+      if (li < G::WLOADS) load_to_lds_16(vsrc + v_off[i], stage + G::TILE_BYTES + li * 1024);
+    }
+    if (with_k) {
+      const bf16_t* ksrc = kbase + (int64_t)tk * C_ * a.k_stride_n;
+#pragma unroll
+      for (int i = 0; i < G::LPW; ++i) {
+        const int li = wave + NW * i;
+        if (li < G::WLOADS) load_to_lds_16(ksrc + k_off[i], stage + li * 1024);
+      }
+    }
+  };
+  // wave loads this wave issues per (V or K) tile: a compile-time count unless the tile is
+  // smaller than one load per wave
+  const int n_issue = G::WLOADS >= NW ? G::LPW : (wave < G::WLOADS ? 1 : 0);
+
+  // prologue: tiles 0 .. STAGES-2 in flight.  Where the set-up scratch fits into what the
+  // prologue leaves alone (the last stage and the time-bias slabs, both first written after the
+  // first barrier of the key loop) the tiles are requested right away, so that their round trip
+  // overlaps the set-up instead of following it.
+  if (G::EARLY) {
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s)
+      if (s <= tq_hi) issue_tile(s, s, s >= tk_near);
+  }
 
   // =========================== setup: Qu, Qv, channel bias tile, Ec ===========================
   bf16x8 Qu[KS], Qv[KS];     // (q+u), (q+v) * scale as QK^T / time-slab B operands
@@ -391,50 +442,12 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[mt][i] = 0.f;
 
-  // =========================== tile ring ===========================
-  // Wave-load li of a tile covers bytes [li*1024, li*1024+1024): lane L delivers physical chunk
-  // li*64+L, i.e. row (li*64+L)/CHUNKS; the logical chunk it fetches is un-swizzled here.  Rows of
-  // padded channels fetch the last real channel instead; whatever lands in rows of padded or
-  // absent channels is neutralised by Ec = 0 / Bc = -inf.
-  int k_off[G::LPW], v_off[G::LPW];
+  if (!G::EARLY) {
+    lds_barrier();           // the set-up scratch aliases the stages the prologue fills
 #pragma unroll
-  for (int i = 0; i < G::LPW; ++i) {
-    const int pc = (wave + NW * i) * 64 + lane;
-    const int row = pc / CHUNKS, phys = pc % CHUNKS;
-    const int rowc = min(row, C_ - 1);
-    k_off[i] = (int)(rowc * a.k_stride_n) + ((phys ^ swz_k<DH>(row)) << 3);
-    v_off[i] = (int)(rowc * a.v_stride_n) + ((phys ^ swz_v<DH>(row)) << 3);
+    for (int s = 0; s < STAGES - 1; ++s)
+      if (s <= tq_hi) issue_tile(s, s, s >= tk_near);
   }
-  // first key step that needs K: the band of the earliest query step of this workgroup
-  const int tk_near = !has_content ? tq_hi + 1 : (W <= 0 || tq_hi == T_ - 1) ? 0 : max(0, tq0 - W);
-  const uint32_t ring_lds = (uint32_t)(uintptr_t)(LDS_PTR(unsigned char))smem_raw;
-  auto issue_tile = [&](int tk, int stage_idx, bool with_k) {
-    const uint32_t stage = ring_lds + stage_idx * G::STAGE_BYTES;
-    const bf16_t* vsrc = vbase + (int64_t)tk * C_ * a.v_stride_n;
-#pragma unroll
-    for (int i = 0; i < G::LPW; ++i) {
-      const int li = wave + NW * i;
-      if (li < G::WLOADS) load_to_lds_16(vsrc + v_off[i], stage + G::TILE_BYTES + li * 1024);
-    }
-    if (with_k) {
-      const bf16_t* ksrc = kbase + (int64_t)tk * C_ * a.k_stride_n;
-#pragma unroll
-      for (int i = 0; i < G::LPW; ++i) {
-        const int li = wave + NW * i;
-        if (li < G::WLOADS) load_to_lds_16(ksrc + k_off[i], stage + li * 1024);
-      }
-    }
-  };
-  // wave loads this wave issues per (V or K) tile: a compile-time count unless the tile is
-  // smaller than one load per wave
-  const int n_issue = G::WLOADS >= NW ? G::LPW : (wave < G::WLOADS ? 1 : 0);
-
-  lds_barrier();             // setup scratch aliases the ring
-
-  // prologue: tiles 0 .. STAGES-2 in flight
-#pragma unroll
-  for (int s = 0; s < STAGES - 1; ++s)
-    if (s <= tq_hi) issue_tile(s, s, s >= tk_near);
 
   float* Stb = Stb_all + wave * (32 * 32);
   // key steps 0 .. far_max are "far" for this wave's queries (content term absent or zeroed)
