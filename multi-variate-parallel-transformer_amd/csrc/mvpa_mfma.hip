@@ -248,9 +248,19 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
           tile = nt - 2 - r / merged;
         }
       }
+    } else if (nt > 1) {
+      // no XCD affinity to keep (the (b, h) do not divide over the 8 XCDs): last tiles first,
+      // then (b, h) by (b, h)
+      if (L < nbh) {
+        bh = L;
+        tile = nt - 1;
+      } else {
+        bh = (L - nbh) / (nt - 1);
+        tile = nt - 2 - (L - nbh) % (nt - 1);
+      }
     } else {
-      bh = L / nt;
-      tile = nt - 1 - L % nt;
+      bh = L;
+      tile = 0;
     }
   }
   const int b = bh / a.H, h = bh % a.H;

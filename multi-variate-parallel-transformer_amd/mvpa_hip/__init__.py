@@ -323,6 +323,22 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = 
     return out.view(*x.shape[:-1], N)
 
 
+def _as_f32_weight(weight: torch.Tensor) -> torch.Tensor:
+    """fp32 contiguous copy of a (norm) weight, kept on the tensor object and refreshed when the
+    tensor is modified in place, so a bf16 module does not convert its weight on every call."""
+    if weight.dtype == torch.float32 and weight.is_contiguous():
+        return weight.detach()
+    cached = getattr(weight, "_mvpa_f32", None)
+    if cached is not None and cached[0] == weight._version and cached[1].device == weight.device:
+        return cached[1]
+    w32 = weight.detach().to(torch.float32).contiguous()
+    try:
+        weight._mvpa_f32 = (weight._version, w32)
+    except AttributeError:
+        pass
+    return w32
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5,
             out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """RMSNorm over the last dim.  x may be a 2-D row-pitched view (unit last stride); `out`, if
@@ -342,8 +358,8 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5,
     else:
         y = y2 = out
         assert out.dim() == 2 and out.shape == (rows, cols) and out.stride(-1) == 1
-    w = weight if weight.dtype == torch.float32 else weight.to(torch.float32)
-    _check(lib.mvpa_rmsnorm(x2.data_ptr(), w.contiguous().data_ptr(), y2.data_ptr(), rows, cols,
+    w = _as_f32_weight(weight)
+    _check(lib.mvpa_rmsnorm(x2.data_ptr(), w.data_ptr(), y2.data_ptr(), rows, cols,
                             x2.stride(0), y2.stride(0), eps, _dtype_code(x.dtype), _dtype_code(od),
                             _stream()))
     return y
@@ -372,7 +388,7 @@ def add3_rmsnorm(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, weight: torc
     if cols % 8 != 0:
         total = add3(a, b, c)
         return total, rmsnorm(total, weight, eps)
-    w = weight.detach().float().contiguous()
+    w = _as_f32_weight(weight)
     total, normed = torch.empty_like(a), torch.empty_like(a)
     _check(lib.mvpa_add3_rmsnorm_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), w.data_ptr(),
                                       total.data_ptr(), normed.data_ptr(), a.numel() // cols, cols,
