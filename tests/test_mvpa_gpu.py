@@ -170,6 +170,9 @@ MFMA_SHAPES = [
     dict(B=1, C=20, T=37, H=1, Dh=128, validity=True),
     dict(B=1, C=1, T=45, H=2, Dh=32),
     dict(B=3, C=33, T=5, H=3, Dh=32),                              # B*H not a multiple of 8
+    dict(B=2, C=16, T=1, H=4, Dh=64),                              # a single time step
+    dict(B=4, C=64, T=9, H=4, Dh=64),                              # two (b,h) per XCD: merged tail order
+    dict(B=2, C=48, T=11, H=8, Dh=64, Hkv=2),                      # window just vacuous, GQA 4:1
 ]
 
 
