@@ -278,7 +278,7 @@ __global__ __launch_bounds__(BWD_THREADS) void mvpa_bwd_key_kernel(mvpa_bwd_args
 }
 
 template <typename T, int DH>
-static int launch_bwd_t(const mvpa_bwd_args* a, hipStream_t stream) {
+static int launch_bwd_t(const mvpa_bwd_args* a, hipStream_t stream, bool query_pass) {
   const int N = a->T * a->C;
   const size_t lds_q = (size_t)(2 * BWD_TILE * DH + BWD_THREADS * (a->C + 1)) * sizeof(float);
   const size_t lds_k = (size_t)(2 * BWD_TILE * DH + 2 * BWD_TILE) * sizeof(float);
@@ -287,19 +287,21 @@ static int launch_bwd_t(const mvpa_bwd_args* a, hipStream_t stream) {
   auto kk = mvpa_bwd_key_kernel<T, DH>;
   (void)hipFuncSetAttribute((const void*)kq, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_q);
   const unsigned nb = (unsigned)((N + BWD_THREADS - 1) / BWD_THREADS);
-  hipLaunchKernelGGL(kq, dim3(nb, a->B * a->H), dim3(BWD_THREADS), lds_q, stream, *a);
-  if (hipGetLastError() != hipSuccess) return MVPA_ERR_LAUNCH;
+  if (query_pass) {
+    hipLaunchKernelGGL(kq, dim3(nb, a->B * a->H), dim3(BWD_THREADS), lds_q, stream, *a);
+    if (hipGetLastError() != hipSuccess) return MVPA_ERR_LAUNCH;
+  }
   hipLaunchKernelGGL(kk, dim3(nb, a->B * a->Hkv), dim3(BWD_THREADS), lds_k, stream, *a);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 
 template <typename T>
-static int launch_bwd_dh(const mvpa_bwd_args* a, hipStream_t stream) {
+static int launch_bwd_dh(const mvpa_bwd_args* a, hipStream_t stream, bool query_pass) {
   switch (a->Dh) {
-    case 16: return launch_bwd_t<T, 16>(a, stream);
-    case 32: return launch_bwd_t<T, 32>(a, stream);
-    case 64: return launch_bwd_t<T, 64>(a, stream);
-    case 128: return launch_bwd_t<T, 128>(a, stream);
+    case 16: return launch_bwd_t<T, 16>(a, stream, query_pass);
+    case 32: return launch_bwd_t<T, 32>(a, stream, query_pass);
+    case 64: return launch_bwd_t<T, 64>(a, stream, query_pass);
+    case 128: return launch_bwd_t<T, 128>(a, stream, query_pass);
   }
   return MVPA_ERR_HEAD_DIM;
 }
@@ -319,7 +321,16 @@ extern "C" int mvpa_backward(const mvpa_bwd_args* a, void* stream) {
   if (a->B <= 0) return MVPA_ERR_SHAPE;
   if ((a->flags & (MVPA_FLAG_TIME_BIAS | MVPA_FLAG_CHAN_BIAS)) && !(a->flags & MVPA_FLAG_CAUSAL))
     return MVPA_ERR_NONCAUSAL_BIAS;
-  if (a->dtype == MVPA_F32) return mvpa::launch_bwd_dh<float>(a, (hipStream_t)stream);
-  if (a->dtype == MVPA_BF16) return mvpa::launch_bwd_dh<mvpa::bf16_t>(a, (hipStream_t)stream);
+  if (a->dtype == MVPA_F32) return mvpa::launch_bwd_dh<float>(a, (hipStream_t)stream, true);
+  if (a->dtype == MVPA_BF16) {
+    // bf16, Dh = 64, C <= 64: the query pass runs on MFMA; the key pass is still the fp32 one
+    bool query_pass = true;
+    if (mvpa_bwd_query_mfma_supported(a)) {
+      const int st = mvpa_launch_bwd_query_mfma(a, (hipStream_t)stream);
+      if (st != MVPA_OK) return st;
+      query_pass = false;
+    }
+    return mvpa::launch_bwd_dh<mvpa::bf16_t>(a, (hipStream_t)stream, query_pass);
+  }
   return MVPA_ERR_DTYPE;
 }

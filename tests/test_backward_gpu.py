@@ -104,6 +104,32 @@ def test_backward_bf16_within_tolerance():
         assert rel <= 2e-2, (n, rel)
 
 
+BF16_CASES = [
+    dict(B=1, C=64, T=12, H=2, Hkv=2, Dh=64, window=10),      # two waves per time step
+    dict(B=1, C=40, T=37, H=2, Hkv=1, Dh=64, window=10),      # ragged channels, two 32-step slabs, GQA
+    dict(B=2, C=8, T=70, H=1, Hkv=1, Dh=64, window=4),        # three slabs, narrow window
+    dict(B=1, C=33, T=9, H=2, Hkv=2, Dh=64, window=0),        # content everywhere
+]
+
+
+@pytest.mark.parametrize("case", BF16_CASES, ids=lambda c: "B{B}C{C}T{T}H{H}g{Hkv}w{window}".format(**c))
+def test_backward_bf16_mfma_query_pass(case):
+    """bf16, Dh = 64, C <= 64 takes the MFMA query pass (dq, bias-table gradients)."""
+    cfg = dict(case)
+    window = cfg.pop("window")
+    inp = make_mvpa_inputs(seed=13, qkv_unit=True, **cfg).round_to(torch.bfloat16)
+    d_out = torch.randn(inp.q.shape, generator=torch.Generator().manual_seed(6)).bfloat16().float()
+    valid = None
+    if cfg["C"] == 40:
+        valid = torch.ones(cfg["B"], 40, dtype=torch.bool)
+        valid[:, [3, 17, 39]] = False
+    _, ref = _oracle_grads(inp, d_out, window, chan_valid=valid)
+    _, got = _gpu_grads(inp, d_out, window, torch.bfloat16, chan_valid=valid)
+    for n in NAMES:
+        rel = (got[n].double() - ref[n]).norm().item() / max(ref[n].norm().item(), 1e-30)
+        assert rel <= 2e-2, (n, rel)
+
+
 def test_backward_rows_are_causal():
     """do confined to the first time steps must leave dk/dv of later keys exactly zero."""
     inp = make_mvpa_inputs(B=1, C=4, T=10, H=2, Hkv=2, Dh=32, seed=1, qkv_unit=True)
