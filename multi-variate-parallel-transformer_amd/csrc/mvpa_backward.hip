@@ -323,14 +323,13 @@ extern "C" int mvpa_backward(const mvpa_bwd_args* a, void* stream) {
     return MVPA_ERR_NONCAUSAL_BIAS;
   if (a->dtype == MVPA_F32) return mvpa::launch_bwd_dh<float>(a, (hipStream_t)stream, true);
   if (a->dtype == MVPA_BF16) {
-    // bf16, Dh = 64, C <= 64: the query pass runs on MFMA; the key pass is still the fp32 one
-    bool query_pass = true;
+    // bf16, Dh = 64, C <= 64: both passes run on MFMA
     if (mvpa_bwd_query_mfma_supported(a)) {
       const int st = mvpa_launch_bwd_query_mfma(a, (hipStream_t)stream);
       if (st != MVPA_OK) return st;
-      query_pass = false;
+      return mvpa_launch_bwd_key_mfma(a, (hipStream_t)stream);
     }
-    return mvpa::launch_bwd_dh<mvpa::bf16_t>(a, (hipStream_t)stream, query_pass);
+    return mvpa::launch_bwd_dh<mvpa::bf16_t>(a, (hipStream_t)stream, true);
   }
   return MVPA_ERR_DTYPE;
 }

@@ -1,4 +1,4 @@
-// MVPA backward on MFMA (bf16, Dh = 64, C <= 64): the QUERY pass.
+// MVPA backward on MFMA (bf16, Dh = 64, C <= 64): the QUERY pass (the KEY pass follows below).
 //
 // Same tiling as the forward kernel: queries and keys are tiled by time step, a wave owns 32
 // query channels of one time step, products are formed transposed (a lane owns one query), the
@@ -388,6 +388,221 @@ int mvpa_launch_bwd_query_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
     auto kern = mvpa_bwd_query_mfma_kernel<2>;
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, *a);
+  }
+  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+}
+
+// ==========================================================================================
+// The KEY pass: dk, dv.  One workgroup per key time step tk and kv head; a wave owns 32 key
+// channels (its K and V rows stay in registers as MFMA B operands) and one of the NCT query-channel
+// tiles; it walks the query time steps tq >= tk of every query head of the group.  Products are
+// formed NON-transposed here, S[q][key] = (q+u) K^T, so that a lane owns one key and the
+// contraction index of dv^T = dO^T P and dk^T = (q+u)^T dS is the register index:
+//     S   = (q+u) K^T (inside the window) + chan[q][C-1-|cq-ck|] + time[q][tk]
+//     P   = exp2(S - L[q]),  dP = dO V^T,  dS = P o (dP - delta[q])
+//     dv^T[d][key] += dO^T[d][q] P[q][key],   dk^T[d][key] += (q+u)^T[d][q] dS[q][key]
+// The per-query bias tables, L and delta come from the query pass (workspace, natural units).
+// Per (head, tq) the workgroup stages (q+u) * scale and dO (each in the two swizzles), the
+// channel-table rows and the per-query scalars in LDS.
+// ==========================================================================================
+namespace mvpa {
+namespace bwdq {
+
+template <int NCT>
+__global__ __launch_bounds__(NCT * NCT * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_args a) {
+  constexpr int CP = NCT * 32, TILE = CP * ROWB, NWK = NCT * NCT, NTHR = NWK * 64;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  unsigned char* Qrow = smem;                     // (q+u)*scale, row-fragment swizzle
+  unsigned char* Qtr = smem + TILE;               // same, transposing-read swizzle
+  unsigned char* Drow = smem + 2 * TILE;          // dO, row-fragment swizzle
+  unsigned char* Dtr = smem + 3 * TILE;           // dO, transposing-read swizzle
+  float* Cs = (float*)(smem + 4 * TILE);          // [CP][CP] channel-table rows * scale
+  float* Ls = Cs + CP * CP;                       // [CP] log-sum-exp (+inf for padded queries)
+  float* Es = Ls + CP;                            // [CP] delta
+  float* Ts = Es + CP;                            // [CP] time-table entry for this tk * scale
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 31, hh = lane >> 5;
+  const int kt = wave % NCT, qt = wave / NCT;     // this wave's key tile and query tile
+  const int T_ = a.T, C_ = a.C, W = a.window, N = a.T * a.C;
+  const bool has_content = a.flags & MVPA_FLAG_CONTENT;
+  const bool has_time = a.flags & MVPA_FLAG_TIME_BIAS;
+  const bool has_chan = a.flags & MVPA_FLAG_CHAN_BIAS;
+  const int tk = blockIdx.x;                      // early key steps (most queries) first
+  const int b = blockIdx.y / a.Hkv, g = blockIdx.y % a.Hkv;
+  const int grp = a.H / a.Hkv;
+  const float sc2 = a.sm_scale * kLog2e;
+
+  const int ck = kt * 32 + ln;
+  bool key_ok = ck < C_;
+  if (key_ok && a.chan_valid) key_ok = a.chan_valid[(int64_t)b * C_ + ck] != 0;
+  const int64_t nk = (int64_t)tk * C_ + min(ck, C_ - 1);
+  const bf16_t* krow = (const bf16_t*)a.k + b * a.k_stride_b + g * a.k_stride_h + nk * a.k_stride_n;
+  const bf16_t* vrow = (const bf16_t*)a.v + b * a.v_stride_b + g * a.v_stride_h + nk * a.v_stride_n;
+  const bf16_t* bu = (const bf16_t*)a.bias_u + g * DH;
+  bf16x8 Kf[KS], Vf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    Kf[ks] = as_frag(*(const u32x4*)(krow + ks * 16 + hh * 8));
+    Vf[ks] = as_frag(*(const u32x4*)(vrow + ks * 16 + hh * 8));
+  }
+
+  f32x16 dK[MT], dV[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { dK[mt][i] = 0.f; dV[mt][i] = 0.f; }
+
+  int r_lane[KS], t_lane[MT];
+  {
+    const int e = (ln & 15) >> 2, aa = ln & 3, grp16 = ln >> 4;
+    const int row0 = 4 * hh + e;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      r_lane[ks] = (qt * 32 + ln) * ROWB + (((2 * ks + hh) ^ swz_row(ln)) << 4);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      t_lane[mt] = (qt * 32 + row0) * ROWB + (((4 * mt + 2 * grp16 + (aa >> 1)) ^ swz_tr(row0)) << 4) + ((aa & 1) << 3);
+  }
+  auto tr_frag = [&](const unsigned char* tile_p, int s, int mt) -> bf16x8 {
+    const unsigned char* p = tile_p + t_lane[mt] + 16 * s * ROWB;
+    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((BWD_LDS_PTR(bf16x4))p);
+    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((BWD_LDS_PTR(bf16x4))(p + 8 * ROWB));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+
+  constexpr int CHUNKS = CP * 8;
+  for (int hq = 0; hq < grp; ++hq) {
+    const int h = g * grp + hq;
+    const bf16_t* qbase = (const bf16_t*)a.q + b * a.q_stride_b + h * a.q_stride_h;
+    const bf16_t* dbase = (const bf16_t*)a.d_o + b * a.do_stride_b + h * a.do_stride_h;
+    const int64_t rbase = ((int64_t)b * a.H + h) * N;
+    for (int tq = tk; tq < T_; ++tq) {
+      const bool near = has_content && (W <= 0 || tq - tk <= W || tq == T_ - 1);
+      const int jt = time_row(tq, tk, T_);
+      __syncthreads();                            // everyone is done with the previous stage
+      for (int c = tid; c < CHUNKS; c += NTHR) {
+        const int r = c >> 3, ch = c & 7;
+        const int64_t n = (int64_t)tq * C_ + min(r, C_ - 1);
+        const u32x4 qq = *(const u32x4*)(qbase + n * a.q_stride_n + ch * 8);
+        const u32x4 dd = *(const u32x4*)(dbase + n * a.do_stride_n + ch * 8);
+        const bf16x8 qu = qfrag(qq, bu + ch * 8, sc2);
+        union { bf16x8 f; u32x4 u; } cv;
+        cv.f = qu;
+        *(u32x4*)(Qrow + r * ROWB + ((ch ^ swz_row(r)) << 4)) = cv.u;
+        *(u32x4*)(Qtr + r * ROWB + ((ch ^ swz_tr(r)) << 4)) = cv.u;
+        *(u32x4*)(Drow + r * ROWB + ((ch ^ swz_row(r)) << 4)) = dd;
+        *(u32x4*)(Dtr + r * ROWB + ((ch ^ swz_tr(r)) << 4)) = dd;
+      }
+      for (int idx = tid; idx < C_ * C_; idx += NTHR) {
+        const int r = idx / C_, i = idx - r * C_;
+        Cs[r * CP + i] = has_chan ? a.ws_chan[(rbase + (int64_t)tq * C_ + r) * C_ + i] * sc2 : 0.f;
+      }
+      for (int r = tid; r < CP; r += NTHR) {
+        const bool ok = r < C_;
+        const int64_t rw = rbase + (int64_t)tq * C_ + min(r, C_ - 1);
+        Ls[r] = ok ? a.lse[rw] : INFINITY;        // padded queries: exp2(-inf) = 0
+        Es[r] = ok ? a.ws_delta[rw] : 0.f;
+        Ts[r] = (ok && has_time) ? a.ws_time[rw * T_ + jt] * sc2 : 0.f;
+      }
+      __syncthreads();
+
+      // ---- S[q][key] and dP[q][key] for this wave's (query tile, key tile)
+      f32x16 S, dP;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) { S[i] = 0.f; dP[i] = 0.f; }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (near) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Qrow + r_lane[ks]), Kf[ks], S, 0, 0, 0);
+        dP = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Drow + r_lane[ks]), Vf[ks], dP, 0, 0, 0);
+      }
+      f32x16 dS;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int r = qt * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);     // query channel of this row
+        const int dist = r > ck ? r - ck : ck - r;
+        const int col = min(max(C_ - 1 - dist, 0), CP - 1);
+        const float s = S[i] + Cs[r * CP + col] + Ts[r] - Ls[r];
+        const float p = (key_ok && r < C_) ? __builtin_amdgcn_exp2f(s) : 0.f;   // padded rows/keys
+        S[i] = p;
+        dS[i] = p * (dP[i] - Es[r]) * (1.f / kLog2e);
+      }
+      // ---- dv^T[d][key] += dO^T[d][q] P[q][key];  dk^T[d][key] += (q+u)^T[d][q] dS[q][key]
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const bf16x8 pf = pack8(S, 8 * s);
+        const bf16x8 sf = pack8(dS, 8 * s);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          dV[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Dtr, s, mt), pf, dV[mt], 0, 0, 0);
+          if (near) dK[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Qtr, s, mt), sf, dK[mt], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // ---- reduce the query tiles' partial sums (waves with the same key tile) and store
+  __syncthreads();
+  float* red = (float*)smem;                      // [NCT key tiles][2][64 d][32 keys] fp32
+  if (NCT > 1) {
+    for (int round = 1; round < NCT; ++round) {
+      if (qt == round) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int d = mt * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
+            red[((kt * 2 + 0) * 64 + d) * 32 + ln] = dK[mt][i];
+            red[((kt * 2 + 1) * 64 + d) * 32 + ln] = dV[mt][i];
+          }
+      }
+      __syncthreads();
+      if (qt == 0) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int d = mt * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
+            dK[mt][i] += red[((kt * 2 + 0) * 64 + d) * 32 + ln];
+            dV[mt][i] += red[((kt * 2 + 1) * 64 + d) * 32 + ln];
+          }
+      }
+      __syncthreads();
+    }
+  }
+  if (qt == 0 && ck < C_) {
+    const int64_t o = ((((int64_t)b * a.Hkv + g) * N) + (int64_t)tk * C_ + ck) * DH;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int a4 = 0; a4 < 4; ++a4) {
+        const int d = mt * 32 + a4 * 8 + hh * 4;
+        *(float4*)(a.dk + o + d) = make_float4(dK[mt][a4 * 4], dK[mt][a4 * 4 + 1], dK[mt][a4 * 4 + 2], dK[mt][a4 * 4 + 3]);
+        *(float4*)(a.dv + o + d) = make_float4(dV[mt][a4 * 4], dV[mt][a4 * 4 + 1], dV[mt][a4 * 4 + 2], dV[mt][a4 * 4 + 3]);
+      }
+  }
+}
+
+}  // namespace bwdq
+}  // namespace mvpa
+
+int mvpa_launch_bwd_key_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
+  using namespace mvpa::bwdq;
+  const int nct = a->C <= 32 ? 1 : 2;
+  const int cp = nct * 32;
+  size_t lds = (size_t)4 * cp * ROWB + (size_t)(cp * cp + 3 * cp) * sizeof(float);
+  const size_t red = (size_t)nct * 2 * 64 * 32 * sizeof(float);
+  if (red > lds) lds = red;
+  dim3 grid((unsigned)a->T, (unsigned)(a->B * a->Hkv));
+  if (nct == 1) {
+    auto kern = mvpa_bwd_key_mfma_kernel<1>;
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(kern, grid, dim3(64), lds, stream, *a);
+  } else {
+    auto kern = mvpa_bwd_key_mfma_kernel<2>;
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, *a);
   }
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
