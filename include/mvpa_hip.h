@@ -120,8 +120,8 @@ int mvpa_forward(const mvpa_fwd_args* args, void* stream);
 /* ---- backward ------------------------------------------------------------------------------
  * Argument block of mvpa_backward: the boundary of FlashMVPA.backward
  * (attentions/attn.py:1140-1302).  Inputs as in mvpa_fwd_args plus the forward output o, the
- * incoming gradient d_o and the forward's base-2 log-sum-exp.  Every gradient and workspace
- * buffer is fp32, contiguous and caller-allocated; none needs to be cleared. */
+ * incoming gradient d_o and the forward's base-2 log-sum-exp.  Every gradient buffer and every
+ * workspace but ws_qu is fp32; all are contiguous and caller-allocated; none needs to be cleared. */
 typedef struct mvpa_bwd_args {
   uint32_t struct_size;      /* = sizeof(mvpa_bwd_args)                                       */
   int32_t dtype;             /* dtype of q, k, v, o, d_o, biases and tables                   */
@@ -153,9 +153,12 @@ typedef struct mvpa_bwd_args {
   float* dv;                 /* [B,Hkv,N,Dh]                                                  */
   float* dbias_time;         /* [B,H,N,T] gradient of the table (q+v).k_time^T, by table column */
   float* dbias_chan;         /* [B,H,N,C] gradient of the table (q+z).k_chan^T, by table column */
-  float* ws_delta;           /* workspace [B*H,N]                                             */
+  float* ws_delta;           /* workspace [B*H,N]      (contents after the call unspecified)  */
   float* ws_time;            /* workspace [B,H,N,T]                                           */
   float* ws_chan;            /* workspace [B,H,N,C]                                           */
+  void* ws_qu;               /* nullable workspace [B,H,N,Dh] of `dtype`, 16-byte aligned; the
+                                matrix-core kernels (bf16, Dh = 64, even C <= 64, no key_bias)
+                                run only when it is given                                     */
 } mvpa_bwd_args;
 
 /* Backward of the fused forward; replaces FlashMVPA.backward and its _bwd_kernel

@@ -11,11 +11,15 @@
 //     dS^T = P^T o (dP^T - delta) * scale,          delta = dO . O
 //     dq^T += K^T dS^T                     (inside the window)
 //     dbias_time[q, tk] = sum_ck dS,       dbias_chan[q, |cq-ck|] += dS.
-// Outputs and workspace are those of mvpa_backward (include/mvpa_hip.h): the content share of dq,
-// the two bias-table gradients, delta, and the forward bias tables in natural units for the key
-// pass.  K and V tiles are staged through LDS once per key step for the whole workgroup, K in two
-// copies (row fragments for K Q^T, transposed fragments for K^T dS^T).
+// Outputs are those of mvpa_backward (include/mvpa_hip.h): the content share of dq and the two
+// bias-table gradients.  For the key pass the workspace receives, in base-2 score units, delta,
+// the channel-table rows, (time bias - L) laid out [b,h,tq,tk,cq] and (q+u) * scale in bf16.
+// K and V tiles come through a ring of LDS stages filled by direct-to-LDS loads two key steps
+// ahead, K in two copies (row fragments for K Q^T, transposed fragments for K^T dS^T); far key
+// steps fetch V only.
 #include "mvpa_common.h"
+
+#include <type_traits>
 
 namespace mvpa {
 namespace bwdq {
@@ -28,11 +32,47 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 #define BWD_LDS_PTR(T) __attribute__((address_space(3))) T*
 
 constexpr int DH = 64, KS = 4, MT = 2, ROWB = 128, NW = 4;
+constexpr int QSTAGES = 3, KSTAGES = 3;          // ring depth of the query / key pass
 
 __device__ inline void wave_sync_lds() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// workgroup barrier that orders LDS traffic only (global loads of the ring stay in flight)
+__device__ inline void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// direct-to-LDS loads: lane L's 16 (4) bytes land at lds_base + 16 L (4 L).  Inline assembly so
+// that the compiler does not drain the ring in front of later LDS reads; completion is awaited
+// with wait_vmcnt() before the barrier that publishes a stage.
+__device__ inline void dma16(const void* gptr, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :: "v"(gptr), "s"(lds_base) : "memory", "m0");
+}
+__device__ inline void dma4(const void* gptr, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+               :: "v"(gptr), "s"(lds_base) : "memory", "m0");
+}
+
+template <int N>
+__device__ inline void wait_vmcnt_imm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// wait until at most n (0..6) of this wave's vector-memory operations are outstanding
+__device__ inline void wait_vmcnt(int n) {
+  switch (n) {
+    case 0: wait_vmcnt_imm<0>(); break;
+    case 1: wait_vmcnt_imm<1>(); break;
+    case 2: wait_vmcnt_imm<2>(); break;
+    case 3: wait_vmcnt_imm<3>(); break;
+    case 4: wait_vmcnt_imm<4>(); break;
+    case 5: wait_vmcnt_imm<5>(); break;
+    default: wait_vmcnt_imm<6>(); break;
+  }
 }
 
 __device__ inline bf16x8 as_frag(u32x4 v) {
@@ -70,11 +110,10 @@ __device__ inline int swz_tr(int row) { return ((row >> 1) & 1) << 2; }
 template <int NCT>
 __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_args a) {
   constexpr int CP = NCT * 32, TQW = NW / NCT, TILE = CP * ROWB;
+  constexpr int STAGES = QSTAGES, STAGE_BYTES = 3 * TILE;   // stage: V | K | K (transposing)
+  constexpr int LPW = CP / 8 / NW;                // 1 KiB wave loads per wave and tile copy
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  unsigned char* Krow = smem;                     // K tile, row-fragment swizzle
-  unsigned char* Ktr = smem + TILE;               // K tile, transposing-read swizzle
-  unsigned char* Vrow = smem + 2 * TILE;          // V tile, row-fragment swizzle
-  float* wave_base = (float*)(smem + 3 * TILE);
+  float* wave_base = (float*)(smem + STAGES * STAGE_BYTES);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -88,8 +127,21 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
   const bool has_time = a.flags & MVPA_FLAG_TIME_BIAS;
   const bool has_chan = a.flags & MVPA_FLAG_CHAN_BIAS;
   const int nt = (T_ + TQW - 1) / TQW;
-  const int tile = nt - 1 - (int)blockIdx.x;      // long tiles first
-  const int bh = blockIdx.y;
+  // blocks go round-robin over the 8 XCDs: keep the tiles of one (b,h) on one XCD (they walk the
+  // same K and V in step, so its L2 serves all but the first), long tiles first
+  const int nbh = a.B * a.H;
+  int bh, tile;
+  {
+    const int L = blockIdx.x;
+    if ((nbh & 7) == 0) {
+      const int s = L >> 3;
+      bh = (L & 7) + 8 * (s / nt);
+      tile = nt - 1 - s % nt;
+    } else {
+      bh = L / nt;
+      tile = nt - 1 - L % nt;
+    }
+  }
   const int b = bh / a.H, h = bh % a.H;
   const int g = h / (a.H / a.Hkv);
   const int tq0 = tile * TQW;
@@ -113,7 +165,38 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
   const bf16_t* bz = (const bf16_t*)a.bias_z + g * DH;
   const uint8_t* valid = a.chan_valid ? a.chan_valid + (int64_t)b * C_ : nullptr;
   const float sc2 = a.sm_scale * kLog2e;          // scores live in the base-2 domain
-  const float inv_sc2 = 1.f / sc2;
+
+  // ---- the ring: per-wave source offsets (the swizzle is applied on the source side), prologue
+  int k_off_r[LPW], k_off_t[LPW], v_off[LPW];
+#pragma unroll
+  for (int i = 0; i < LPW; ++i) {
+    const int pc = (wave + NW * i) * 64 + lane;
+    const int r = pc >> 3, phys = pc & 7;
+    const int rc = min(r, C_ - 1);
+    k_off_r[i] = rc * (int)a.k_stride_n + ((phys ^ swz_row(r)) << 3);
+    k_off_t[i] = rc * (int)a.k_stride_n + ((phys ^ swz_tr(r)) << 3);
+    v_off[i] = rc * (int)a.v_stride_n + ((phys ^ swz_row(r)) << 3);
+  }
+  // first key step whose K is needed: the band of the earliest query step of the workgroup
+  const int tk_near = !has_content ? tq_hi + 1 : (W <= 0 || tq_hi == T_ - 1) ? 0 : max(0, tq0 - W);
+  const uint32_t ring_lds = (uint32_t)(uintptr_t)(BWD_LDS_PTR(unsigned char))smem;
+  auto issue_tile = [&](int tk, int stage_idx, bool with_k) {
+    const uint32_t st = ring_lds + stage_idx * STAGE_BYTES;
+    const bf16_t* vsrc = vbase + (int64_t)tk * C_ * a.v_stride_n;
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) dma16(vsrc + v_off[i], st + (wave + NW * i) * 1024);
+    if (with_k) {
+      const bf16_t* ksrc = kbase + (int64_t)tk * C_ * a.k_stride_n;
+#pragma unroll
+      for (int i = 0; i < LPW; ++i) {
+        dma16(ksrc + k_off_r[i], st + TILE + (wave + NW * i) * 1024);
+        dma16(ksrc + k_off_t[i], st + 2 * TILE + (wave + NW * i) * 1024);
+      }
+    }
+  };
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s)
+    if (s <= tq_hi) issue_tile(s, s, s >= tk_near);
 
   // ---- set-up: operand fragments, delta, channel-bias tile
   bf16x8 Qu[KS], Qv[KS], dOf[KS];
@@ -180,10 +263,16 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
         const bool kv = (kbits[t] >> ((i >> 2) * 8 + (i & 3))) & 1u;
         Bc[t][i] = kv ? val : -INFINITY;
       }
-    // forward tables for the key pass, natural units; rows of dbias_time that no key step reaches
+    // for the key pass: delta, channel-table row (base-2 units), (q+u) * scale; and the rows of
+    // dbias_time that no key step reaches
+    if (qok) {
+      bf16_t* wq = (bf16_t*)a.ws_qu + row * DH;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) *(bf16x8*)(wq + ks * 16 + hh * 8) = Qu[ks];
+    }
     if (qok && hh == 0) {
       a.ws_delta[row] = delta;
-      for (int i = 0; i < C_; ++i) a.ws_chan[row * C_ + i] = scr[i * 32 + ln] * inv_sc2;
+      for (int i = 0; i < C_; ++i) a.ws_chan[row * C_ + i] = scr[i * 32 + ln];
       for (int j = 0; j < T_ - 1 - tq; ++j) a.dbias_time[row * T_ + j] = 0.f;
     }
     wave_sync_lds();
@@ -226,28 +315,35 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
         if (tkk > tq) break;
         const int j = time_row(tq, tkk, T_);
         a.dbias_time[row * T_ + j] = Gtb[jj * 32 + ln];
-        a.ws_time[row * T_ + j] = Stb[jj * 32 + ln] * inv_sc2;
+        a.ws_time[(((int64_t)bh * T_ + tq) * T_ + tkk) * C_ + cq] = Stb[jj * 32 + ln] - lse;
       }
     }
   };
 
-  // per-thread shares of the cooperative tile load: 16-byte chunk c of row r, twice per tile
-  constexpr int CHUNKS = CP * 8;                  // 16-byte chunks per tile
-  for (int tk = 0; tk <= tq_hi; ++tk) {
-    __syncthreads();                              // everyone is done with the previous tiles
-    for (int c = tid; c < CHUNKS; c += NW * 64) {
-      const int r = c >> 3, ch = c & 7;
-      const int rc = min(r, C_ - 1);
-      const int64_t n = (int64_t)tk * C_ + rc;
-      const u32x4 kk = *(const u32x4*)(kbase + n * a.k_stride_n + ch * 8);
-      const u32x4 vv = *(const u32x4*)(vbase + n * a.v_stride_n + ch * 8);
-      *(u32x4*)(Krow + r * ROWB + ((ch ^ swz_row(r)) << 4)) = kk;
-      *(u32x4*)(Ktr + r * ROWB + ((ch ^ swz_tr(r)) << 4)) = kk;
-      *(u32x4*)(Vrow + r * ROWB + ((ch ^ swz_row(r)) << 4)) = vv;
+  int stage = 0;
+  // advances the ring to key step tk and returns the stage that holds its tiles
+  auto ring_step = [&](int tk) -> const unsigned char* {
+    // tile tk has landed once at most the loads of the younger tiles are in flight (a count that
+    // is too small only waits longer)
+    if (tk + 1 >= tk_near && tk + STAGES - 2 <= tq_hi) {
+      wait_vmcnt_imm<(STAGES - 2) * 3 * LPW>();
+    } else {
+      int younger = 0;
+#pragma unroll
+      for (int d = 1; d <= STAGES - 2; ++d)
+        if (tk + d <= tq_hi) younger += LPW * (tk + d >= tk_near ? 3 : 1);
+      wait_vmcnt(younger);
     }
-    __syncthreads();
-    if (!active || tk > tq) continue;             // the workgroup's other time step runs longer
+    lds_barrier();            // tile tk visible to all; everyone is done with tile tk-1's stage
+    if (tk + STAGES - 1 <= tq_hi)
+      issue_tile(tk + STAGES - 1, stage == 0 ? STAGES - 1 : stage - 1, tk + STAGES - 1 >= tk_near);
+    const unsigned char* Vrow = smem + stage * STAGE_BYTES;
+    stage = stage + 1 == STAGES ? 0 : stage + 1;
+    return Vrow;
+  };
 
+  // every 32 key steps: write the finished slab, form the next slab of time-bias scores
+  auto time_slab = [&](int tk) {
     if ((tk & 31) == 0) {
       if (tk > 0) {
         wave_sync_lds();
@@ -269,9 +365,16 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
       for (int i = 0; i < 16; ++i) Stb[((i >> 2) * 8 + hh * 4 + (i & 3)) * 32 + ln] = stc[i];
       wave_sync_lds();
     }
+  };
 
+  // one key step; NEAR = inside the content window.  The far and the near steps of a wave run in
+  // two loops of their own: one loop with a run-time test costs copies of whole accumulator
+  // tiles wherever the two paths join.
+  auto key_step = [&](auto near_c, const unsigned char* Vrow, int tk) {
+    constexpr bool NEAR = decltype(near_c)::value;
+    const unsigned char* Krow = Vrow + TILE;
+    const unsigned char* Ktr = Vrow + 2 * TILE;
     const float st = Stb[(tk & 31) * 32 + ln];
-    const bool near = has_content && (W <= 0 || tq - tk <= W || tq == T_ - 1);
     f32x16 S[NCT], dP[NCT];
 #pragma unroll
     for (int t = 0; t < NCT; ++t) {
@@ -284,7 +387,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
 #pragma unroll
       for (int t = 0; t < NCT; ++t) {
         const int off = r_lane[ks] + t * 32 * ROWB;
-        if (near) S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Krow + off), Qu[ks], S[t], 0, 0, 0);
+        if (NEAR) S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Krow + off), Qu[ks], S[t], 0, 0, 0);
         dP[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Vrow + off), dOf[ks], dP[t], 0, 0, 0);
       }
     const float off2 = st - lse;
@@ -301,7 +404,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
       }
     gt = xhalf_sum(gt);
     if (hh == 0) Gtb[(tk & 31) * 32 + ln] = gt;
-    if (near) {
+    if (NEAR) {
 #pragma unroll
       for (int t = 0; t < NCT; ++t)
 #pragma unroll
@@ -311,6 +414,23 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
           for (int mt = 0; mt < MT; ++mt)
             dq[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Ktr, t, s, mt), dsf, dq[mt], 0, 0, 0);
         }
+    }
+  };
+
+  // far steps first (none for the last time step, whose queries keep the content term everywhere),
+  // then the steps inside the window; waves that are done keep the ring and the barriers going
+  const int far_end = !active ? 0 : !has_content ? tq + 1 : (W <= 0 || tq == T_ - 1) ? 0 : max(0, tq - W);
+  int tk = 0;
+  for (; tk < far_end; ++tk) {
+    const unsigned char* Vrow = ring_step(tk);
+    time_slab(tk);
+    key_step(std::false_type{}, Vrow, tk);
+  }
+  for (; tk <= tq_hi; ++tk) {
+    const unsigned char* Vrow = ring_step(tk);
+    if (active && tk <= tq) {
+      time_slab(tk);
+      key_step(std::true_type{}, Vrow, tk);
     }
   }
 
@@ -359,11 +479,13 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
 // 1 if the MFMA query pass can serve these (already validated) arguments
 int mvpa_bwd_query_mfma_supported(const mvpa_bwd_args* a) {
   if (a->dtype != MVPA_BF16 || a->Dh != 64 || a->C > 64) return 0;
-  if (!(a->flags & MVPA_FLAG_CAUSAL) || a->key_bias) return 0;
+  if (!(a->flags & MVPA_FLAG_CAUSAL) || a->key_bias || !a->ws_qu) return 0;
+  if (a->C & 1) return 0;      // 16-byte direct-to-LDS loads of the [C][C] channel-table blocks
   const uintptr_t p = (uintptr_t)a->q | (uintptr_t)a->k | (uintptr_t)a->v | (uintptr_t)a->o |
                       (uintptr_t)a->d_o | (uintptr_t)a->bias_u | (uintptr_t)a->bias_v |
                       (uintptr_t)a->bias_z | (uintptr_t)a->k_time | (uintptr_t)a->k_chan |
-                      (uintptr_t)a->dq;
+                      (uintptr_t)a->dq | (uintptr_t)a->ws_qu | (uintptr_t)a->ws_chan |
+                      (uintptr_t)a->dk | (uintptr_t)a->dv;
   const int64_t s = a->q_stride_b | a->q_stride_h | a->q_stride_n | a->k_stride_b | a->k_stride_h |
                     a->k_stride_n | a->v_stride_b | a->v_stride_h | a->v_stride_n |
                     a->o_stride_b | a->o_stride_h | a->o_stride_n | a->do_stride_b |
@@ -378,8 +500,8 @@ int mvpa_launch_bwd_query_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
   const int tqw = NW / nct;
   const int nt = (a->T + tqw - 1) / tqw;
   const int cp = nct * 32;
-  const size_t lds = (size_t)3 * cp * ROWB + (size_t)NW * (2 * 1024 + cp * 32) * sizeof(float);
-  dim3 grid((unsigned)nt, (unsigned)(a->B * a->H));
+  const size_t lds = (size_t)QSTAGES * 3 * cp * ROWB + (size_t)NW * (2 * 1024 + cp * 32) * sizeof(float);
+  dim3 grid((unsigned)(nt * a->B * a->H));
   if (nct == 1) {
     auto kern = mvpa_bwd_query_mfma_kernel<1>;
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -393,60 +515,112 @@ int mvpa_launch_bwd_query_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
 }
 
 // ==========================================================================================
-// The KEY pass: dk, dv.  One workgroup per key time step tk and kv head; a wave owns 32 key
-// channels (its K and V rows stay in registers as MFMA B operands) and one of the NCT query-channel
-// tiles; it walks the query time steps tq >= tk of every query head of the group.  Products are
-// formed NON-transposed here, S[q][key] = (q+u) K^T, so that a lane owns one key and the
-// contraction index of dv^T = dO^T P and dk^T = (q+u)^T dS is the register index:
-//     S   = (q+u) K^T (inside the window) + chan[q][C-1-|cq-ck|] + time[q][tk]
-//     P   = exp2(S - L[q]),  dP = dO V^T,  dS = P o (dP - delta[q])
+// The KEY pass: dk, dv.  A workgroup owns NW / NCT consecutive key time steps of one kv head; a
+// wave owns 32 key channels of one of them (its K and V rows stay in registers as MFMA B
+// operands) and walks every query time step tq >= tk of every query head of the group, both
+// query-channel tiles in turn.  Products are formed NON-transposed here, S[q][key] = (q+u) K^T,
+// so that a lane owns one key and the contraction index of dv^T = dO^T P and dk^T = (q+u)^T dS
+// is the register index:
+//     S   = (q+u) K^T (inside the window) + chan[q][C-1-|cq-ck|] + (time[q][tk] - L[q])
+//     P   = exp2(S),  dP = dO V^T,  dS = P o (dP - delta[q])
 //     dv^T[d][key] += dO^T[d][q] P[q][key],   dk^T[d][key] += (q+u)^T[d][q] dS[q][key]
-// The per-query bias tables, L and delta come from the query pass (workspace, natural units).
-// Per (head, tq) the workgroup stages (q+u) * scale and dO (each in the two swizzles), the
-// channel-table rows and the per-query scalars in LDS.
+// Everything per query comes from the query pass's workspace in the units used here.  Per
+// (head, tq) one ring stage holds (q+u) * scale and dO (each in the two swizzles), the
+// channel-table rows and the per-query scalars, fetched by direct-to-LDS loads two steps ahead.
+// The query steps are walked from the last one down, and the workgroups of one (b, kv head) sit
+// on one XCD: they then read the same stage data at about the same time and share it in L2.
 // ==========================================================================================
 namespace mvpa {
 namespace bwdq {
 
 template <int NCT>
-__global__ __launch_bounds__(NCT * NCT * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_args a) {
-  constexpr int CP = NCT * 32, TILE = CP * ROWB, NWK = NCT * NCT, NTHR = NWK * 64;
+__global__ __launch_bounds__(NW * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_args a) {
+  constexpr int CP = NCT * 32, KT = NW / NCT, TILE = CP * ROWB;
+  constexpr int CS_BYTES = CP * CP * 4, SC_BYTES = (KT + 1) * 256;
+  constexpr int STAGES = KSTAGES, STAGE_BYTES = 4 * TILE + CS_BYTES + SC_BYTES;
+  constexpr int LPW = CP / 8 / NW, CS_LPW = CS_BYTES / 1024 / NW;
+  constexpr int LPS = 4 * LPW + CS_LPW + 2;       // direct-to-LDS loads per wave and step
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  unsigned char* Qrow = smem;                     // (q+u)*scale, row-fragment swizzle
-  unsigned char* Qtr = smem + TILE;               // same, transposing-read swizzle
-  unsigned char* Drow = smem + 2 * TILE;          // dO, row-fragment swizzle
-  unsigned char* Dtr = smem + 3 * TILE;           // dO, transposing-read swizzle
-  float* Cs = (float*)(smem + 4 * TILE);          // [CP][CP] channel-table rows * scale
-  float* Ls = Cs + CP * CP;                       // [CP] log-sum-exp (+inf for padded queries)
-  float* Es = Ls + CP;                            // [CP] delta
-  float* Ts = Es + CP;                            // [CP] time-table entry for this tk * scale
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 31, hh = lane >> 5;
-  const int kt = wave % NCT, qt = wave / NCT;     // this wave's key tile and query tile
+  const int ktw = wave / NCT, kt = wave % NCT;    // this wave's key step and key-channel tile
   const int T_ = a.T, C_ = a.C, W = a.window, N = a.T * a.C;
   const bool has_content = a.flags & MVPA_FLAG_CONTENT;
-  const bool has_time = a.flags & MVPA_FLAG_TIME_BIAS;
-  const bool has_chan = a.flags & MVPA_FLAG_CHAN_BIAS;
-  const int tk = blockIdx.x;                      // early key steps (most queries) first
-  const int b = blockIdx.y / a.Hkv, g = blockIdx.y % a.Hkv;
+  const int nbg = a.B * a.Hkv, ntk = (T_ + KT - 1) / KT;
+  int bg, tile;
+  {
+    const int L = blockIdx.x;
+    if ((nbg & 7) == 0) {
+      const int s = L >> 3;
+      bg = (L & 7) + 8 * (s / ntk);
+      tile = s % ntk;                             // early key steps (most queries) first
+    } else {
+      bg = L / ntk;
+      tile = L % ntk;
+    }
+  }
+  const int b = bg / a.Hkv, g = bg % a.Hkv;
   const int grp = a.H / a.Hkv;
-  const float sc2 = a.sm_scale * kLog2e;
+  const int tk0 = tile * KT;
+  const int tk = tk0 + ktw;
+  const bool wave_on = tk < T_;
+  const int tkc = min(tk, T_ - 1);
 
   const int ck = kt * 32 + ln;
   bool key_ok = ck < C_;
   if (key_ok && a.chan_valid) key_ok = a.chan_valid[(int64_t)b * C_ + ck] != 0;
-  const int64_t nk = (int64_t)tk * C_ + min(ck, C_ - 1);
+  const int64_t nk = (int64_t)tkc * C_ + min(ck, C_ - 1);
   const bf16_t* krow = (const bf16_t*)a.k + b * a.k_stride_b + g * a.k_stride_h + nk * a.k_stride_n;
   const bf16_t* vrow = (const bf16_t*)a.v + b * a.v_stride_b + g * a.v_stride_h + nk * a.v_stride_n;
-  const bf16_t* bu = (const bf16_t*)a.bias_u + g * DH;
   bf16x8 Kf[KS], Vf[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     Kf[ks] = as_frag(*(const u32x4*)(krow + ks * 16 + hh * 8));
     Vf[ks] = as_frag(*(const u32x4*)(vrow + ks * 16 + hh * 8));
   }
+
+  // ---- the ring: per-wave source offsets (swizzles applied on the source side)
+  int q_off_r[LPW], q_off_t[LPW], d_off_r[LPW], d_off_t[LPW], cs_off[CS_LPW];
+#pragma unroll
+  for (int i = 0; i < LPW; ++i) {
+    const int pc = (wave + NW * i) * 64 + lane;
+    const int r = pc >> 3, phys = pc & 7;
+    const int rc = min(r, C_ - 1);
+    q_off_r[i] = rc * DH + ((phys ^ swz_row(r)) << 3);
+    q_off_t[i] = rc * DH + ((phys ^ swz_tr(r)) << 3);
+    d_off_r[i] = rc * (int)a.do_stride_n + ((phys ^ swz_row(r)) << 3);
+    d_off_t[i] = rc * (int)a.do_stride_n + ((phys ^ swz_tr(r)) << 3);
+  }
+#pragma unroll
+  for (int i = 0; i < CS_LPW; ++i)
+    cs_off[i] = min((wave + NW * i) * 64 + lane, C_ * C_ / 4 - 1) * 4;   // C is even here
+  const int sc_lane = min(lane, C_ - 1);
+  const uint32_t ring_lds = (uint32_t)(uintptr_t)(BWD_LDS_PTR(unsigned char))smem;
+  auto issue_step = [&](int hq, int tq, int stage_idx) {
+    const int h = g * grp + hq;
+    const int64_t bhq = (int64_t)b * a.H + h;
+    const int64_t r0 = bhq * N + (int64_t)tq * C_;          // first query row of the step
+    const uint32_t st = ring_lds + stage_idx * STAGE_BYTES;
+    const bf16_t* qsrc = (const bf16_t*)a.ws_qu + r0 * DH;
+    const bf16_t* dsrc = (const bf16_t*)a.d_o + b * a.do_stride_b + h * a.do_stride_h +
+                         (int64_t)tq * C_ * a.do_stride_n;
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+      const uint32_t dst = st + (wave + NW * i) * 1024;
+      dma16(qsrc + q_off_r[i], dst);
+      dma16(qsrc + q_off_t[i], dst + TILE);
+      dma16(dsrc + d_off_r[i], dst + 2 * TILE);
+      dma16(dsrc + d_off_t[i], dst + 3 * TILE);
+    }
+    const float* csrc = a.ws_chan + r0 * C_;
+#pragma unroll
+    for (int i = 0; i < CS_LPW; ++i) dma16(csrc + cs_off[i], st + 4 * TILE + (wave + NW * i) * 1024);
+    // per-query scalars: (time bias - L) for this wave's key step, and delta
+    dma4(a.ws_time + ((bhq * T_ + tq) * T_ + tkc) * C_ + sc_lane, st + 4 * TILE + CS_BYTES + ktw * 256);
+    dma4(a.ws_delta + r0 + sc_lane, st + 4 * TILE + CS_BYTES + KT * 256);
+  };
 
   f32x16 dK[MT], dV[MT];
 #pragma unroll
@@ -459,74 +633,81 @@ __global__ __launch_bounds__(NCT * NCT * 64) void mvpa_bwd_key_mfma_kernel(mvpa_
     const int e = (ln & 15) >> 2, aa = ln & 3, grp16 = ln >> 4;
     const int row0 = 4 * hh + e;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      r_lane[ks] = (qt * 32 + ln) * ROWB + (((2 * ks + hh) ^ swz_row(ln)) << 4);
+    for (int ks = 0; ks < KS; ++ks) r_lane[ks] = ln * ROWB + (((2 * ks + hh) ^ swz_row(ln)) << 4);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
-      t_lane[mt] = (qt * 32 + row0) * ROWB + (((4 * mt + 2 * grp16 + (aa >> 1)) ^ swz_tr(row0)) << 4) + ((aa & 1) << 3);
+      t_lane[mt] = row0 * ROWB + (((4 * mt + 2 * grp16 + (aa >> 1)) ^ swz_tr(row0)) << 4) + ((aa & 1) << 3);
   }
-  auto tr_frag = [&](const unsigned char* tile_p, int s, int mt) -> bf16x8 {
-    const unsigned char* p = tile_p + t_lane[mt] + 16 * s * ROWB;
+  auto tr_frag = [&](const unsigned char* tile_p, int qt, int s, int mt) -> bf16x8 {
+    const unsigned char* p = tile_p + t_lane[mt] + (32 * qt + 16 * s) * ROWB;
     const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((BWD_LDS_PTR(bf16x4))p);
     const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((BWD_LDS_PTR(bf16x4))(p + 8 * ROWB));
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
 
-  constexpr int CHUNKS = CP * 8;
-  for (int hq = 0; hq < grp; ++hq) {
-    const int h = g * grp + hq;
-    const bf16_t* qbase = (const bf16_t*)a.q + b * a.q_stride_b + h * a.q_stride_h;
-    const bf16_t* dbase = (const bf16_t*)a.d_o + b * a.do_stride_b + h * a.do_stride_h;
-    const int64_t rbase = ((int64_t)b * a.H + h) * N;
-    for (int tq = tk; tq < T_; ++tq) {
-      const bool near = has_content && (W <= 0 || tq - tk <= W || tq == T_ - 1);
-      const int jt = time_row(tq, tk, T_);
-      __syncthreads();                            // everyone is done with the previous stage
-      for (int c = tid; c < CHUNKS; c += NTHR) {
-        const int r = c >> 3, ch = c & 7;
-        const int64_t n = (int64_t)tq * C_ + min(r, C_ - 1);
-        const u32x4 qq = *(const u32x4*)(qbase + n * a.q_stride_n + ch * 8);
-        const u32x4 dd = *(const u32x4*)(dbase + n * a.do_stride_n + ch * 8);
-        const bf16x8 qu = qfrag(qq, bu + ch * 8, sc2);
-        union { bf16x8 f; u32x4 u; } cv;
-        cv.f = qu;
-        *(u32x4*)(Qrow + r * ROWB + ((ch ^ swz_row(r)) << 4)) = cv.u;
-        *(u32x4*)(Qtr + r * ROWB + ((ch ^ swz_tr(r)) << 4)) = cv.u;
-        *(u32x4*)(Drow + r * ROWB + ((ch ^ swz_row(r)) << 4)) = dd;
-        *(u32x4*)(Dtr + r * ROWB + ((ch ^ swz_tr(r)) << 4)) = dd;
-      }
-      for (int idx = tid; idx < C_ * C_; idx += NTHR) {
-        const int r = idx / C_, i = idx - r * C_;
-        Cs[r * CP + i] = has_chan ? a.ws_chan[(rbase + (int64_t)tq * C_ + r) * C_ + i] * sc2 : 0.f;
-      }
-      for (int r = tid; r < CP; r += NTHR) {
-        const bool ok = r < C_;
-        const int64_t rw = rbase + (int64_t)tq * C_ + min(r, C_ - 1);
-        Ls[r] = ok ? a.lse[rw] : INFINITY;        // padded queries: exp2(-inf) = 0
-        Es[r] = ok ? a.ws_delta[rw] : 0.f;
-        Ts[r] = (ok && has_time) ? a.ws_time[rw * T_ + jt] * sc2 : 0.f;
-      }
-      __syncthreads();
+  // steps: query heads of the group, and for each the query steps T-1 .. tk0
+  const int span = T_ - tk0, nsteps = grp * span;
+  int ihq = 0, itq = T_ - 1;                      // the step the ring fetches next
+  auto next_issue = [&]() {
+    if (--itq < tk0) { itq = T_ - 1; ++ihq; }
+  };
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s)
+    if (s < nsteps) { issue_step(ihq, itq, s); next_issue(); }
 
-      // ---- S[q][key] and dP[q][key] for this wave's (query tile, key tile)
-      f32x16 S, dP;
+  int stage = 0, it = 0;
+  // advances the ring by one step and returns the stage that holds its data
+  auto ring_step = [&]() -> const unsigned char* {
+    if (it + STAGES - 2 < nsteps) wait_vmcnt_imm<(STAGES - 2) * LPS>();
+    else wait_vmcnt_imm<0>();
+    lds_barrier();            // this step's stage visible to all; the previous one is free
+    if (it + STAGES - 1 < nsteps) { issue_step(ihq, itq, stage == 0 ? STAGES - 1 : stage - 1); next_issue(); }
+    const unsigned char* base = smem + stage * STAGE_BYTES;
+    stage = stage + 1 == STAGES ? 0 : stage + 1;
+    ++it;
+    return base;
+  };
+
+  // one query step; NEAR = inside the content window (as in the query pass, the far and the near
+  // steps run in loops of their own)
+  auto query_step = [&](auto near_c, const unsigned char* Qrow, int tq_now) {
+    constexpr bool NEAR = decltype(near_c)::value;
+    // Qrow: (q+u)*scale, row-fragment swizzle
+    const unsigned char* Qtr = Qrow + TILE;                   // same, transposing-read swizzle
+    const unsigned char* Drow = Qrow + 2 * TILE;              // dO, row-fragment swizzle
+    const unsigned char* Dtr = Qrow + 3 * TILE;               // dO, transposing-read swizzle
+    const float* Cs = (const float*)(Qrow + 4 * TILE);        // [C][C] channel-table rows
+    const float* TL = (const float*)(Qrow + 4 * TILE + CS_BYTES) + ktw * 64;   // time bias - L
+    const float* De = (const float*)(Qrow + 4 * TILE + CS_BYTES) + KT * 64;    // delta
+    (void)tq_now;
+#pragma unroll
+    for (int qt = 0; qt < NCT; ++qt) {
+      // ---- S[q][key] and dP[q][key] for query-channel tile qt
+      f32x16 S, dP, dS;
 #pragma unroll
       for (int i = 0; i < 16; ++i) { S[i] = 0.f; dP[i] = 0.f; }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        if (near) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Qrow + r_lane[ks]), Kf[ks], S, 0, 0, 0);
-        dP = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Drow + r_lane[ks]), Vf[ks], dP, 0, 0, 0);
+        const int off = r_lane[ks] + qt * 32 * ROWB;
+        if (NEAR) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Qrow + off), Kf[ks], S, 0, 0, 0);
+        dP = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Drow + off), Vf[ks], dP, 0, 0, 0);
       }
-      f32x16 dS;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int r = qt * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);     // query channel of this row
-        const int dist = r > ck ? r - ck : ck - r;
-        const int col = min(max(C_ - 1 - dist, 0), CP - 1);
-        const float s = S[i] + Cs[r * CP + col] + Ts[r] - Ls[r];
-        const float p = (key_ok && r < C_) ? __builtin_amdgcn_exp2f(s) : 0.f;   // padded rows/keys
-        S[i] = p;
-        dS[i] = p * (dP[i] - Es[r]) * (1.f / kLog2e);
+      for (int a4 = 0; a4 < 4; ++a4) {
+        const int rb = qt * 32 + a4 * 8 + hh * 4;              // query channels rb .. rb+3
+        const float4 tl = *(const float4*)(TL + rb);
+        const float4 de = *(const float4*)(De + rb);
+        const float tls[4] = {tl.x, tl.y, tl.z, tl.w}, des[4] = {de.x, de.y, de.z, de.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int i = a4 * 4 + j, r = rb + j;
+          const int dist = r > ck ? r - ck : ck - r;
+          const int col = max(C_ - 1 - dist, 0);
+          const float s = S[i] + Cs[r * C_ + col] + tls[j];
+          const float p = (key_ok && r < C_) ? __builtin_amdgcn_exp2f(s) : 0.f;   // padded rows/keys
+          S[i] = p;
+          dS[i] = p * (dP[i] - des[j]) * (1.f / kLog2e);
+        }
       }
       // ---- dv^T[d][key] += dO^T[d][q] P[q][key];  dk^T[d][key] += (q+u)^T[d][q] dS[q][key]
 #pragma unroll
@@ -535,43 +716,36 @@ __global__ __launch_bounds__(NCT * NCT * 64) void mvpa_bwd_key_mfma_kernel(mvpa_
         const bf16x8 sf = pack8(dS, 8 * s);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          dV[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Dtr, s, mt), pf, dV[mt], 0, 0, 0);
-          if (near) dK[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Qtr, s, mt), sf, dK[mt], 0, 0, 0);
+          dV[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Dtr, qt, s, mt), pf, dV[mt], 0, 0, 0);
+          if (NEAR) dK[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Qtr, qt, s, mt), sf, dK[mt], 0, 0, 0);
         }
       }
     }
-  }
+  };
 
-  // ---- reduce the query tiles' partial sums (waves with the same key tile) and store
-  __syncthreads();
-  float* red = (float*)smem;                      // [NCT key tiles][2][64 d][32 keys] fp32
-  if (NCT > 1) {
-    for (int round = 1; round < NCT; ++round) {
-      if (qt == round) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int d = mt * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
-            red[((kt * 2 + 0) * 64 + d) * 32 + ln] = dK[mt][i];
-            red[((kt * 2 + 1) * 64 + d) * 32 + ln] = dV[mt][i];
-          }
-      }
-      __syncthreads();
-      if (qt == 0) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int d = mt * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
-            dK[mt][i] += red[((kt * 2 + 0) * 64 + d) * 32 + ln];
-            dV[mt][i] += red[((kt * 2 + 1) * 64 + d) * 32 + ln];
-          }
-      }
-      __syncthreads();
+  // this wave's steps of one head, walking down from tq = T-1: the last query step keeps the
+  // content term, then the steps beyond the window, then the window, then the steps before tk
+  int n_last = 0, n_far = 0, n_win = 0;
+  if (wave_on) {
+    const int live = T_ - tk;
+    if (!has_content) n_far = live;
+    else if (W <= 0) n_win = live;
+    else {
+      n_last = 1;
+      n_far = max(0, live - 2 - W);
+      n_win = live - 1 - n_far;
     }
   }
-  if (qt == 0 && ck < C_) {
+  const int n_idle = span - n_last - n_far - n_win;
+  for (int hq = 0; hq < grp; ++hq) {
+    int tq = T_ - 1;
+    for (int n = n_last; n > 0; --n, --tq) query_step(std::true_type{}, ring_step(), tq);
+    for (int n = n_far; n > 0; --n, --tq) query_step(std::false_type{}, ring_step(), tq);
+    for (int n = n_win; n > 0; --n, --tq) query_step(std::true_type{}, ring_step(), tq);
+    for (int n = n_idle; n > 0; --n) (void)ring_step();
+  }
+
+  if (wave_on && ck < C_) {
     const int64_t o = ((((int64_t)b * a.Hkv + g) * N) + (int64_t)tk * C_ + ck) * DH;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -590,19 +764,17 @@ __global__ __launch_bounds__(NCT * NCT * 64) void mvpa_bwd_key_mfma_kernel(mvpa_
 int mvpa_launch_bwd_key_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
   using namespace mvpa::bwdq;
   const int nct = a->C <= 32 ? 1 : 2;
-  const int cp = nct * 32;
-  size_t lds = (size_t)4 * cp * ROWB + (size_t)(cp * cp + 3 * cp) * sizeof(float);
-  const size_t red = (size_t)nct * 2 * 64 * 32 * sizeof(float);
-  if (red > lds) lds = red;
-  dim3 grid((unsigned)a->T, (unsigned)(a->B * a->Hkv));
+  const int cp = nct * 32, kt = NW / nct;
+  const size_t lds = (size_t)KSTAGES * (4 * cp * ROWB + cp * cp * 4 + (kt + 1) * 256);
+  dim3 grid((unsigned)(((a->T + kt - 1) / kt) * a->B * a->Hkv));
   if (nct == 1) {
     auto kern = mvpa_bwd_key_mfma_kernel<1>;
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(kern, grid, dim3(64), lds, stream, *a);
+    hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, *a);
   } else {
     auto kern = mvpa_bwd_key_mfma_kernel<2>;
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, *a);
+    hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, *a);
   }
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }

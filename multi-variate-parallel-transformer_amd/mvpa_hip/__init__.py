@@ -55,7 +55,7 @@ class MvpaBwdArgs(ctypes.Structure):
         + [(f"{t}_stride_{ax}", ctypes.c_int64) for t in ("q", "k", "v", "o", "do") for ax in "bhn"]
         + [(n, ctypes.c_void_p) for n in (
             "bias_u", "bias_v", "bias_z", "k_time", "k_chan", "chan_valid", "key_bias", "lse",
-            "dq", "dk", "dv", "dbias_time", "dbias_chan", "ws_delta", "ws_time", "ws_chan")]
+            "dq", "dk", "dv", "dbias_time", "dbias_chan", "ws_delta", "ws_time", "ws_chan", "ws_qu")]
     )
 
 
@@ -259,6 +259,7 @@ def mvpa_backward(q, k, v, o, d_o, lse, u, vb, z, k_time, k_chan, *,
     ws_delta = torch.empty((B, H, N), **f32)
     ws_time = torch.empty((B, H, N, T), **f32)
     ws_chan = torch.empty((B, H, N, C), **f32)
+    ws_qu = torch.empty((B, H, N, Dh), dtype=dt, device=q.device)
     a = MvpaBwdArgs()
     a.struct_size = ctypes.sizeof(MvpaBwdArgs)
     a.dtype = _dtype_code(dt)
@@ -281,6 +282,7 @@ def mvpa_backward(q, k, v, o, d_o, lse, u, vb, z, k_time, k_chan, *,
     a.dq, a.dk, a.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
     a.dbias_time, a.dbias_chan = dbt.data_ptr(), dbc.data_ptr()
     a.ws_delta, a.ws_time, a.ws_chan = ws_delta.data_ptr(), ws_time.data_ptr(), ws_chan.data_ptr()
+    a.ws_qu = ws_qu.data_ptr()
     _check(lib.mvpa_backward(ctypes.byref(a), _stream()))
     return dq, dk, dv, dbt, dbc
 
