@@ -26,6 +26,8 @@ namespace bwdq {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
@@ -94,11 +96,13 @@ __device__ inline bf16x8 qfrag(u32x4 raw, const bf16_t* __restrict__ bias, float
   return out;
 }
 
+// 8 floats to a bf16 fragment, two per conversion instruction
 __device__ inline bf16x8 pack8(const f32x16& v, int base) {
-  bf16x8 out;
+  union { bf16x8 f; bf16x2 q[4]; } out;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) out[i] = (__bf16)v[base + i];
-  return out;
+  for (int i = 0; i < 4; ++i)
+    out.q[i] = __builtin_convertvector(f32x2{v[base + 2 * i], v[base + 2 * i + 1]}, bf16x2);
+  return out.f;
 }
 
 __device__ inline float xhalf_sum(float x) { return x + __shfl_xor(x, 32); }
@@ -200,9 +204,26 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
 
   // ---- set-up: operand fragments, delta, channel-bias tile
   bf16x8 Qu[KS], Qv[KS], dOf[KS];
-  f32x16 Bc[NCT];
-  float delta = 0.f;
+  f32x16 Ec[NCT];            // exp2(channel bias - mc): the far steps' probabilities up to a scalar
+  float delta = 0.f, mc = -INFINITY, sumEc = 0.f;
   uint32_t kbits[NCT];
+  // channel-bias tile of this lane's query from the per-wave table in the scratch; -inf where
+  // the key channel is padding or invalid
+  auto gather_bc = [&](f32x16 (&Bc)[NCT]) {
+    const uint32_t cq4 = (uint32_t)(cq - 4 * hh + 4);
+    const int gbase = ((C_ - 1) * 32 + ln) * 4;
+    const unsigned char* scr_b = (const unsigned char*)scr;
+#pragma unroll
+    for (int t = 0; t < NCT; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const uint32_t ci4 = (uint32_t)(t * 32 + (i >> 2) * 8 + (i & 3) + 4);
+        const uint32_t dist = min(max(cq4, ci4) - min(cq4, ci4), (uint32_t)(C_ - 1));
+        const float val = *(const float*)(scr_b + (gbase - (int)(dist * 128u)));
+        const bool kv = (kbits[t] >> ((i >> 2) * 8 + (i & 3))) & 1u;
+        Bc[t][i] = kv ? val : -INFINITY;
+      }
+  };
   {
     f32x16 sct[NCT];
 #pragma unroll
@@ -250,32 +271,47 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
 #pragma unroll
     for (int t = 0; t < NCT; ++t) kbits[t] = (uint32_t)(kmask[t >> 1] >> ((t & 1) * 32 + 4 * hh));
     wave_sync_lds();
-    const uint32_t cq4 = (uint32_t)(cq - 4 * hh + 4);
-    const int gbase = ((C_ - 1) * 32 + ln) * 4;
-    const unsigned char* scr_b = (const unsigned char*)scr;
+    gather_bc(Ec);
+#pragma unroll
+    for (int t = 0; t < NCT; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mc = fmaxf(mc, Ec[t][i]);
+    mc = fmaxf(mc, __shfl_xor(mc, 32));
+    if (mc == -INFINITY) mc = 0.f;                // no valid key channel at all
 #pragma unroll
     for (int t = 0; t < NCT; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const uint32_t ci4 = (uint32_t)(t * 32 + (i >> 2) * 8 + (i & 3) + 4);
-        const uint32_t dist = min(max(cq4, ci4) - min(cq4, ci4), (uint32_t)(C_ - 1));
-        const float val = *(const float*)(scr_b + (gbase - (int)(dist * 128u)));
-        const bool kv = (kbits[t] >> ((i >> 2) * 8 + (i & 3))) & 1u;
-        Bc[t][i] = kv ? val : -INFINITY;
+        Ec[t][i] = __builtin_amdgcn_exp2f(Ec[t][i] - mc);
+        sumEc += Ec[t][i];
       }
-    // for the key pass: delta, channel-table row (base-2 units), (q+u) * scale; and the rows of
-    // dbias_time that no key step reaches
+    sumEc = xhalf_sum(sumEc);
+    // for the key pass: (q+u) * scale, delta, and the tile exp2(channel bias - mc) by
+    // [query][key channel]; and the rows of dbias_time that no key step reaches
     if (qok) {
       bf16_t* wq = (bf16_t*)a.ws_qu + row * DH;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) *(bf16x8*)(wq + ks * 16 + hh * 8) = Qu[ks];
+      float* wc = a.ws_chan + row * C_;
+#pragma unroll
+      for (int t = 0; t < NCT; ++t)
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) {
+          const int ci = t * 32 + a4 * 8 + hh * 4;
+          if ((C_ & 3) == 0) {
+            if (ci < C_)
+              *(float4*)(wc + ci) = make_float4(Ec[t][a4 * 4], Ec[t][a4 * 4 + 1], Ec[t][a4 * 4 + 2], Ec[t][a4 * 4 + 3]);
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (ci + j < C_) wc[ci + j] = Ec[t][a4 * 4 + j];
+          }
+        }
     }
     if (qok && hh == 0) {
       a.ws_delta[row] = delta;
-      for (int i = 0; i < C_; ++i) a.ws_chan[row * C_ + i] = scr[i * 32 + ln];
       for (int j = 0; j < T_ - 1 - tq; ++j) a.dbias_time[row * T_ + j] = 0.f;
     }
-    wave_sync_lds();
   }
   const float lse = a.lse[row];
 
@@ -315,7 +351,9 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
         if (tkk > tq) break;
         const int j = time_row(tq, tkk, T_);
         a.dbias_time[row * T_ + j] = Gtb[jj * 32 + ln];
-        a.ws_time[(((int64_t)bh * T_ + tq) * T_ + tkk) * C_ + cq] = Stb[jj * 32 + ln] - lse;
+        const float e = Stb[jj * 32 + ln] - lse + mc;
+        const bool near_pair = has_content && (W <= 0 || tq - tkk <= W || tq == T_ - 1);
+        a.ws_time[(((int64_t)bh * T_ + tq) * T_ + tkk) * C_ + cq] = near_pair ? e : __builtin_amdgcn_exp2f(e);
       }
     }
   };
@@ -367,11 +405,41 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
     }
   };
 
-  // one key step; NEAR = inside the content window.  The far and the near steps of a wave run in
-  // two loops of their own: one loop with a run-time test costs copies of whole accumulator
-  // tiles wherever the two paths join.
-  auto key_step = [&](auto near_c, const unsigned char* Vrow, int tk) {
-    constexpr bool NEAR = decltype(near_c)::value;
+  // A far key step (content term dropped): P^T = Ec et with et = exp2(time bias - L + mc) one
+  // scalar per query, so with dP^T = V dO^T
+  //     dbias_time[q, tk]  = scale et (sum_keys Ec dP - delta sumEc)
+  //     dbias_chan share   = Ec (sum_tk scale et dP - delta sum_tk scale et)   (formed after the loop)
+  // costs two FMAs per element and no exponential per element.
+  float esum = 0.f;
+  auto far_step = [&](const unsigned char* Vrow, int tk) {
+    const float st = Stb[(tk & 31) * 32 + ln];
+    f32x16 dP[NCT];
+#pragma unroll
+    for (int t = 0; t < NCT; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) dP[t][i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int t = 0; t < NCT; ++t)
+        dP[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Vrow + r_lane[ks] + t * 32 * ROWB), dOf[ks], dP[t], 0, 0, 0);
+    const float et = __builtin_amdgcn_exp2f(st - lse + mc) * a.sm_scale;
+    float dot[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < NCT; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        dot[i & 3] += Ec[t][i] * dP[t][i];
+        dSc[t][i] += et * dP[t][i];
+      }
+    esum += et;
+    const float gt = et * (xhalf_sum((dot[0] + dot[1]) + (dot[2] + dot[3])) - delta * sumEc);
+    if (hh == 0) Gtb[(tk & 31) * 32 + ln] = gt;
+  };
+
+  // A key step inside the content window
+  f32x16 Bc[NCT];
+  auto near_step = [&](const unsigned char* Vrow, int tk) {
     const unsigned char* Krow = Vrow + TILE;
     const unsigned char* Ktr = Vrow + 2 * TILE;
     const float st = Stb[(tk & 31) * 32 + ln];
@@ -387,7 +455,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
 #pragma unroll
       for (int t = 0; t < NCT; ++t) {
         const int off = r_lane[ks] + t * 32 * ROWB;
-        if (NEAR) S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Krow + off), Qu[ks], S[t], 0, 0, 0);
+        S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Krow + off), Qu[ks], S[t], 0, 0, 0);
         dP[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Vrow + off), dOf[ks], dP[t], 0, 0, 0);
       }
     const float off2 = st - lse;
@@ -404,17 +472,15 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
       }
     gt = xhalf_sum(gt);
     if (hh == 0) Gtb[(tk & 31) * 32 + ln] = gt;
-    if (NEAR) {
 #pragma unroll
-      for (int t = 0; t < NCT; ++t)
+    for (int t = 0; t < NCT; ++t)
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-          const bf16x8 dsf = pack8(S[t], 8 * s);
+      for (int s = 0; s < 2; ++s) {
+        const bf16x8 dsf = pack8(S[t], 8 * s);
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            dq[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Ktr, t, s, mt), dsf, dq[mt], 0, 0, 0);
-        }
-    }
+        for (int mt = 0; mt < MT; ++mt)
+          dq[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Ktr, t, s, mt), dsf, dq[mt], 0, 0, 0);
+      }
   };
 
   // far steps first (none for the last time step, whose queries keep the content term everywhere),
@@ -424,13 +490,19 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
   for (; tk < far_end; ++tk) {
     const unsigned char* Vrow = ring_step(tk);
     time_slab(tk);
-    key_step(std::false_type{}, Vrow, tk);
+    far_step(Vrow, tk);
   }
+  // the far steps' share of the channel-table gradient; from here on the tile holds the bias
+#pragma unroll
+  for (int t = 0; t < NCT; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dSc[t][i] = Ec[t][i] * (dSc[t][i] - delta * esum);
+  gather_bc(Bc);
   for (; tk <= tq_hi; ++tk) {
     const unsigned char* Vrow = ring_step(tk);
     if (active && tk <= tq) {
       time_slab(tk);
-      key_step(std::true_type{}, Vrow, tk);
+      near_step(Vrow, tk);
     }
   }
 
@@ -480,7 +552,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
 int mvpa_bwd_query_mfma_supported(const mvpa_bwd_args* a) {
   if (a->dtype != MVPA_BF16 || a->Dh != 64 || a->C > 64) return 0;
   if (!(a->flags & MVPA_FLAG_CAUSAL) || a->key_bias || !a->ws_qu) return 0;
-  if (a->C & 1) return 0;      // 16-byte direct-to-LDS loads of the [C][C] channel-table blocks
+  if (a->C & 3) return 0;      // 16-byte direct-to-LDS loads of the rows of the [C][C] Ec tiles
   const uintptr_t p = (uintptr_t)a->q | (uintptr_t)a->k | (uintptr_t)a->v | (uintptr_t)a->o |
                       (uintptr_t)a->d_o | (uintptr_t)a->bias_u | (uintptr_t)a->bias_v |
                       (uintptr_t)a->bias_z | (uintptr_t)a->k_time | (uintptr_t)a->k_chan |
@@ -520,26 +592,34 @@ int mvpa_launch_bwd_query_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
 // operands) and walks every query time step tq >= tk of every query head of the group, both
 // query-channel tiles in turn.  Products are formed NON-transposed here, S[q][key] = (q+u) K^T,
 // so that a lane owns one key and the contraction index of dv^T = dO^T P and dk^T = (q+u)^T dS
-// is the register index:
-//     S   = (q+u) K^T (inside the window) + chan[q][C-1-|cq-ck|] + (time[q][tk] - L[q])
-//     P   = exp2(S),  dP = dO V^T,  dS = P o (dP - delta[q])
-//     dv^T[d][key] += dO^T[d][q] P[q][key],   dk^T[d][key] += (q+u)^T[d][q] dS[q][key]
-// Everything per query comes from the query pass's workspace in the units used here.  Per
-// (head, tq) one ring stage holds (q+u) * scale and dO (each in the two swizzles), the
-// channel-table rows and the per-query scalars, fetched by direct-to-LDS loads two steps ahead.
-// The query steps are walked from the last one down, and the workgroups of one (b, kv head) sit
-// on one XCD: they then read the same stage data at about the same time and share it in L2.
+// is the register index.  With Ec[q][key] = exp2(channel bias - mc[q]) and, per (query, tk), one
+// scalar from the query pass (the exponent e = time bias - L + mc inside the content window,
+// exp2(e) outside it):
+//     inside :  P = exp2((q+u) K^T + e) o Ec,  dP = dO V^T,  dS = P o (dP - delta[q])
+//               dv^T[d][key] += dO^T[d][q] P[q][key],   dk^T[d][key] += (q+u)^T[d][q] dS[q][key]
+//     outside:  P = exp2(e) Ec,                dv^T += dO^T P           (dk gets nothing)
+// Per (head, tq) one ring stage holds dO in the transposing-read swizzle, the Ec tile and the
+// scalars, and for steps that are inside the window for some wave also dO in the row-fragment
+// swizzle, (q+u) * scale in both swizzles and delta; direct-to-LDS loads fetch it two steps
+// ahead.  The query steps are walked from the last one down and the workgroups of one
+// (b, kv head) sit on one XCD: they then read the same stage data at about the same time and
+// share it in L2.  MASKED: C is not a multiple of 32, padded query rows and key lanes are cut.
 // ==========================================================================================
 namespace mvpa {
 namespace bwdq {
 
-template <int NCT>
+template <int NCT, bool MASKED>
 __global__ __launch_bounds__(NW * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_args a) {
   constexpr int CP = NCT * 32, KT = NW / NCT, TILE = CP * ROWB;
   constexpr int CS_BYTES = CP * CP * 4, SC_BYTES = (KT + 1) * 256;
   constexpr int STAGES = KSTAGES, STAGE_BYTES = 4 * TILE + CS_BYTES + SC_BYTES;
+  static_assert(STAGES == 3, "the wait below counts the loads of exactly one younger step");
   constexpr int LPW = CP / 8 / NW, CS_LPW = CS_BYTES / 1024 / NW;
-  constexpr int LPS = 4 * LPW + CS_LPW + 2;       // direct-to-LDS loads per wave and step
+  // direct-to-LDS loads per wave and step
+  constexpr int LPS_FAR = LPW + CS_LPW + 1, LPS_NEAR = 4 * LPW + CS_LPW + 2;
+  // stage layout: dO (transposing) | Ec | scalars | dO (rows) | (q+u) (rows) | (q+u) (transposing)
+  constexpr int OFF_DTR = 0, OFF_EC = TILE, OFF_SC = TILE + CS_BYTES, OFF_DROW = OFF_SC + SC_BYTES,
+                OFF_QROW = OFF_DROW + TILE, OFF_QTR = OFF_QROW + TILE;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -569,8 +649,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_arg
   const int tkc = min(tk, T_ - 1);
 
   const int ck = kt * 32 + ln;
-  bool key_ok = ck < C_;
-  if (key_ok && a.chan_valid) key_ok = a.chan_valid[(int64_t)b * C_ + ck] != 0;
+  const bool key_live = ck < C_;                  // invalid channels have Ec = 0 already
   const int64_t nk = (int64_t)tkc * C_ + min(ck, C_ - 1);
   const bf16_t* krow = (const bf16_t*)a.k + b * a.k_stride_b + g * a.k_stride_h + nk * a.k_stride_n;
   const bf16_t* vrow = (const bf16_t*)a.v + b * a.v_stride_b + g * a.v_stride_h + nk * a.v_stride_n;
@@ -593,33 +672,44 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_arg
     d_off_r[i] = rc * (int)a.do_stride_n + ((phys ^ swz_row(r)) << 3);
     d_off_t[i] = rc * (int)a.do_stride_n + ((phys ^ swz_tr(r)) << 3);
   }
+  // the Ec tile [C][C] lands with a row pitch of CP floats
 #pragma unroll
-  for (int i = 0; i < CS_LPW; ++i)
-    cs_off[i] = min((wave + NW * i) * 64 + lane, C_ * C_ / 4 - 1) * 4;   // C is even here
+  for (int i = 0; i < CS_LPW; ++i) {
+    const int pc = (wave + NW * i) * 64 + lane;   // 16-byte chunk: row pc / (CP/4), 4 columns
+    const int r = min(pc / (CP / 4), C_ - 1), c4 = min((pc % (CP / 4)) * 4, (C_ - 1) & ~3);
+    cs_off[i] = r * C_ + c4;
+  }
   const int sc_lane = min(lane, C_ - 1);
   const uint32_t ring_lds = (uint32_t)(uintptr_t)(BWD_LDS_PTR(unsigned char))smem;
+  // a step is fetched in full when it lies inside the content window of one of the waves
+  auto wg_near = [&](int tq) -> bool {
+    return has_content && (W <= 0 || tq == T_ - 1 || tq - tk0 <= W + KT - 1);
+  };
   auto issue_step = [&](int hq, int tq, int stage_idx) {
     const int h = g * grp + hq;
     const int64_t bhq = (int64_t)b * a.H + h;
     const int64_t r0 = bhq * N + (int64_t)tq * C_;          // first query row of the step
     const uint32_t st = ring_lds + stage_idx * STAGE_BYTES;
-    const bf16_t* qsrc = (const bf16_t*)a.ws_qu + r0 * DH;
     const bf16_t* dsrc = (const bf16_t*)a.d_o + b * a.do_stride_b + h * a.do_stride_h +
                          (int64_t)tq * C_ * a.do_stride_n;
-#pragma unroll
-    for (int i = 0; i < LPW; ++i) {
-      const uint32_t dst = st + (wave + NW * i) * 1024;
-      dma16(qsrc + q_off_r[i], dst);
-      dma16(qsrc + q_off_t[i], dst + TILE);
-      dma16(dsrc + d_off_r[i], dst + 2 * TILE);
-      dma16(dsrc + d_off_t[i], dst + 3 * TILE);
-    }
     const float* csrc = a.ws_chan + r0 * C_;
 #pragma unroll
-    for (int i = 0; i < CS_LPW; ++i) dma16(csrc + cs_off[i], st + 4 * TILE + (wave + NW * i) * 1024);
-    // per-query scalars: (time bias - L) for this wave's key step, and delta
-    dma4(a.ws_time + ((bhq * T_ + tq) * T_ + tkc) * C_ + sc_lane, st + 4 * TILE + CS_BYTES + ktw * 256);
-    dma4(a.ws_delta + r0 + sc_lane, st + 4 * TILE + CS_BYTES + KT * 256);
+    for (int i = 0; i < LPW; ++i) dma16(dsrc + d_off_t[i], st + OFF_DTR + (wave + NW * i) * 1024);
+#pragma unroll
+    for (int i = 0; i < CS_LPW; ++i) dma16(csrc + cs_off[i], st + OFF_EC + (wave + NW * i) * 1024);
+    // per-query scalar of this wave's key step
+    dma4(a.ws_time + ((bhq * T_ + tq) * T_ + tkc) * C_ + sc_lane, st + OFF_SC + ktw * 256);
+    if (wg_near(tq)) {
+      const bf16_t* qsrc = (const bf16_t*)a.ws_qu + r0 * DH;
+#pragma unroll
+      for (int i = 0; i < LPW; ++i) {
+        const uint32_t dst = st + (wave + NW * i) * 1024;
+        dma16(dsrc + d_off_r[i], dst + OFF_DROW);
+        dma16(qsrc + q_off_r[i], dst + OFF_QROW);
+        dma16(qsrc + q_off_t[i], dst + OFF_QTR);
+      }
+      dma4(a.ws_delta + r0 + sc_lane, st + OFF_SC + KT * 256);
+    }
   };
 
   f32x16 dK[MT], dV[MT];
@@ -655,61 +745,87 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_arg
   for (int s = 0; s < STAGES - 1; ++s)
     if (s < nsteps) { issue_step(ihq, itq, s); next_issue(); }
 
-  int stage = 0, it = 0;
+  int stage = 0, it = 0, ring_tq = T_ - 1;        // ring_tq: query step of the stage handed out next
   // advances the ring by one step and returns the stage that holds its data
   auto ring_step = [&]() -> const unsigned char* {
-    if (it + STAGES - 2 < nsteps) wait_vmcnt_imm<(STAGES - 2) * LPS>();
-    else wait_vmcnt_imm<0>();
+    // the step has landed once only the loads of the one younger step are in flight
+    const int next_tq = ring_tq - 1 < tk0 ? T_ - 1 : ring_tq - 1;
+    if (it + 1 >= nsteps) wait_vmcnt_imm<0>();
+    else if (wg_near(next_tq)) wait_vmcnt_imm<LPS_NEAR>();
+    else wait_vmcnt_imm<LPS_FAR>();
     lds_barrier();            // this step's stage visible to all; the previous one is free
     if (it + STAGES - 1 < nsteps) { issue_step(ihq, itq, stage == 0 ? STAGES - 1 : stage - 1); next_issue(); }
     const unsigned char* base = smem + stage * STAGE_BYTES;
     stage = stage + 1 == STAGES ? 0 : stage + 1;
+    ring_tq = next_tq;
     ++it;
     return base;
   };
 
-  // one query step; NEAR = inside the content window (as in the query pass, the far and the near
-  // steps run in loops of their own)
-  auto query_step = [&](auto near_c, const unsigned char* Qrow, int tq_now) {
-    constexpr bool NEAR = decltype(near_c)::value;
-    // Qrow: (q+u)*scale, row-fragment swizzle
-    const unsigned char* Qtr = Qrow + TILE;                   // same, transposing-read swizzle
-    const unsigned char* Drow = Qrow + 2 * TILE;              // dO, row-fragment swizzle
-    const unsigned char* Dtr = Qrow + 3 * TILE;               // dO, transposing-read swizzle
-    const float* Cs = (const float*)(Qrow + 4 * TILE);        // [C][C] channel-table rows
-    const float* TL = (const float*)(Qrow + 4 * TILE + CS_BYTES) + ktw * 64;   // time bias - L
-    const float* De = (const float*)(Qrow + 4 * TILE + CS_BYTES) + KT * 64;    // delta
-    (void)tq_now;
+  // ---- a query step outside the content window: P = Ec * exp2(e), dv only
+  auto far_step = [&](const unsigned char* base) {
+    const unsigned char* Dtr = base + OFF_DTR;
+    const float* Ecs = (const float*)(base + OFF_EC) + ck;
+    const float* ET = (const float*)(base + OFF_SC) + ktw * 64;
 #pragma unroll
     for (int qt = 0; qt < NCT; ++qt) {
-      // ---- S[q][key] and dP[q][key] for query-channel tile qt
+      f32x16 P;
+#pragma unroll
+      for (int a4 = 0; a4 < 4; ++a4) {
+        const int rb = qt * 32 + a4 * 8 + hh * 4;              // query channels rb .. rb+3
+        const float4 e4 = *(const float4*)(ET + rb);
+        const float es[4] = {e4.x, e4.y, e4.z, e4.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float p = Ecs[(rb + j) * CP] * es[j];
+          P[a4 * 4 + j] = (!MASKED || (key_live && rb + j < C_)) ? p : 0.f;
+        }
+      }
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const bf16x8 pf = pack8(P, 8 * s);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          dV[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Dtr, qt, s, mt), pf, dV[mt], 0, 0, 0);
+      }
+    }
+  };
+
+  // ---- a query step inside the content window
+  auto near_step = [&](const unsigned char* base) {
+    const unsigned char* Dtr = base + OFF_DTR;
+    const unsigned char* Drow = base + OFF_DROW;
+    const unsigned char* Qrow = base + OFF_QROW;
+    const unsigned char* Qtr = base + OFF_QTR;
+    const float* Ecs = (const float*)(base + OFF_EC) + ck;
+    const float* TL = (const float*)(base + OFF_SC) + ktw * 64;
+    const float* De = (const float*)(base + OFF_SC) + KT * 64;
+#pragma unroll
+    for (int qt = 0; qt < NCT; ++qt) {
       f32x16 S, dP, dS;
 #pragma unroll
       for (int i = 0; i < 16; ++i) { S[i] = 0.f; dP[i] = 0.f; }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const int off = r_lane[ks] + qt * 32 * ROWB;
-        if (NEAR) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Qrow + off), Kf[ks], S, 0, 0, 0);
+        S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Qrow + off), Kf[ks], S, 0, 0, 0);
         dP = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Drow + off), Vf[ks], dP, 0, 0, 0);
       }
 #pragma unroll
       for (int a4 = 0; a4 < 4; ++a4) {
-        const int rb = qt * 32 + a4 * 8 + hh * 4;              // query channels rb .. rb+3
+        const int rb = qt * 32 + a4 * 8 + hh * 4;
         const float4 tl = *(const float4*)(TL + rb);
         const float4 de = *(const float4*)(De + rb);
         const float tls[4] = {tl.x, tl.y, tl.z, tl.w}, des[4] = {de.x, de.y, de.z, de.w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const int i = a4 * 4 + j, r = rb + j;
-          const int dist = r > ck ? r - ck : ck - r;
-          const int col = max(C_ - 1 - dist, 0);
-          const float s = S[i] + Cs[r * C_ + col] + tls[j];
-          const float p = (key_ok && r < C_) ? __builtin_amdgcn_exp2f(s) : 0.f;   // padded rows/keys
+          const int i = a4 * 4 + j;
+          float p = __builtin_amdgcn_exp2f(S[i] + tls[j]) * Ecs[(rb + j) * CP];
+          if (MASKED) p = (key_live && rb + j < C_) ? p : 0.f;
           S[i] = p;
           dS[i] = p * (dP[i] - des[j]) * (1.f / kLog2e);
         }
       }
-      // ---- dv^T[d][key] += dO^T[d][q] P[q][key];  dk^T[d][key] += (q+u)^T[d][q] dS[q][key]
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         const bf16x8 pf = pack8(S, 8 * s);
@@ -717,7 +833,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_arg
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           dV[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Dtr, qt, s, mt), pf, dV[mt], 0, 0, 0);
-          if (NEAR) dK[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Qtr, qt, s, mt), sf, dK[mt], 0, 0, 0);
+          dK[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Qtr, qt, s, mt), sf, dK[mt], 0, 0, 0);
         }
       }
     }
@@ -738,10 +854,9 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_arg
   }
   const int n_idle = span - n_last - n_far - n_win;
   for (int hq = 0; hq < grp; ++hq) {
-    int tq = T_ - 1;
-    for (int n = n_last; n > 0; --n, --tq) query_step(std::true_type{}, ring_step(), tq);
-    for (int n = n_far; n > 0; --n, --tq) query_step(std::false_type{}, ring_step(), tq);
-    for (int n = n_win; n > 0; --n, --tq) query_step(std::true_type{}, ring_step(), tq);
+    for (int n = n_last; n > 0; --n) near_step(ring_step());
+    for (int n = n_far; n > 0; --n) far_step(ring_step());
+    for (int n = n_win; n > 0; --n) near_step(ring_step());
     for (int n = n_idle; n > 0; --n) (void)ring_step();
   }
 
@@ -761,20 +876,21 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_arg
 }  // namespace bwdq
 }  // namespace mvpa
 
-int mvpa_launch_bwd_key_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
+template <int NCT, bool MASKED>
+static void launch_key(const mvpa_bwd_args* a, hipStream_t stream) {
   using namespace mvpa::bwdq;
-  const int nct = a->C <= 32 ? 1 : 2;
-  const int cp = nct * 32, kt = NW / nct;
+  constexpr int cp = NCT * 32, kt = NW / NCT;
   const size_t lds = (size_t)KSTAGES * (4 * cp * ROWB + cp * cp * 4 + (kt + 1) * 256);
   dim3 grid((unsigned)(((a->T + kt - 1) / kt) * a->B * a->Hkv));
-  if (nct == 1) {
-    auto kern = mvpa_bwd_key_mfma_kernel<1>;
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, *a);
-  } else {
-    auto kern = mvpa_bwd_key_mfma_kernel<2>;
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, *a);
-  }
+  auto kern = mvpa_bwd_key_mfma_kernel<NCT, MASKED>;
+  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, *a);
+}
+
+int mvpa_launch_bwd_key_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
+  if (a->C == 32) launch_key<1, false>(a, stream);
+  else if (a->C < 32) launch_key<1, true>(a, stream);
+  else if (a->C == 64) launch_key<2, false>(a, stream);
+  else launch_key<2, true>(a, stream);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
