@@ -35,6 +35,8 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 constexpr int DH = 64, KS = 4, MT = 2, ROWB = 128, NW = 4;
 constexpr int QSTAGES = 3, KSTAGES = 3;          // ring depth of the query / key pass
+// floats of per-wave scratch in the query pass: two time-bias slabs and the channel table
+template <int NCT> constexpr int WAVE_SCRATCH = 1024 + 32 * 33 + 32 * (NCT * 32 + 1);
 
 __device__ inline void wave_sync_lds() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -51,10 +53,12 @@ __device__ inline void lds_barrier() {
 // that the compiler does not drain the ring in front of later LDS reads; completion is awaited
 // with wait_vmcnt() before the barrier that publishes a stage.
 __device__ inline void dma16(const void* gptr, uint32_t lds_base) {
+  lds_base = __builtin_amdgcn_readfirstlane(lds_base);    // uniform by construction; pins it to an SGPR
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :: "v"(gptr), "s"(lds_base) : "memory", "m0");
 }
 __device__ inline void dma4(const void* gptr, uint32_t lds_base) {
+  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
                :: "v"(gptr), "s"(lds_base) : "memory", "m0");
 }
@@ -122,9 +126,10 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 31, hh = lane >> 5;
-  float* Stb = wave_base + wave * (2 * 1024 + CP * 32);   // [32][32] time-bias scores of a slab
-  float* Gtb = Stb + 1024;                                // [32][32] their gradients
-  float* scr = Gtb + 1024;                                // [CP][32] channel table, later [32][CP]
+  constexpr int GP = 33, PC = CP + 1;             // padded pitches: the transposed reads spread over the banks
+  float* Stb = wave_base + wave * WAVE_SCRATCH<NCT>;      // [32][32] time-bias scores of a slab
+  float* Gtb = Stb + 1024;                                // [32][GP] their gradients
+  float* scr = Gtb + 32 * GP;                             // [CP][32] channel table, later [32][PC]
 
   const int T_ = a.T, C_ = a.C, W = a.window, N = a.T * a.C;
   const bool has_content = a.flags & MVPA_FLAG_CONTENT;
@@ -203,7 +208,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
     if (s <= tq_hi) issue_tile(s, s, s >= tk_near);
 
   // ---- set-up: operand fragments, delta, channel-bias tile
-  bf16x8 Qu[KS], Qv[KS], dOf[KS];
+  bf16x8 dOf[KS];            // (q+u), (q+v) fragments are re-formed where needed, not kept
   f32x16 Ec[NCT];            // exp2(channel bias - mc): the far steps' probabilities up to a scalar
   float delta = 0.f, mc = -INFINITY, sumEc = 0.f;
   uint32_t kbits[NCT];
@@ -236,8 +241,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
       const u32x4 raw = *(const u32x4*)(qrow + d0);
       const u32x4 draw = *(const u32x4*)(drow + d0);
       const u32x4 oraw = *(const u32x4*)(orow + d0);
-      Qu[ks] = qfrag(raw, bu + d0, sc2);
-      Qv[ks] = qfrag(raw, bv + d0, sc2);
+      if (qok) *(bf16x8*)((bf16_t*)a.ws_qu + row * DH + d0) = qfrag(raw, bu + d0, sc2);   // for the key pass
       const bf16x8 qz = qfrag(raw, bz + d0, sc2);
       dOf[ks] = as_frag(draw);
 #pragma unroll
@@ -289,9 +293,6 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
     // for the key pass: (q+u) * scale, delta, and the tile exp2(channel bias - mc) by
     // [query][key channel]; and the rows of dbias_time that no key step reaches
     if (qok) {
-      bf16_t* wq = (bf16_t*)a.ws_qu + row * DH;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) *(bf16x8*)(wq + ks * 16 + hh * 8) = Qu[ks];
       float* wc = a.ws_chan + row * C_;
 #pragma unroll
       for (int t = 0; t < NCT; ++t)
@@ -308,12 +309,12 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
           }
         }
     }
-    if (qok && hh == 0) {
-      a.ws_delta[row] = delta;
-      for (int j = 0; j < T_ - 1 - tq; ++j) a.dbias_time[row * T_ + j] = 0.f;
-    }
+    if (qok && hh == 0) a.ws_delta[row] = delta;
   }
   const float lse = a.lse[row];
+  // consumed here so that the wait for this load stands in front of the loops: left to the first
+  // use inside them, it would drain the whole ring (vmcnt 0) at every key step
+  asm volatile("" :: "v"(lse));
 
   f32x16 dq[MT], dSc[NCT];
 #pragma unroll
@@ -324,6 +325,16 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
   for (int t = 0; t < NCT; ++t)
 #pragma unroll
     for (int i = 0; i < 16; ++i) dSc[t][i] = 0.f;
+
+  // this wave's query rows are consecutive in memory; outputs are written a row at a time (the
+  // two half-waves take alternate rows) so that each store covers one contiguous run
+  const int cq0 = (wave % NCT) * 32;
+  const int nq_live = active ? max(0, min(32, C_ - cq0)) : 0;
+  const int64_t wrow0 = ((int64_t)b * a.H + h) * N + (int64_t)(active ? tq : 0) * C_ + cq0;
+
+  // the columns of dbias_time that no key step reaches
+  for (int q = hh; q < nq_live; q += 2)
+    for (int j = ln; j < T_ - 1 - tq; j += 32) a.dbias_time[(wrow0 + q) * T_ + j] = 0.f;
 
   // ---- loop-invariant fragment offsets
   int r_lane[KS], t_lane[MT];
@@ -343,19 +354,21 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
 
-  // writes the gradients of the slab that started at key step tk0 (and its forward scores)
-  auto flush_slab = [&](int tk0) {
+  // writes the gradients of the slab that started at key step tks, and its per-pair scalars for
+  // the key pass (the exponent e = time bias - L + mc for pairs inside the window, else exp2(e))
+  auto flush_slab = [&](int tks) {
+    const int nj = min(32, tq - tks + 1);
     if (hh == 0 && qok) {
-      for (int jj = 0; jj < 32; ++jj) {
-        const int tkk = tk0 + jj;
-        if (tkk > tq) break;
-        const int j = time_row(tq, tkk, T_);
-        a.dbias_time[row * T_ + j] = Gtb[jj * 32 + ln];
+      for (int jj = 0; jj < nj; ++jj) {
+        const int tkk = tks + jj;
         const float e = Stb[jj * 32 + ln] - lse + mc;
         const bool near_pair = has_content && (W <= 0 || tq - tkk <= W || tq == T_ - 1);
         a.ws_time[(((int64_t)bh * T_ + tq) * T_ + tkk) * C_ + cq] = near_pair ? e : __builtin_amdgcn_exp2f(e);
       }
     }
+    const int j0 = time_row(tq, tks, T_);
+    for (int q = hh; q < nq_live; q += 2)
+      if (ln < nj) a.dbias_time[(wrow0 + q) * T_ + j0 + ln] = Gtb[ln * GP + q];
   };
 
   int stage = 0;
@@ -396,7 +409,8 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const u32x4 rr = *(const u32x4*)(ktime + (int64_t)j * DH + ks * 16 + hh * 8);
-          stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(rr), Qv[ks], stc, 0, 0, 0);
+          const bf16x8 qv = qfrag(*(const u32x4*)(qrow + ks * 16 + hh * 8), bv + ks * 16 + hh * 8, sc2);
+          stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(rr), qv, stc, 0, 0, 0);
         }
       }
 #pragma unroll
@@ -410,20 +424,13 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
   //     dbias_time[q, tk]  = scale et (sum_keys Ec dP - delta sumEc)
   //     dbias_chan share   = Ec (sum_tk scale et dP - delta sum_tk scale et)   (formed after the loop)
   // costs two FMAs per element and no exponential per element.
+  // The loop is software-pipelined: the products of step tk are issued to the matrix cores, and
+  // the vector work on the products of step tk-1 runs meanwhile.
   float esum = 0.f;
-  auto far_step = [&](const unsigned char* Vrow, int tk) {
-    const float st = Stb[(tk & 31) * 32 + ln];
-    f32x16 dP[NCT];
-#pragma unroll
-    for (int t = 0; t < NCT; ++t)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) dP[t][i] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-      for (int t = 0; t < NCT; ++t)
-        dP[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Vrow + r_lane[ks] + t * 32 * ROWB), dOf[ks], dP[t], 0, 0, 0);
-    const float et = __builtin_amdgcn_exp2f(st - lse + mc) * a.sm_scale;
+  // reduces the products of far step tkp (none if tkp < 0)
+  auto far_reduce = [&](const f32x16 (&dP)[NCT], int tkp) {
+    if (tkp < 0) return;
+    const float et = __builtin_amdgcn_exp2f(Stb[(tkp & 31) * 32 + ln] - lse + mc) * a.sm_scale;
     float dot[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int t = 0; t < NCT; ++t)
@@ -434,11 +441,37 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
       }
     esum += et;
     const float gt = et * (xhalf_sum((dot[0] + dot[1]) + (dot[2] + dot[3])) - delta * sumEc);
-    if (hh == 0) Gtb[(tk & 31) * 32 + ln] = gt;
+    if (hh == 0) Gtb[(tkp & 31) * GP + ln] = gt;
+  };
+  // one far step: products of tile tk into cur, reduction of step tk-1 (in prev) alongside
+  auto far_step = [&](int tk, int& tkp, f32x16 (&cur)[NCT], const f32x16 (&prev)[NCT]) {
+    const unsigned char* Vrow = ring_step(tk);
+    if ((tk & 31) == 0) {                         // the slab about to be written must be complete
+      far_reduce(prev, tkp);
+      tkp = -1;
+      time_slab(tk);
+    }
+    bf16x8 vf[KS][NCT];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int t = 0; t < NCT; ++t) vf[ks][t] = *(const bf16x8*)(Vrow + r_lane[ks] + t * 32 * ROWB);
+#pragma unroll
+    for (int t = 0; t < NCT; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) cur[t][i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int t = 0; t < NCT; ++t)
+        cur[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[ks][t], dOf[ks], cur[t], 0, 0, 0);
+    far_reduce(prev, tkp);
+    tkp = tk;
   };
 
   // A key step inside the content window
   f32x16 Bc[NCT];
+  bf16x8 Qu[KS];
   auto near_step = [&](const unsigned char* Vrow, int tk) {
     const unsigned char* Krow = Vrow + TILE;
     const unsigned char* Ktr = Vrow + 2 * TILE;
@@ -471,7 +504,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
         gt += ds;
       }
     gt = xhalf_sum(gt);
-    if (hh == 0) Gtb[(tk & 31) * 32 + ln] = gt;
+    if (hh == 0) Gtb[(tk & 31) * GP + ln] = gt;
 #pragma unroll
     for (int t = 0; t < NCT; ++t)
 #pragma unroll
@@ -487,10 +520,20 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
   // then the steps inside the window; waves that are done keep the ring and the barriers going
   const int far_end = !active ? 0 : !has_content ? tq + 1 : (W <= 0 || tq == T_ - 1) ? 0 : max(0, tq - W);
   int tk = 0;
-  for (; tk < far_end; ++tk) {
-    const unsigned char* Vrow = ring_step(tk);
-    time_slab(tk);
-    far_step(Vrow, tk);
+  {
+    f32x16 dPa[NCT], dPb[NCT];
+    int tkp = -1;
+    for (; tk + 1 < far_end; tk += 2) {
+      far_step(tk, tkp, dPa, dPb);
+      far_step(tk + 1, tkp, dPb, dPa);
+    }
+    if (tk < far_end) {
+      far_step(tk, tkp, dPa, dPb);
+      ++tk;
+      far_reduce(dPa, tkp);
+    } else {
+      far_reduce(dPb, tkp);
+    }
   }
   // the far steps' share of the channel-table gradient; from here on the tile holds the bias
 #pragma unroll
@@ -498,6 +541,9 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
 #pragma unroll
     for (int i = 0; i < 16; ++i) dSc[t][i] = Ec[t][i] * (dSc[t][i] - delta * esum);
   gather_bc(Bc);
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    Qu[ks] = qfrag(*(const u32x4*)(qrow + ks * 16 + hh * 8), bu + ks * 16 + hh * 8, sc2);
   for (; tk <= tq_hi; ++tk) {
     const unsigned char* Vrow = ring_step(tk);
     if (active && tk <= tq) {
@@ -522,9 +568,9 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
   }
 
   // channel-table gradient: element (ck) of query cq goes to column C-1-|cq-ck|; the two key
-  // channels at the same distance add up.  Per-wave table [32 queries][CP] in the scratch.
+  // channels at the same distance add up.  Per-wave table [32 queries][PC] in the scratch.
   wave_sync_lds();
-  for (int i = lane; i < 32 * CP; i += 64) scr[i] = 0.f;
+  for (int i = lane; i < 32 * PC; i += 64) scr[i] = 0.f;
   wave_sync_lds();
   {
     const uint32_t cq4 = (uint32_t)(cq - 4 * hh + 4);
@@ -535,14 +581,12 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
         const uint32_t ci4 = (uint32_t)(t * 32 + (i >> 2) * 8 + (i & 3) + 4);
         const uint32_t dist = max(cq4, ci4) - min(cq4, ci4);
         const bool kv = (kbits[t] >> ((i >> 2) * 8 + (i & 3))) & 1u;
-        if (kv && dist < (uint32_t)C_ && qok) atomicAdd(&scr[ln * CP + (C_ - 1 - (int)dist)], dSc[t][i]);
+        if (kv && dist < (uint32_t)C_ && qok) atomicAdd(&scr[ln * PC + (C_ - 1 - (int)dist)], dSc[t][i]);
       }
   }
   wave_sync_lds();
-  if (qok && hh == 0) {
-    float* gc = a.dbias_chan + row * C_;
-    for (int i = 0; i < C_; ++i) gc[i] = scr[ln * CP + i];
-  }
+  for (int q = 0; q < nq_live; ++q)
+    if (lane < C_) a.dbias_chan[(wrow0 + q) * C_ + lane] = scr[q * PC + lane];
 }
 
 }  // namespace bwdq
@@ -572,7 +616,8 @@ int mvpa_launch_bwd_query_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
   const int tqw = NW / nct;
   const int nt = (a->T + tqw - 1) / tqw;
   const int cp = nct * 32;
-  const size_t lds = (size_t)QSTAGES * 3 * cp * ROWB + (size_t)NW * (2 * 1024 + cp * 32) * sizeof(float);
+  const size_t lds = (size_t)QSTAGES * 3 * cp * ROWB +
+                     (size_t)NW * (nct == 1 ? WAVE_SCRATCH<1> : WAVE_SCRATCH<2>) * sizeof(float);
   dim3 grid((unsigned)(nt * a->B * a->H));
   if (nct == 1) {
     auto kern = mvpa_bwd_query_mfma_kernel<1>;
