@@ -50,14 +50,25 @@ class FlashMVPA(torch.autograd.Function):
         dbt = dbt.view(B, Hkv, grp, N, -1)
         dbc = dbc.view(B, Hkv, grp, N, -1)
         rt, ec = k_time.float(), k_chan.float()                    # [Hkv,T,Dh], [Hkv,C,Dh]
-        dq_t = torch.einsum("bgrnj,gjd->bgrnd", dbt, rt)
-        dq_ch = torch.einsum("bgrnj,gjd->bgrnd", dbc, ec)
-        dq = dq_c.view(B, Hkv, grp, N, Dh) + dq_t + dq_ch
-        du = dq_c.view(B, Hkv, grp, N, Dh).sum(dim=(0, 2, 3))
-        dvb = dq_t.sum(dim=(0, 2, 3))
-        dz = dq_ch.sum(dim=(0, 2, 3))
-        dk_time = torch.einsum("bgrnj,bgrnd->gjd", dbt, qf + vb.float()[None, :, None, None, :])
-        dk_chan = torch.einsum("bgrnj,bgrnd->gjd", dbc, qf + z.float()[None, :, None, None, :])
+        dq_cv = dq_c.view(B, Hkv, grp, N, Dh)
+        dq = dq_cv
+        du = dq_cv.sum(dim=(0, 2, 3))
+        # a bias term that is switched off takes no part in the forward: its table, its query
+        # bias and the query get nothing through it
+        if time_bias:
+            dq_t = torch.einsum("bgrnj,gjd->bgrnd", dbt, rt)
+            dq = dq + dq_t
+            dvb = dq_t.sum(dim=(0, 2, 3))
+            dk_time = torch.einsum("bgrnj,bgrnd->gjd", dbt, qf + vb.float()[None, :, None, None, :])
+        else:
+            dvb, dk_time = torch.zeros_like(vb, dtype=torch.float32), torch.zeros_like(rt)
+        if chan_bias:
+            dq_ch = torch.einsum("bgrnj,gjd->bgrnd", dbc, ec)
+            dq = dq + dq_ch
+            dz = dq_ch.sum(dim=(0, 2, 3))
+            dk_chan = torch.einsum("bgrnj,bgrnd->gjd", dbc, qf + z.float()[None, :, None, None, :])
+        else:
+            dz, dk_chan = torch.zeros_like(z, dtype=torch.float32), torch.zeros_like(ec)
         return (dq.view(B, H, N, Dh).to(q.dtype), du.to(u.dtype), dvb.to(vb.dtype), dz.to(z.dtype),
                 dk.to(k.dtype), dk_time.to(k_time.dtype), dk_chan.to(k_chan.dtype), dv.to(v.dtype),
                 None, None, None, None, None, None)

@@ -108,7 +108,11 @@ BF16_CASES = [
     dict(B=1, C=64, T=12, H=2, Hkv=2, Dh=64, window=10),      # two waves per time step
     dict(B=1, C=40, T=37, H=2, Hkv=1, Dh=64, window=10),      # ragged channels, two 32-step slabs, GQA
     dict(B=2, C=8, T=70, H=1, Hkv=1, Dh=64, window=4),        # three slabs, narrow window
-    dict(B=1, C=33, T=9, H=2, Hkv=2, Dh=64, window=0),        # content everywhere
+    dict(B=1, C=33, T=9, H=2, Hkv=2, Dh=64, window=0),        # content everywhere; C % 4 != 0: generic kernels
+    dict(B=1, C=36, T=9, H=2, Hkv=2, Dh=64, window=0),        # content everywhere, ragged second channel tile
+    dict(B=1, C=32, T=21, H=2, Hkv=1, Dh=64, window=3),       # one channel tile, four key steps per workgroup, GQA
+    dict(B=2, C=20, T=40, H=2, Hkv=2, Dh=64, window=5),       # one ragged channel tile, two slabs
+    dict(B=1, C=64, T=45, H=1, Hkv=1, Dh=64, window=2),       # odd T: the last key pair of a workgroup is half empty
 ]
 
 
@@ -120,9 +124,9 @@ def test_backward_bf16_mfma_query_pass(case):
     inp = make_mvpa_inputs(seed=13, qkv_unit=True, **cfg).round_to(torch.bfloat16)
     d_out = torch.randn(inp.q.shape, generator=torch.Generator().manual_seed(6)).bfloat16().float()
     valid = None
-    if cfg["C"] == 40:
-        valid = torch.ones(cfg["B"], 40, dtype=torch.bool)
-        valid[:, [3, 17, 39]] = False
+    if cfg["C"] in (40, 20):
+        valid = torch.ones(cfg["B"], cfg["C"], dtype=torch.bool)
+        valid[:, [3, 17, cfg["C"] - 1]] = False
     _, ref = _oracle_grads(inp, d_out, window, chan_valid=valid)
     _, got = _gpu_grads(inp, d_out, window, torch.bfloat16, chan_valid=valid)
     for n in NAMES:
@@ -139,3 +143,62 @@ def test_backward_rows_are_causal():
     assert got["k"][:, :, 3 * 4:].abs().max().item() == 0.0
     assert got["v"][:, :, 3 * 4:].abs().max().item() == 0.0
     assert got["q"][:, :, 3 * 4:].abs().max().item() == 0.0
+
+
+@pytest.mark.parametrize("flags", [dict(time_bias=False), dict(chan_bias=False)],
+                         ids=lambda f: "+".join(sorted(f)))
+def test_backward_bf16_mfma_bias_flags(flags):
+    """The matrix-core passes with a bias term switched off: its parameters get zero gradient."""
+    inp = make_mvpa_inputs(B=1, C=64, T=20, H=2, Hkv=2, Dh=64, seed=21, qkv_unit=True).round_to(torch.bfloat16)
+    d_out = torch.randn(inp.q.shape, generator=torch.Generator().manual_seed(3)).bfloat16().float()
+    _, ref = _oracle_grads(inp, d_out, 4, **flags)
+    _, got = _gpu_grads(inp, d_out, 4, torch.bfloat16, **flags)
+    for n in NAMES:
+        if ref[n].abs().max().item() == 0.0:
+            assert got[n].abs().max().item() == 0.0, n
+            continue
+        rel = (got[n].double() - ref[n]).norm().item() / max(ref[n].norm().item(), 1e-30)
+        assert rel <= 2e-2, (n, rel)
+
+
+def test_backward_bf16_mfma_rows_are_causal():
+    """As test_backward_rows_are_causal, on the matrix-core passes."""
+    inp = make_mvpa_inputs(B=1, C=32, T=10, H=2, Hkv=2, Dh=64, seed=1, qkv_unit=True)
+    d_out = torch.zeros(inp.q.shape)
+    d_out[:, :, : 3 * 32] = torch.randn(1, 2, 96, 64, generator=torch.Generator().manual_seed(8))
+    _, got = _gpu_grads(inp, d_out, 10, torch.bfloat16)
+    assert got["k"][:, :, 3 * 32:].abs().max().item() == 0.0
+    assert got["v"][:, :, 3 * 32:].abs().max().item() == 0.0
+    assert got["q"][:, :, 3 * 32:].abs().max().item() == 0.0
+
+
+def test_backward_bf16_full_size_invariants():
+    """At the benchmark shape (B4 C64 T128 H16 Dh64, too large for the float64 oracle) the
+    gradients must satisfy what the softmax fixes for ANY d_o:
+      * dS rows sum to zero, so every row of dbias_time and of dbias_chan sums to zero
+        (up to the bf16 rounding of the probabilities: <= 1e-2 of the absolute sum of the row of
+        dbias_chan, which stands for sum_keys |dS|);
+      * with d_o = 1 the columns of dv are the column sums of P, so dv summed over the keys of a
+        (batch, kv head) equals the number of queries of the group's heads, N * H/Hkv."""
+    import mvpa_hip
+    cfg = dict(B=4, C=64, T=128, H=16, Hkv=16, Dh=64)
+    inp = make_mvpa_inputs(seed=0, **cfg).to("cuda", torch.bfloat16)
+    out, lse = mvpa_hip.mvpa_forward(inp.q, inp.k, inp.v, inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan,
+                                     return_lse=True)
+    d_o = torch.randn(out.shape, device="cuda", generator=torch.Generator("cuda").manual_seed(5)).bfloat16()
+    dq, dk, dv, dbt, dbc = mvpa_hip.mvpa_backward(inp.q, inp.k, inp.v, out, d_o, lse, inp.u, inp.vb, inp.z,
+                                                  inp.k_time, inp.k_chan)
+    for t in (dq, dk, dv, dbt, dbc):
+        assert torch.isfinite(t).all()
+    scale = dbc.abs().sum(-1)                          # ~ sum_keys |dS| of the row (measured: ratio <= 3.4e-3)
+    for g in (dbt, dbc):
+        rows = g.sum(-1).abs()
+        assert (rows <= 1e-2 * scale).all(), (rows / scale).max().item()
+    # the two tables hold the same dS, summed differently
+    assert torch.allclose(dbt.sum(-1), dbc.sum(-1), atol=1e-4, rtol=0)
+    ones = torch.ones_like(out)
+    _, _, dv1, _, _ = mvpa_hip.mvpa_backward(inp.q, inp.k, inp.v, out, ones, lse, inp.u, inp.vb, inp.z,
+                                             inp.k_time, inp.k_chan)
+    n_q = cfg["T"] * cfg["C"] * (cfg["H"] // cfg["Hkv"])
+    tot = dv1.sum(2)                                  # [B,Hkv,Dh]
+    assert (tot / n_q - 1).abs().max().item() <= 2e-3, (tot / n_q - 1).abs().max().item()
