@@ -137,18 +137,26 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
   const bool has_chan = a.flags & MVPA_FLAG_CHAN_BIAS;
   const int nt = (T_ + TQW - 1) / TQW;
   // blocks go round-robin over the 8 XCDs: keep the tiles of one (b,h) on one XCD (they walk the
-  // same K and V in step, so its L2 serves all but the first), long tiles first
+  // same K and V in step, so its L2 serves all but the first), long tiles first.  The tile with
+  // the last time step keeps the content term at every key step and runs about twice as long as
+  // the next one: all of those go first, or the last of them would end the launch alone.
   const int nbh = a.B * a.H;
   int bh, tile;
   {
     const int L = blockIdx.x;
-    if ((nbh & 7) == 0) {
-      const int s = L >> 3;
-      bh = (L & 7) + 8 * (s / nt);
-      tile = nt - 1 - s % nt;
+    if (nt == 1) {
+      bh = L;
+      tile = 0;
+    } else if (L < nbh) {
+      bh = L;
+      tile = nt - 1;
+    } else if ((nbh & 7) == 0) {
+      const int s = (L - nbh) >> 3;
+      bh = ((L - nbh) & 7) + 8 * (s / (nt - 1));
+      tile = nt - 2 - s % (nt - 1);
     } else {
-      bh = L / nt;
-      tile = nt - 1 - L % nt;
+      bh = (L - nbh) / (nt - 1);
+      tile = nt - 2 - (L - nbh) % (nt - 1);
     }
   }
   const int b = bh / a.H, h = bh % a.H;
@@ -358,17 +366,22 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
   // the key pass (the exponent e = time bias - L + mc for pairs inside the window, else exp2(e))
   auto flush_slab = [&](int tks) {
     const int nj = min(32, tq - tks + 1);
-    if (hh == 0 && qok) {
-      for (int jj = 0; jj < nj; ++jj) {
-        const int tkk = tks + jj;
-        const float e = Stb[jj * 32 + ln] - lse + mc;
-        const bool near_pair = has_content && (W <= 0 || tq - tkk <= W || tq == T_ - 1);
-        a.ws_time[(((int64_t)bh * T_ + tq) * T_ + tkk) * C_ + cq] = near_pair ? e : __builtin_amdgcn_exp2f(e);
-      }
+    // fixed trip counts with predicates: the LDS reads of several iterations go out together
+#pragma unroll 8
+    for (int it = 0; it < 16; ++it) {
+      const int jj = 2 * it + hh, tkk = tks + jj;
+      const float e = Stb[jj * 32 + ln] - lse + mc;
+      const bool near_pair = has_content && (W <= 0 || tq - tkk <= W || tq == T_ - 1);
+      const float val = near_pair ? e : __builtin_amdgcn_exp2f(e);
+      if (qok && jj < nj) a.ws_time[(((int64_t)bh * T_ + tq) * T_ + tkk) * C_ + cq] = val;
     }
     const int j0 = time_row(tq, tks, T_);
-    for (int q = hh; q < nq_live; q += 2)
-      if (ln < nj) a.dbias_time[(wrow0 + q) * T_ + j0 + ln] = Gtb[ln * GP + q];
+#pragma unroll 8
+    for (int it = 0; it < 16; ++it) {
+      const int q = 2 * it + hh;
+      const float g = Gtb[ln * GP + q];
+      if (q < nq_live && ln < nj) a.dbias_time[(wrow0 + q) * T_ + j0 + ln] = g;
+    }
   };
 
   int stage = 0;
@@ -406,12 +419,15 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
       for (int i = 0; i < 16; ++i) stc[i] = 0.f;
       if (has_time) {
         const int j = min(time_row(tq, tk, T_) + ln, T_ - 1);
+        u32x4 rr[KS], qr[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const u32x4 rr = *(const u32x4*)(ktime + (int64_t)j * DH + ks * 16 + hh * 8);
-          const bf16x8 qv = qfrag(*(const u32x4*)(qrow + ks * 16 + hh * 8), bv + ks * 16 + hh * 8, sc2);
-          stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(rr), qv, stc, 0, 0, 0);
+        for (int ks = 0; ks < KS; ++ks) {         // every load before the first use
+          rr[ks] = *(const u32x4*)(ktime + (int64_t)j * DH + ks * 16 + hh * 8);
+          qr[ks] = *(const u32x4*)(qrow + ks * 16 + hh * 8);
         }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(rr[ks]), qfrag(qr[ks], bv + ks * 16 + hh * 8, sc2), stc, 0, 0, 0);
       }
 #pragma unroll
       for (int i = 0; i < 16; ++i) Stb[((i >> 2) * 8 + hh * 4 + (i & 3)) * 32 + ln] = stc[i];
@@ -567,26 +583,28 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
             make_float4(dq[mt][a4 * 4], dq[mt][a4 * 4 + 1], dq[mt][a4 * 4 + 2], dq[mt][a4 * 4 + 3]);
   }
 
-  // channel-table gradient: element (ck) of query cq goes to column C-1-|cq-ck|; the two key
-  // channels at the same distance add up.  Per-wave table [32 queries][PC] in the scratch.
+  // channel-table gradient: element (ck) of query cq goes to column C-1-|cq-ck|, so column
+  // C-1-d collects the two key channels cq-d and cq+d.  The tile goes to a per-wave table
+  // [32 queries][PC] by key channel, and each output row is gathered from it (LDS float atomics
+  // for the scatter form were measured at ~0.3 us apiece).
   wave_sync_lds();
-  for (int i = lane; i < 32 * PC; i += 64) scr[i] = 0.f;
+#pragma unroll
+  for (int t = 0; t < NCT; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) scr[ln * PC + t * 32 + (i >> 2) * 8 + hh * 4 + (i & 3)] = dSc[t][i];
   wave_sync_lds();
   {
-    const uint32_t cq4 = (uint32_t)(cq - 4 * hh + 4);
-#pragma unroll
-    for (int t = 0; t < NCT; ++t)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const uint32_t ci4 = (uint32_t)(t * 32 + (i >> 2) * 8 + (i & 3) + 4);
-        const uint32_t dist = max(cq4, ci4) - min(cq4, ci4);
-        const bool kv = (kbits[t] >> ((i >> 2) * 8 + (i & 3))) & 1u;
-        if (kv && dist < (uint32_t)C_ && qok) atomicAdd(&scr[ln * PC + (C_ - 1 - (int)dist)], dSc[t][i]);
-      }
+    const int d = C_ - 1 - lane;                  // this lane's column holds distance d
+#pragma unroll 8
+    for (int q = 0; q < 32; ++q) {
+      const int lo = cq0 + q - d, hi = cq0 + q + d;
+      float g = scr[q * PC + max(0, min(lo, CP - 1))];
+      const float g2 = scr[q * PC + max(0, min(hi, CP - 1))];
+      if (lo < 0 || d < 0) g = 0.f;
+      if (d > 0 && hi < C_) g += g2;
+      if (q < nq_live && lane < C_) a.dbias_chan[(wrow0 + q) * C_ + lane] = g;
+    }
   }
-  wave_sync_lds();
-  for (int q = 0; q < nq_live; ++q)
-    if (lane < C_) a.dbias_chan[(wrow0 + q) * C_ + lane] = scr[q * PC + lane];
 }
 
 }  // namespace bwdq
