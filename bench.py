@@ -96,6 +96,7 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-model", action="store_true", help="skip the MVPFormer-S forward leg")
+    ap.add_argument("--no-backward", action="store_true", help="skip the MVPA backward leg")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 256 MiB device copy (calibrates HBM traffic counters)")
     args = ap.parse_args()
@@ -159,6 +160,28 @@ def main():
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "kernel": "mvpa_mfma_kernel",
                      "kernel_ms": round(kern_ms, 4)},
     }
+    if not args.no_backward and C <= 64 and C % 4 == 0:   # shapes the matrix-core backward serves
+        # the backward of the same workload (reported beside the headline, never part of `value`):
+        # both passes of mvpa_backward, gradients and workspace allocated outside the timed region
+        # by torch's caching allocator after the first call
+        _, lse = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
+                                       chan_valid=d.chan_valid, return_lse=True)
+        d_o = torch.randn_like(out)
+
+        def bwd():
+            return mvpa_hip.mvpa_backward(d.q, d.k, d.v, out, d_o, lse, d.u, d.vb, d.z, d.k_time,
+                                          d.k_chan, chan_valid=d.chan_valid)
+        n_bwd = max(1, min(args.steps, 10))
+        bwd()
+        torch.cuda.synchronize()
+        ev0.record()
+        for _ in range(n_bwd):
+            bwd()
+        ev1.record()
+        torch.cuda.synchronize()
+        line["backward"] = {"ms_per_step": round(ev0.elapsed_time(ev1) / n_bwd, 4), "steps": n_bwd,
+                            "kernels": "mvpa_bwd_query_mfma_kernel + mvpa_bwd_key_mfma_kernel",
+                            "outputs": "dq (content share), dk, dv, dbias_time, dbias_chan (fp32)"}
     if not args.no_model:
         try:
             from models.bench_model import mvpformer_s_windows_per_s

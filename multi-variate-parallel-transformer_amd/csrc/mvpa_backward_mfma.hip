@@ -237,6 +237,30 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
         Bc[t][i] = kv ? val : -INFINITY;
       }
   };
+  // every global load of the set-up goes out before the first use: one round trip, not one per
+  // fragment.  The log-sum-exp is among them so that its wait does not fall into the loops, where
+  // it would drain the whole ring (vmcnt 0) at every key step.
+  u32x4 raw_[KS], draw_[KS], oraw_[KS], er_[KS][NCT];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d0 = ks * 16 + hh * 8;
+    raw_[ks] = *(const u32x4*)(qrow + d0);
+    draw_[ks] = *(const u32x4*)(drow + d0);
+    oraw_[ks] = *(const u32x4*)(orow + d0);
+#pragma unroll
+    for (int t = 0; t < NCT; ++t)
+      er_[ks][t] = *(const u32x4*)(kchan + (int64_t)min(t * 32 + ln, C_ - 1) * DH + d0);
+  }
+  const float lse = a.lse[row];
+  uint64_t kmask[2];
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    const int ck = w * 64 + lane;
+    bool ok = ck < C_;
+    if (valid) ok = ok && valid[min(ck, C_ - 1)] != 0;
+    kmask[w] = __ballot(ok);
+  }
+  asm volatile("" :: "v"(lse));
   {
     f32x16 sct[NCT];
 #pragma unroll
@@ -246,9 +270,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d0 = ks * 16 + hh * 8;
-      const u32x4 raw = *(const u32x4*)(qrow + d0);
-      const u32x4 draw = *(const u32x4*)(drow + d0);
-      const u32x4 oraw = *(const u32x4*)(orow + d0);
+      const u32x4 raw = raw_[ks], draw = draw_[ks], oraw = oraw_[ks];
       if (qok) *(bf16x8*)((bf16_t*)a.ws_qu + row * DH + d0) = qfrag(raw, bu + d0, sc2);   // for the key pass
       const bf16x8 qz = qfrag(raw, bz + d0, sc2);
       dOf[ks] = as_frag(draw);
@@ -258,11 +280,8 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
         delta += __uint_as_float(draw[i] & 0xffff0000u) * __uint_as_float(oraw[i] & 0xffff0000u);
       }
 #pragma unroll
-      for (int t = 0; t < NCT; ++t) {
-        const int j = min(t * 32 + ln, C_ - 1);
-        const u32x4 er = *(const u32x4*)(kchan + (int64_t)j * DH + d0);
-        sct[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(er), qz, sct[t], 0, 0, 0);
-      }
+      for (int t = 0; t < NCT; ++t)
+        sct[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(er_[ks][t]), qz, sct[t], 0, 0, 0);
     }
     delta = xhalf_sum(delta);
 #pragma unroll
@@ -272,14 +291,6 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
         const int j = t * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
         scr[j * 32 + ln] = has_chan ? sct[t][i] : 0.f;
       }
-    uint64_t kmask[2];
-#pragma unroll
-    for (int w = 0; w < 2; ++w) {
-      const int ck = w * 64 + lane;
-      bool ok = ck < C_;
-      if (valid) ok = ok && valid[min(ck, C_ - 1)] != 0;
-      kmask[w] = __ballot(ok);
-    }
 #pragma unroll
     for (int t = 0; t < NCT; ++t) kbits[t] = (uint32_t)(kmask[t >> 1] >> ((t & 1) * 32 + 4 * hh));
     wave_sync_lds();
@@ -319,10 +330,6 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
     }
     if (qok && hh == 0) a.ws_delta[row] = delta;
   }
-  const float lse = a.lse[row];
-  // consumed here so that the wait for this load stands in front of the loops: left to the first
-  // use inside them, it would drain the whole ring (vmcnt 0) at every key step
-  asm volatile("" :: "v"(lse));
 
   f32x16 dq[MT], dSc[NCT];
 #pragma unroll
