@@ -657,7 +657,7 @@ int mvpa_launch_bwd_query_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
 }
 
 // ==========================================================================================
-// The KEY pass: dk, dv.  A workgroup owns NW / NCT consecutive key time steps of one kv head; a
+// The KEY pass: dk, dv.  A workgroup owns 4 consecutive key time steps of one kv head; a
 // wave owns 32 key channels of one of them (its K and V rows stay in registers as MFMA B
 // operands) and walks every query time step tq >= tk of every query head of the group, both
 // query-channel tiles in turn.  Products are formed NON-transposed here, S[q][key] = (q+u) K^T,
@@ -678,8 +678,14 @@ int mvpa_launch_bwd_query_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
 namespace mvpa {
 namespace bwdq {
 
+// waves per workgroup of the key pass: every wave of a workgroup reads the same stage (only the
+// per-key-step scalars differ), so with two channel tiles 8 waves (4 key steps) share it and each
+// SIMD holds two waves
+template <int NCT> constexpr int KEY_WAVES = NCT == 2 ? 8 : 4;
+
 template <int NCT, bool MASKED>
-__global__ __launch_bounds__(NW * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_args a) {
+__global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_args a) {
+  constexpr int NW = KEY_WAVES<NCT>;              // shadows the query pass's wave count
   constexpr int CP = NCT * 32, KT = NW / NCT, TILE = CP * ROWB;
   constexpr int CS_BYTES = CP * CP * 4, SC_BYTES = (KT + 1) * 256;
   constexpr int STAGES = KSTAGES, STAGE_BYTES = 4 * TILE + CS_BYTES + SC_BYTES;
@@ -949,12 +955,12 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_arg
 template <int NCT, bool MASKED>
 static void launch_key(const mvpa_bwd_args* a, hipStream_t stream) {
   using namespace mvpa::bwdq;
-  constexpr int cp = NCT * 32, kt = NW / NCT;
+  constexpr int nw = KEY_WAVES<NCT>, cp = NCT * 32, kt = nw / NCT;
   const size_t lds = (size_t)KSTAGES * (4 * cp * ROWB + cp * cp * 4 + (kt + 1) * 256);
   dim3 grid((unsigned)(((a->T + kt - 1) / kt) * a->B * a->Hkv));
   auto kern = mvpa_bwd_key_mfma_kernel<NCT, MASKED>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, *a);
+  hipLaunchKernelGGL(kern, grid, dim3(nw * 64), lds, stream, *a);
 }
 
 int mvpa_launch_bwd_key_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
