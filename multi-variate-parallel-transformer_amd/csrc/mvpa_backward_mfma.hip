@@ -35,8 +35,12 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 constexpr int DH = 64, KS = 4, MT = 2, ROWB = 128, NW = 4;
 constexpr int QSTAGES = 3, KSTAGES = 3;          // ring depth of the query / key pass
-// floats of per-wave scratch in the query pass: two time-bias slabs and the channel table
-template <int NCT> constexpr int WAVE_SCRATCH = 1024 + 32 * 33 + 32 * (NCT * 32 + 1);
+// waves per workgroup of the query pass: with two channel tiles 8 waves (4 query time steps) share
+// the K/V ring and each SIMD holds two waves
+template <int NCT> constexpr int QUERY_WAVES = NCT == 2 ? 8 : 4;
+// floats of per-wave scratch in the query pass: the two time-bias slabs [32][32] + [32][33]; the
+// channel tables of the set-up ([32 NCT][32]) and of the epilogue ([32][32 NCT + 1]) overlay them
+constexpr int WAVE_SCRATCH = 1024 + 32 * 33;
 
 __device__ inline void wave_sync_lds() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -116,8 +120,10 @@ __device__ inline int swz_row(int row) { return (row >> 1) & 7; }
 __device__ inline int swz_tr(int row) { return ((row >> 1) & 1) << 2; }
 
 template <int NCT>
-__global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_args a) {
+__global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_args a) {
+  constexpr int NW = QUERY_WAVES<NCT>;
   constexpr int CP = NCT * 32, TQW = NW / NCT, TILE = CP * ROWB;
+  static_assert(CP * 32 <= WAVE_SCRATCH && 32 * (CP + 1) <= WAVE_SCRATCH, "channel tables overlay the slabs");
   constexpr int STAGES = QSTAGES, STAGE_BYTES = 3 * TILE;   // stage: V | K | K (transposing)
   constexpr int LPW = CP / 8 / NW;                // 1 KiB wave loads per wave and tile copy
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -127,9 +133,9 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 31, hh = lane >> 5;
   constexpr int GP = 33, PC = CP + 1;             // padded pitches: the transposed reads spread over the banks
-  float* Stb = wave_base + wave * WAVE_SCRATCH<NCT>;      // [32][32] time-bias scores of a slab
+  float* Stb = wave_base + wave * WAVE_SCRATCH;           // [32][32] time-bias scores of a slab
   float* Gtb = Stb + 1024;                                // [32][GP] their gradients
-  float* scr = Gtb + 32 * GP;                             // [CP][32] channel table, later [32][PC]
+  float* scr = Stb;       // before the first slab [CP][32] channel table, after the last one [32][PC]
 
   const int T_ = a.T, C_ = a.C, W = a.window, N = a.T * a.C;
   const bool has_content = a.flags & MVPA_FLAG_CONTENT;
@@ -498,45 +504,37 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
   auto near_step = [&](const unsigned char* Vrow, int tk) {
     const unsigned char* Krow = Vrow + TILE;
     const unsigned char* Ktr = Vrow + 2 * TILE;
-    const float st = Stb[(tk & 31) * 32 + ln];
-    f32x16 S[NCT], dP[NCT];
-#pragma unroll
-    for (int t = 0; t < NCT; ++t) {
-      S[t] = Bc[t];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) dP[t][i] = 0.f;
-    }
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-      for (int t = 0; t < NCT; ++t) {
-        const int off = r_lane[ks] + t * 32 * ROWB;
-        S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Krow + off), Qu[ks], S[t], 0, 0, 0);
-        dP[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Vrow + off), dOf[ks], dP[t], 0, 0, 0);
-      }
-    const float off2 = st - lse;
+    const float off2 = Stb[(tk & 31) * 32 + ln] - lse;
     float gt = 0.f;
 #pragma unroll
-    for (int t = 0; t < NCT; ++t)
+    for (int t = 0; t < NCT; ++t) {               // one key-channel tile at a time: fewer live tiles
+      f32x16 S = Bc[t], dP;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) dP[i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int off = r_lane[ks] + t * 32 * ROWB;
+        S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Krow + off), Qu[ks], S, 0, 0, 0);
+        dP = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(Vrow + off), dOf[ks], dP, 0, 0, 0);
+      }
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const float p = __builtin_amdgcn_exp2f(S[t][i] + off2);     // masked keys: exp2(-inf) = 0
-        const float ds = p * (dP[t][i] - delta) * a.sm_scale;
-        S[t][i] = ds;
+        const float p = __builtin_amdgcn_exp2f(S[i] + off2);        // masked keys: exp2(-inf) = 0
+        const float ds = p * (dP[i] - delta) * a.sm_scale;
+        S[i] = ds;
         dSc[t][i] += ds;
         gt += ds;
       }
-    gt = xhalf_sum(gt);
-    if (hh == 0) Gtb[(tk & 31) * GP + ln] = gt;
-#pragma unroll
-    for (int t = 0; t < NCT; ++t)
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        const bf16x8 dsf = pack8(S[t], 8 * s);
+        const bf16x8 dsf = pack8(S, 8 * s);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
           dq[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Ktr, t, s, mt), dsf, dq[mt], 0, 0, 0);
       }
+    }
+    gt = xhalf_sum(gt);
+    if (hh == 0) Gtb[(tk & 31) * GP + ln] = gt;
   };
 
   // far steps first (none for the last time step, whose queries keep the content term everywhere),
@@ -563,7 +561,12 @@ __global__ __launch_bounds__(NW * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_a
   for (int t = 0; t < NCT; ++t)
 #pragma unroll
     for (int i = 0; i < 16; ++i) dSc[t][i] = Ec[t][i] * (dSc[t][i] - delta * esum);
-  gather_bc(Bc);
+  // Bc = mc + log2(Ec): the table it was gathered from lies under the slabs by now (-inf where
+  // Ec = 0: masked keys, and biases more than 126 octaves below the row's largest)
+#pragma unroll
+  for (int t = 0; t < NCT; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) Bc[t][i] = mc + __builtin_amdgcn_logf(Ec[t][i]);
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
     Qu[ks] = qfrag(*(const u32x4*)(qrow + ks * 16 + hh * 8), bu + ks * 16 + hh * 8, sc2);
@@ -638,20 +641,20 @@ int mvpa_bwd_query_mfma_supported(const mvpa_bwd_args* a) {
 int mvpa_launch_bwd_query_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
   using namespace mvpa::bwdq;
   const int nct = a->C <= 32 ? 1 : 2;
-  const int tqw = NW / nct;
+  const int nw = nct == 1 ? QUERY_WAVES<1> : QUERY_WAVES<2>;
+  const int tqw = nw / nct;
   const int nt = (a->T + tqw - 1) / tqw;
   const int cp = nct * 32;
-  const size_t lds = (size_t)QSTAGES * 3 * cp * ROWB +
-                     (size_t)NW * (nct == 1 ? WAVE_SCRATCH<1> : WAVE_SCRATCH<2>) * sizeof(float);
+  const size_t lds = (size_t)QSTAGES * 3 * cp * ROWB + (size_t)nw * WAVE_SCRATCH * sizeof(float);
   dim3 grid((unsigned)(nt * a->B * a->H));
   if (nct == 1) {
     auto kern = mvpa_bwd_query_mfma_kernel<1>;
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, *a);
+    hipLaunchKernelGGL(kern, grid, dim3(nw * 64), lds, stream, *a);
   } else {
     auto kern = mvpa_bwd_query_mfma_kernel<2>;
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, *a);
+    hipLaunchKernelGGL(kern, grid, dim3(nw * 64), lds, stream, *a);
   }
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
