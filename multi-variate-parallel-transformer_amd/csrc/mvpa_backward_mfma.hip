@@ -764,30 +764,43 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
   auto wg_near = [&](int tq) -> bool {
     return has_content && (W <= 0 || tq == T_ - 1 || tq - tk0 <= W + KT - 1);
   };
-  auto issue_step = [&](int hq, int tq, int stage_idx) {
+  // source pointers of the step the ring fetches next: re-based at each head, stepped down by
+  // one query time step otherwise (the full address arithmetic per step cost as many scalar
+  // instructions as a far step has vector ones)
+  const bf16_t* p_do = nullptr;
+  const bf16_t* p_qu = nullptr;
+  const float* p_ec = nullptr;
+  const float* p_sc = nullptr;
+  const float* p_de = nullptr;
+  const int64_t d_do = (int64_t)C_ * a.do_stride_n, d_sc = (int64_t)T_ * C_;
+  const int d_ec = C_ * C_, d_qu = C_ * DH;
+  auto rebase = [&](int hq) {
     const int h = g * grp + hq;
     const int64_t bhq = (int64_t)b * a.H + h;
-    const int64_t r0 = bhq * N + (int64_t)tq * C_;          // first query row of the step
+    const int64_t r0 = bhq * N + (int64_t)(T_ - 1) * C_;    // first query row of step T-1
+    p_do = (const bf16_t*)a.d_o + b * a.do_stride_b + h * a.do_stride_h + (int64_t)(T_ - 1) * d_do;
+    p_qu = (const bf16_t*)a.ws_qu + r0 * DH;
+    p_ec = a.ws_chan + r0 * C_;
+    p_sc = a.ws_time + ((bhq * T_ + (T_ - 1)) * T_ + tkc) * C_;
+    p_de = a.ws_delta + r0;
+  };
+  auto issue_step = [&](int tq, int stage_idx) {
     const uint32_t st = ring_lds + stage_idx * STAGE_BYTES;
-    const bf16_t* dsrc = (const bf16_t*)a.d_o + b * a.do_stride_b + h * a.do_stride_h +
-                         (int64_t)tq * C_ * a.do_stride_n;
-    const float* csrc = a.ws_chan + r0 * C_;
 #pragma unroll
-    for (int i = 0; i < LPW; ++i) dma16(dsrc + d_off_t[i], st + OFF_DTR + (wave + NW * i) * 1024);
+    for (int i = 0; i < LPW; ++i) dma16(p_do + d_off_t[i], st + OFF_DTR + (wave + NW * i) * 1024);
 #pragma unroll
-    for (int i = 0; i < CS_LPW; ++i) dma16(csrc + cs_off[i], st + OFF_EC + (wave + NW * i) * 1024);
+    for (int i = 0; i < CS_LPW; ++i) dma16(p_ec + cs_off[i], st + OFF_EC + (wave + NW * i) * 1024);
     // per-query scalar of this wave's key step
-    dma4(a.ws_time + ((bhq * T_ + tq) * T_ + tkc) * C_ + sc_lane, st + OFF_SC + ktw * 256);
+    dma4(p_sc + sc_lane, st + OFF_SC + ktw * 256);
     if (wg_near(tq)) {
-      const bf16_t* qsrc = (const bf16_t*)a.ws_qu + r0 * DH;
 #pragma unroll
       for (int i = 0; i < LPW; ++i) {
         const uint32_t dst = st + (wave + NW * i) * 1024;
-        dma16(dsrc + d_off_r[i], dst + OFF_DROW);
-        dma16(qsrc + q_off_r[i], dst + OFF_QROW);
-        dma16(qsrc + q_off_t[i], dst + OFF_QTR);
+        dma16(p_do + d_off_r[i], dst + OFF_DROW);
+        dma16(p_qu + q_off_r[i], dst + OFF_QROW);
+        dma16(p_qu + q_off_t[i], dst + OFF_QTR);
       }
-      dma4(a.ws_delta + r0 + sc_lane, st + OFF_SC + KT * 256);
+      dma4(p_de + sc_lane, st + OFF_SC + KT * 256);
     }
   };
 
@@ -817,12 +830,22 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
   // steps: query heads of the group, and for each the query steps T-1 .. tk0
   const int span = T_ - tk0, nsteps = grp * span;
   int ihq = 0, itq = T_ - 1;                      // the step the ring fetches next
+  rebase(0);
   auto next_issue = [&]() {
-    if (--itq < tk0) { itq = T_ - 1; ++ihq; }
+    if (--itq < tk0) {
+      itq = T_ - 1;
+      if (++ihq < grp) rebase(ihq);
+    } else {
+      p_do -= d_do;
+      p_qu -= d_qu;
+      p_ec -= d_ec;
+      p_sc -= d_sc;
+      p_de -= C_;
+    }
   };
 #pragma unroll
   for (int s = 0; s < STAGES - 1; ++s)
-    if (s < nsteps) { issue_step(ihq, itq, s); next_issue(); }
+    if (s < nsteps) { issue_step(itq, s); next_issue(); }
 
   int stage = 0, it = 0, ring_tq = T_ - 1;        // ring_tq: query step of the stage handed out next
   // advances the ring by one step and returns the stage that holds its data
@@ -833,7 +856,7 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
     else if (wg_near(next_tq)) wait_vmcnt_imm<LPS_NEAR>();
     else wait_vmcnt_imm<LPS_FAR>();
     lds_barrier();            // this step's stage visible to all; the previous one is free
-    if (it + STAGES - 1 < nsteps) { issue_step(ihq, itq, stage == 0 ? STAGES - 1 : stage - 1); next_issue(); }
+    if (it + STAGES - 1 < nsteps) { issue_step(itq, stage == 0 ? STAGES - 1 : stage - 1); next_issue(); }
     const unsigned char* base = smem + stage * STAGE_BYTES;
     stage = stage + 1 == STAGES ? 0 : stage + 1;
     ring_tq = next_tq;
