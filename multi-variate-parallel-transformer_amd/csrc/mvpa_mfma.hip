@@ -221,7 +221,13 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   // every key step (no far steps at all), which makes it several times longer than any other
   // workgroup, and it must not be what the rest of the grid ends up waiting for.  After those,
   // within a (b, h) the latest (= longest) time tiles are issued first.
-  const int nt = (T_ + G::TQW - 1) / G::TQW;
+  // SPLIT (two query time steps per workgroup, ring of 4): the last time step gets a workgroup
+  // of its own, both pairs of waves on tq = T-1; the ring then advances two key steps per
+  // barrier, one pair of waves takes the even and the other the odd one at the same time, and the
+  // two partial soft-max states are merged through LDS at the end.  That workgroup is the critical
+  // path of a launch (content term at every key step), and this halves it.
+  constexpr bool SPLIT = G::TQW == 2 && STAGES == 4;
+  const int nt = SPLIT ? 1 + T_ / 2 : (T_ + G::TQW - 1) / G::TQW;
   const int nbh = a.B * a.H;
   constexpr int TAIL_MERGE = 2;
   int bh, tile;
@@ -265,10 +271,12 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   }
   const int b = bh / a.H, h = bh % a.H;
   const int g = h / (a.H / a.Hkv);
-  const int tq0 = tile * G::TQW;
-  const int tq_hi = min(T_ - 1, tq0 + G::TQW - 1);
-  const int tq = tq0 + wave / NCT;
-  const bool active = tq < T_;
+  const bool split_last = SPLIT && tile == nt - 1;
+  const int par = wave / NCT;                      // split_last: parity of this wave's key steps
+  const int tq0 = split_last ? T_ - 1 : tile * G::TQW;
+  const int tq_hi = split_last ? T_ - 1 : min(T_ - 1 - (SPLIT ? 1 : 0), tq0 + G::TQW - 1);
+  const int tq = split_last ? T_ - 1 : tq0 + wave / NCT;
+  const bool active = tq <= tq_hi;
   const int cq = (wave % NCT) * 32 + ln;           // this lane's query channel
   const bool qok = active && cq < C_;
 
@@ -625,6 +633,34 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
           acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(stage, t, s, mt), P[t][s], acc[mt], 0, 0, 0);
   };
 
+  // =========================== split last time step: two key steps per barrier ===============
+  // Tile t lives in stage t % 4.  The prologue has tiles 0..2 in flight; at the barrier of pair k
+  // the stages of pair k-1 are free and receive pair k+1 (tile 3 alone at k = 0), which then has
+  // the whole pair k to arrive: one wait for everything outstanding in front of each barrier.
+  if (split_last) {
+    for (int k2 = 0; k2 <= T_ - 1; k2 += 4) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int t0 = k2 + 2 * u;                 // first tile of this pair, stage 2u
+        if (t0 > T_ - 1) break;                    // uniform over the workgroup
+        wait_vmcnt_imm<0>();
+        lds_barrier();
+        if (t0 == 0) {
+          if (3 <= T_ - 1) issue_tile(3, 3, 3 >= tk_near);
+        } else {
+          if (t0 + 2 <= T_ - 1) issue_tile(t0 + 2, 2 - 2 * u, t0 + 2 >= tk_near);
+          if (t0 + 3 <= T_ - 1) issue_tile(t0 + 3, 3 - 2 * u, t0 + 3 >= tk_near);
+        }
+        if ((t0 & 31) == 0) time_slab(t0);
+        const int tkw = t0 + par;
+        if (tkw <= T_ - 1) {
+          const unsigned char* stage = smem_raw + (2 * u) * G::STAGE_BYTES + par * G::STAGE_BYTES;
+          if (is_far(tkw)) far_step(stage, tkw);
+          else near_step(stage, tkw);
+        }
+      }
+    }
+  } else {
   // =========================== phase A: far tiles for every wave ===========================
   // Key steps below tk_near are far for all queries of the workgroup and only V is in flight, so
   // the number of younger loads is a compile-time constant.  The loop is unrolled over the ring so
@@ -717,8 +753,35 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
       }
     }
   }
+  }   // !split_last
 
   // =========================== epilogue ===========================
+  if (split_last) {
+    // merge the odd key steps' state (waves with par = 1) into the even ones': m, l and the
+    // accumulator tiles of every lane
+    lds_barrier();                                 // every wave is done with the ring
+    float* mb = (float*)smem_raw + (wave % NCT) * ((2 + MT * 16) * 64) + lane;
+    if (par == 1) {
+      mb[0] = m_run;
+      mb[64] = l_run;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mb[(2 + mt * 16 + i) * 64] = acc[mt][i];
+    }
+    lds_barrier();
+    if (par == 1) return;
+    const float m1 = mb[0], l1 = mb[64];
+    const float m = fmaxf(m_run, m1);
+    const float a0 = m_run == -INFINITY ? 0.f : fast_exp2(m_run - m);
+    const float a1 = m1 == -INFINITY ? 0.f : fast_exp2(m1 - m);
+    m_run = m;
+    l_run = a0 * l_run + a1 * l1;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mt][i] = a0 * acc[mt][i] + a1 * mb[(2 + mt * 16 + i) * 64];
+  }
   {
     const float ltot = l_run + __shfl_xor(l_run, 32);
     if (qok) {
@@ -748,7 +811,7 @@ static int launch_one(const mvpa_fwd_args* a, hipStream_t stream) {
   auto kern = mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)G::LDS_BYTES);
-  const int nt = (a->T + G::TQW - 1) / G::TQW;
+  const int nt = (G::TQW == 2 && STAGES == 4) ? 1 + a->T / 2 : (a->T + G::TQW - 1) / G::TQW;   // as in the kernel
   dim3 grid((unsigned)(nt * a->B * a->H));
   hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), G::LDS_BYTES, stream, *a);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
@@ -791,7 +854,7 @@ int mvpa_launch_mfma(const mvpa_fwd_args* a, hipStream_t stream) {
       return launch_cfg<32, 4, 4, 4>(a, stream);
     case 64:
       if (nct == 1) return launch_cfg<64, 1, 8, 4>(a, stream);
-      if (nct == 2) return launch_cfg<64, 2, 4, 3, 2>(a, stream);   // two workgroups per CU
+      if (nct == 2) return launch_cfg<64, 2, 4, 4, 2>(a, stream);   // two workgroups per CU (2 x 80 KiB)
       return launch_cfg<64, 4, 4, 3>(a, stream);
     case 128:
       if (nct == 1) return launch_cfg<128, 1, 4, 4>(a, stream);
