@@ -28,7 +28,7 @@ BF16_DENSE_PEAK_TFLOPS = 2500.0       # MI355X published dense bf16 MFMA peak
 
 # HBM bytes per launch of the attention kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by
 # what the same counters read for a plain 256 MiB copy (profiles/mvpa_mfma_kernel_c2.md).
-MEASURED_TRAFFIC_BYTES = {"c2": 397.8e6}
+MEASURED_TRAFFIC_BYTES = {"c2": 402.4e6}
 
 WORKLOADS = {
     "c2": dict(B=4, C=64, T=128, H=16, Hkv=16, Dh=64, validity=False),
