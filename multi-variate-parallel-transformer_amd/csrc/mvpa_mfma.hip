@@ -553,7 +553,10 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
       for (int i = 0; i < 16; ++i) acc[mt][i] += et * tmp[mt][i];
   };
 
-  // ---- near tile: S^T = K Q^T + Bc, online soft-max, acc += V^T P^T
+  // ---- near tile: S^T = K Q^T + Bc, online soft-max, acc += V^T P^T.  The key-channel tiles are
+  // taken one after the other (QK^T chains issued tile by tile, then per tile: row max, lazy
+  // rescale, exp2, PV), so that the matrix cores work on the next tile's QK^T / the previous
+  // tile's PV while this wave does the vector work of a tile.
   auto near_step = [&](const unsigned char* stage, int tk) {
     const float st = Stb[(tk & 31) * 32 + ln];
     f32x16 S[NCT];
@@ -561,14 +564,14 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     for (int t = 0; t < NCT; ++t) S[t] = Bc[t];
     if (FP8) {
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
+      for (int t = 0; t < NCT; ++t)
 #pragma unroll
-        for (int t = 0; t < NCT; ++t) {
+        for (int ks = 0; ks < KS; ++ks) {
           const u32x4 kr = *(const u32x4*)(stage + k_lane[ks] + t * 32 * ROWB);
           S[t] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(kfrag_fp8(kr, fp8_inv_sk), Qu8[ks], S[t], 0, 0, 0);
         }
     } else {
-      // every K fragment of the tile is requested before the first MFMA waits for one
+      // every K fragment of the step is requested before the first MFMA waits for one
       bf16x8 ka[KS][NCT];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
@@ -576,61 +579,57 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
         for (int t = 0; t < NCT; ++t) ka[ks][t] = *(const bf16x8*)(stage + k_lane[ks] + t * 32 * ROWB);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
+      for (int t = 0; t < NCT; ++t)
 #pragma unroll
-        for (int t = 0; t < NCT; ++t)
+        for (int ks = 0; ks < KS; ++ks)
           S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][t], Qu[ks], S[t], 0, 0, 0);
     }
-    float rmax = -INFINITY;
-#pragma unroll
-    for (int t = 0; t < NCT; ++t)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) rmax = fmaxf(rmax, S[t][i]);
-    rmax = xhalf_max(rmax);
-    if (FP8) rmax *= fp8_d;
-    // Lazy running max: the reference point only moves when some query's row max outgrew it by
-    // more than 2^8; until then probabilities are formed against the old reference (at most 256
-    // times larger, harmless in fp32/bf16) and the accumulator rescale is skipped altogether.
-    const float cand = rmax + st;
-    const bool grow = __ballot(cand > m_run + 8.f) != 0ull;
-    const float m_new = grow ? fmaxf(m_run, cand) : m_run;
-    const float off = st - m_new;
     float ls = 0.f;
-    bf16x8 P[NCT][2];
 #pragma unroll
     for (int t = 0; t < NCT; ++t) {
+      float rmax = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) rmax = fmaxf(rmax, S[t][i]);
+      rmax = xhalf_max(rmax);
+      if (FP8) rmax *= fp8_d;
+      // Lazy running max: the reference point only moves when some query's row max outgrew it by
+      // more than 2^8; until then probabilities are formed against the old reference (at most
+      // 256 times larger, harmless in fp32/bf16) and the accumulator rescale is skipped.
+      const float cand = rmax + st;
+      if (__ballot(cand > m_run + 8.f) != 0ull) {
+        const float m_new = fmaxf(m_run, cand);
+        const float alpha = fast_exp2(m_run - m_new);
+        m_run = m_new;
+        l_run *= alpha;
+        ls *= alpha;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[mt][i] *= alpha;
+      }
+      const float off = st - m_run;
 #pragma unroll
       for (int i = 0; i < 16; ++i)
         S[t][i] = FP8 ? fast_exp2(__builtin_fmaf(S[t][i], fp8_d, off)) : fast_exp2(S[t][i] + off);
-      P[t][0] = pack8(S[t], 0);
-      P[t][1] = pack8(S[t], 8);
+      bf16x8 P[2];
+      P[0] = pack8(S[t], 0);
+      P[1] = pack8(S[t], 8);
       // the row sum is taken over the bf16 probabilities the PV product uses, two per
       // instruction (v_dot2c_f32_bf16 against a pair of ones), accumulated in fp32
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         union { bf16x8 v; bf16x2 q[4]; } u;
-        u.v = P[t][s];
+        u.v = P[s];
 #pragma unroll
         for (int j = 0; j < 4; ++j) ls = __builtin_amdgcn_fdot2_f32_bf16(u.q[j], kOnes2, ls, false);
       }
-    }
-    if (grow) {
-      const float alpha = fast_exp2(m_run - m_new);
-      m_run = m_new;
-      l_run *= alpha;
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[mt][i] *= alpha;
-    }
-    l_run += ls;
-#pragma unroll
-    for (int t = 0; t < NCT; ++t)
 #pragma unroll
       for (int s = 0; s < 2; ++s)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-          acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(stage, t, s, mt), P[t][s], acc[mt], 0, 0, 0);
+          acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(stage, t, s, mt), P[s], acc[mt], 0, 0, 0);
+    }
+    l_run += ls;
   };
 
   // =========================== split last time step: two key steps per barrier ===============
