@@ -26,7 +26,7 @@ def build_mvpformer_s(seg: int = 512, device="cuda:0", seed: int = 0, n_layer=No
 
 
 def mvpformer_s_windows_per_s(B: int = 4, C: int = 64, T: int = 64, seg: int = 512,
-                              steps: int = 5, warmup: int = 2) -> dict:
+                              steps: int = 20, warmup: int = 10) -> dict:
     model = build_mvpformer_s(seg)
     x = make_ieeg(B, C, T, seg, seed=0).to("cuda:0")
     for _ in range(warmup):
