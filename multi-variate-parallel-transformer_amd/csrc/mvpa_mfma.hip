@@ -171,12 +171,17 @@ template <int DH> __device__ inline int swz_v(int row) {
   return DH == 64 ? (((row >> 1) & 1) << 2) : DH == 128 ? ((row & 3) << 2) : 0;
 }
 
-template <int DH, int NCT, int NW, int STAGES>
+// NCT = key-channel tiles a WAVE handles per key step; KH = parts the keys of a step are split
+// into (each part has its own waves, which keep a partial soft-max state over their keys and merge
+// at the end).  Queries and keys cover the same QT = NCT * KH tiles of 32 channels.
+template <int DH, int NCT, int NW, int STAGES, int KH = 1>
 struct Cfg {
-  static constexpr int CP = NCT * 32;          // padded channels per time step
+  static constexpr int QT = NCT * KH;          // 32-channel tiles per time step
+  static constexpr int CP = QT * 32;           // padded channels per time step (rows of a K/V tile)
+  static constexpr int WPT = QT * KH;          // waves per time step: query tiles x key parts
   static constexpr int KS = DH / 16;           // k-steps of the QK^T contraction
   static constexpr int MT = DH / 32;           // 32-row tiles of O^T
-  static constexpr int TQW = NW / NCT;         // time steps per workgroup
+  static constexpr int TQW = NW / WPT;         // time steps per workgroup
   static constexpr int THREADS = NW * 64;
   static constexpr int ROWB = DH * 2;          // bytes per K/V row
   static constexpr int CHUNKS = DH / 8;        // 16-byte chunks per row
@@ -191,14 +196,14 @@ struct Cfg {
   static constexpr int LDS_BYTES = MAIN_BYTES > SETUP_BYTES ? MAIN_BYTES : SETUP_BYTES;
   // the set-up scratch fits behind the stages of the prologue tiles
   static constexpr bool EARLY = STAGES >= 2 && SETUP_BYTES <= STAGE_BYTES + STB_BYTES;
-  static_assert(NW % NCT == 0, "waves must cover whole time steps");
+  static_assert(NW % WPT == 0, "waves must cover whole time steps");
   static_assert(TILE_BYTES % 1024 == 0, "tile must be a whole number of wave loads");
   static_assert(WLOADS % NW == 0 || WLOADS < NW, "every loading wave issues the same number of loads");
 };
 
-template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8>
+template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8, int KH>
 __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args a) {
-  using G = Cfg<DH, NCT, NW, STAGES>;
+  using G = Cfg<DH, NCT, NW, STAGES, KH>;
   constexpr int CP = G::CP, KS = G::KS, MT = G::MT, ROWB = G::ROWB, CHUNKS = G::CHUNKS;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   float* Stb_all = (float*)(smem_raw + G::RING_BYTES);          // [NW][32][32]
@@ -226,7 +231,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   // barrier, one pair of waves takes the even and the other the odd one at the same time, and the
   // two partial soft-max states are merged through LDS at the end.  That workgroup is the critical
   // path of a launch (content term at every key step), and this halves it.
-  constexpr bool SPLIT = G::TQW == 2 && STAGES == 4;
+  constexpr bool SPLIT = G::TQW == 2 && STAGES == 4 && KH == 1;
   const int nt = SPLIT ? 1 + T_ / 2 : (T_ + G::TQW - 1) / G::TQW;
   const int nbh = a.B * a.H;
   constexpr int TAIL_MERGE = 2;
@@ -272,12 +277,15 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   const int b = bh / a.H, h = bh % a.H;
   const int g = h / (a.H / a.Hkv);
   const bool split_last = SPLIT && tile == nt - 1;
-  const int par = wave / NCT;                      // split_last: parity of this wave's key steps
+  const int par = wave / G::WPT;                   // split_last: parity of this wave's key steps
+  const int kh = KH > 1 ? (wave / G::QT) % KH : 0; // the part of the keys this wave works on
+  const int key0 = kh * (NCT * 32);                // its first key channel
+  const int key_off = key0 * G::ROWB;              // ... as a byte offset into a K or V tile
   const int tq0 = split_last ? T_ - 1 : tile * G::TQW;
   const int tq_hi = split_last ? T_ - 1 : min(T_ - 1 - (SPLIT ? 1 : 0), tq0 + G::TQW - 1);
-  const int tq = split_last ? T_ - 1 : tq0 + wave / NCT;
+  const int tq = split_last ? T_ - 1 : tq0 + wave / G::WPT;
   const bool active = tq <= tq_hi;
-  const int cq = (wave % NCT) * 32 + ln;           // this lane's query channel
+  const int cq = (wave % G::QT) * 32 + ln;         // this lane's query channel
   const bool qok = active && cq < C_;
 
   // Loads below are unconditional: rows that do not exist (padded channels, time steps past the
@@ -359,9 +367,9 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     u32x4 raw[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) raw[ks] = *(const u32x4*)(qrow + ks * 16 + hh * 8);
-    f32x16 sct[NCT];
+    f32x16 sct[G::QT];       // the whole channel table (every distance), whatever the key part
 #pragma unroll
-    for (int t = 0; t < NCT; ++t)
+    for (int t = 0; t < G::QT; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i) sct[t][i] = 0.f;
 #pragma unroll
@@ -372,7 +380,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
       Qv[ks] = make_qfrag(raw[ks], bv + d0, sc2);
       const bf16x8 qz = make_qfrag(raw[ks], bz + d0, sc2);
 #pragma unroll
-      for (int t = 0; t < NCT; ++t) {
+      for (int t = 0; t < G::QT; ++t) {
         const int j = min(t * 32 + ln, C_ - 1);
         const u32x4 er = *(const u32x4*)(kchan + (int64_t)j * DH + d0);
         sct[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(er), qz, sct[t], 0, 0, 0);
@@ -380,7 +388,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     }
     float* scr = setup_all + wave * (CP * 32);
 #pragma unroll
-    for (int t = 0; t < NCT; ++t)
+    for (int t = 0; t < G::QT; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int j = t * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
@@ -400,7 +408,10 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
         kmask[w] = __ballot(ok);
       }
 #pragma unroll
-      for (int t = 0; t < NCT; ++t) kbits[t] = (uint32_t)(kmask[t >> 1] >> ((t & 1) * 32 + 4 * hh));
+      for (int t = 0; t < NCT; ++t) {
+        const int gt = kh * NCT + t;           // key tile within the time step
+        kbits[t] = (uint32_t)(kmask[gt >> 1] >> ((gt & 1) * 32 + 4 * hh));
+      }
     }
     wave_lds_sync();
     // Bc[ck][q] = scr[C-1-|cq-ck|][q].  With ck = c_i + 4hh (c_i a compile-time constant) the
@@ -413,7 +424,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     for (int t = 0; t < NCT; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const uint32_t ci4 = (uint32_t)(t * 32 + (i >> 2) * 8 + (i & 3) + 4);
+        const uint32_t ci4 = (uint32_t)(key0 + t * 32 + (i >> 2) * 8 + (i & 3) + 4);
         const uint32_t dist = min(max(cq4, ci4) - min(cq4, ci4), (uint32_t)(C_ - 1));
         const float val = *(const float*)(scr_b + (gbase - (int)(dist * 128u)));
         const bool kv = (kbits[t] >> ((i >> 2) * 8 + (i & 3))) & 1u;
@@ -697,7 +708,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
           time_slab(tk);
         }
         if (active) {
-          const unsigned char* stage = smem_raw + s * G::STAGE_BYTES;
+          const unsigned char* stage = smem_raw + s * G::STAGE_BYTES + key_off;
           const float st = Stb[(tk & 31) * 32 + ln];
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
@@ -746,7 +757,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
         issue_tile(tk + STAGES - 1, (s + STAGES - 1) % STAGES, tk + STAGES - 1 >= tk_near);
       if ((tk & 31) == 0 && active) time_slab(tk);
       if (active && tk <= tq) {
-        const unsigned char* stage = smem_raw + s * G::STAGE_BYTES;
+        const unsigned char* stage = smem_raw + s * G::STAGE_BYTES + key_off;
         if (is_far(tk)) far_step(stage, tk);
         else near_step(stage, tk);
       }
@@ -755,12 +766,15 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   }   // !split_last
 
   // =========================== epilogue ===========================
-  if (split_last) {
-    // merge the odd key steps' state (waves with par = 1) into the even ones': m, l and the
-    // accumulator tiles of every lane
+  if (split_last || KH > 1) {
+    // two waves hold partial soft-max states of the same queries (split last time step: even and
+    // odd key steps; KH = 2: the two parts of the key channels): the second one's m, l and
+    // accumulator tiles go through LDS into the first one's
     lds_barrier();                                 // every wave is done with the ring
-    float* mb = (float*)smem_raw + (wave % NCT) * ((2 + MT * 16) * 64) + lane;
-    if (par == 1) {
+    const int mpar = KH > 1 ? kh : par;
+    const int slot = KH > 1 ? (wave / G::WPT) * G::QT + wave % G::QT : wave % NCT;
+    float* mb = (float*)smem_raw + slot * ((2 + MT * 16) * 64) + lane;
+    if (mpar == 1) {
       mb[0] = m_run;
       mb[64] = l_run;
 #pragma unroll
@@ -769,7 +783,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
         for (int i = 0; i < 16; ++i) mb[(2 + mt * 16 + i) * 64] = acc[mt][i];
     }
     lds_barrier();
-    if (par == 1) return;
+    if (mpar == 1) return;
     const float m1 = mb[0], l1 = mb[64];
     const float m = fmaxf(m_run, m1);
     const float a0 = m_run == -INFINITY ? 0.f : fast_exp2(m_run - m);
@@ -803,23 +817,24 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   }
 }
 
-template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8>
+template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8, int KH>
 static int launch_one(const mvpa_fwd_args* a, hipStream_t stream) {
-  using G = Cfg<DH, NCT, NW, STAGES>;
+  using G = Cfg<DH, NCT, NW, STAGES, KH>;
+  static_assert(KH <= 2 && (KH == 1 || G::TQW * G::QT * (2 + G::MT * 16) * 256 <= G::RING_BYTES), "merge buffer");
   static_assert(G::LDS_BYTES <= 160 * 1024, "LDS budget");
-  auto kern = mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8>;
+  auto kern = mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)G::LDS_BYTES);
-  const int nt = (G::TQW == 2 && STAGES == 4) ? 1 + a->T / 2 : (a->T + G::TQW - 1) / G::TQW;   // as in the kernel
+  const int nt = (G::TQW == 2 && STAGES == 4 && KH == 1) ? 1 + a->T / 2 : (a->T + G::TQW - 1) / G::TQW;   // as in the kernel
   dim3 grid((unsigned)(nt * a->B * a->H));
   hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), G::LDS_BYTES, stream, *a);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 
-template <int DH, int NCT, int NW, int STAGES, int MINB = 1>
+template <int DH, int NCT, int NW, int STAGES, int MINB = 1, int KH = 1>
 static int launch_cfg(const mvpa_fwd_args* a, hipStream_t stream) {
-  if (a->flags & MVPA_FLAG_FP8_QK) return launch_one<DH, NCT, NW, STAGES, MINB, true>(a, stream);
-  return launch_one<DH, NCT, NW, STAGES, MINB, false>(a, stream);
+  if (a->flags & MVPA_FLAG_FP8_QK) return launch_one<DH, NCT, NW, STAGES, MINB, true, KH>(a, stream);
+  return launch_one<DH, NCT, NW, STAGES, MINB, false, KH>(a, stream);
 }
 
 }  // namespace mvpa
@@ -854,7 +869,9 @@ int mvpa_launch_mfma(const mvpa_fwd_args* a, hipStream_t stream) {
     case 64:
       if (nct == 1) return launch_cfg<64, 1, 8, 4>(a, stream);
       if (nct == 2) return launch_cfg<64, 2, 4, 4, 2>(a, stream);   // two workgroups per CU (2 x 80 KiB)
-      return launch_cfg<64, 4, 4, 3>(a, stream);
+      // 65..128 channels: the keys of a step in two parts of two tiles, 8 waves for one time step
+      // (4 query tiles x 2 key parts), two waves per SIMD
+      return launch_cfg<64, 2, 8, 3, 1, 2>(a, stream);
     case 128:
       if (nct == 1) return launch_cfg<128, 1, 4, 4>(a, stream);
       if (nct == 2) return launch_cfg<128, 2, 4, 3>(a, stream);

@@ -165,6 +165,9 @@ MFMA_SHAPES = [
     dict(B=1, C=32, T=70, H=2, Dh=64),                             # crosses two 32-step slabs
     dict(B=2, C=40, T=20, H=4, Dh=64, Hkv=2, validity=True),       # ragged channels, GQA
     dict(B=1, C=117, T=14, H=2, Dh=64, validity=True),             # c3's channel count
+    dict(B=1, C=65, T=40, H=2, Dh=64),                             # just past 64: keys in two parts, far steps, two slabs
+    dict(B=2, C=128, T=21, H=4, Dh=64, Hkv=2, validity=True),      # both key parts full, GQA, absent channels
+    dict(B=1, C=96, T=45, H=3, Dh=64),                             # second key part half empty; B*H not a multiple of 8
     dict(B=1, C=128, T=6, H=2, Dh=128, Hkv=1),                     # base-model head size
     dict(B=1, C=64, T=13, H=2, Dh=128),
     dict(B=1, C=20, T=37, H=1, Dh=128, validity=True),
