@@ -99,6 +99,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-model", action="store_true", help="skip the MVPFormer-S forward leg")
     ap.add_argument("--no-backward", action="store_true", help="skip the MVPA backward leg")
+    ap.add_argument("--base-model", action="store_true",
+                    help="also time the base-size classification forward (B1 C128 T512, bf16 and fp8 QK^T)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 256 MiB device copy (calibrates HBM traffic counters)")
     args = ap.parse_args()
@@ -191,6 +193,9 @@ def main():
             line["mvpformer_s"] = mvpformer_s_windows_per_s()
         except ImportError:
             line["mvpformer_s"] = None
+    if args.base_model:
+        from models.bench_model import mvpformer_base_forward_ms
+        line["mvpformer_base"] = mvpformer_base_forward_ms()
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(line))

@@ -40,3 +40,34 @@ def mvpformer_s_windows_per_s(B: int = 4, C: int = 64, T: int = 64, seg: int = 5
     return {"windows_per_s": round(B / (ms * 1e-3), 2), "ms_per_forward": round(ms, 3),
             "config": f"MVPFormer-S E768 L12 H12 Hkv4 Dh64 n_inner1728, B={B} C={C} T={T} "
                       f"segments of {seg} samples, bf16, random-init weights, synthetic iEEG"}
+
+
+def mvpformer_base_forward_ms(C: int = 128, T: int = 512, seg: int = 512, steps: int = 3,
+                              warmup: int = 2) -> dict:
+    """Random-init base-size classification forward (E2048 L24 H16 Hkv8 Dh128 n_inner5632, binary
+    head) on one window of C channels x T segments: bf16, then fp8 e4m3 QK^T."""
+    from models.configs import MVPFORMER_BASE
+    x = make_ieeg(1, C, T, seg, seed=7).to("cuda:0")
+    res = {"config": f"MVPFormer base E2048 L24 H16 Hkv8 Dh128 n_inner5632 + binary head, B=1 C={C} "
+                     f"T={T} segments of {seg} samples, random-init weights, synthetic iEEG"}
+    logits = {}
+    for fp8 in (False, True):
+        torch.manual_seed(3)
+        cfg = MVPFormerConfig(**dict(MVPFORMER_BASE, n_positions=max(T, 110)), fp8_qk=fp8)
+        model = HMVPFormer(cfg, WaveEncoder(seg, cfg.n_embd), MVPFormerHead(cfg.n_embd, 2))
+        model = model.to(device="cuda:0", dtype=torch.bfloat16).eval()
+        for _ in range(warmup):
+            y = model.classify(x)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            y = model.classify(x)
+        torch.cuda.synchronize()
+        res["ms_per_forward_fp8_qk" if fp8 else "ms_per_forward_bf16"] = round(
+            (time.perf_counter() - t0) * 1e3 / steps, 1)
+        logits[fp8] = y.float().cpu()
+        del model
+        torch.cuda.empty_cache()
+    res["logits_bf16"] = [round(v, 5) for v in logits[False].flatten().tolist()]
+    res["fp8_vs_bf16_logit_max_abs_diff"] = round((logits[True] - logits[False]).abs().max().item(), 6)
+    return res
