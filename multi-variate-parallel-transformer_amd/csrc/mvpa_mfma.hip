@@ -351,7 +351,11 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   }
 
   // =========================== setup: Qu, Qv, channel bias tile, Ec ===========================
-  bf16x8 Qu[KS], Qv[KS];     // (q+u), (q+v) * scale as QK^T / time-slab B operands
+  // big configurations (Dh 128, or 4 key tiles per wave) are register bound: there the (q+v)
+  // fragments are re-formed at each 32-step slab instead of kept, and the K fragments of a near
+  // step are requested tile by tile instead of all at once
+  constexpr bool LEAN = KS * NCT > 8;
+  bf16x8 Qu[KS], Qv[LEAN ? 1 : KS];     // (q+u), (q+v) * scale as QK^T / time-slab B operands
   // fp8 content term: q' = (q+u)*scale/sq and k' = k/sk are rounded to e4m3 with the per-head
   // amax scales sq, sk chosen by the caller; the MFMA accumulates in units of 1/(sq*sk), the
   // channel-bias tile is pre-divided accordingly and the product sq*sk returns inside the exp2 fma
@@ -377,7 +381,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
       const int d0 = ks * 16 + hh * 8;
       Qu[ks] = make_qfrag(raw[ks], bu + d0, sc2);
       if (FP8) Qu8[ks] = make_qfrag_fp8(raw[ks], bu + d0, sc2 / a.fp8_q_scale[h]);
-      Qv[ks] = make_qfrag(raw[ks], bv + d0, sc2);
+      if (!LEAN) Qv[ks] = make_qfrag(raw[ks], bv + d0, sc2);
       const bf16x8 qz = make_qfrag(raw[ks], bz + d0, sc2);
 #pragma unroll
       for (int t = 0; t < G::QT; ++t) {
@@ -517,7 +521,9 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const u32x4 rr = *(const u32x4*)(ktime + (int64_t)j * DH + ks * 16 + hh * 8);
-        stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(rr), Qv[ks], stc, 0, 0, 0);
+        const bf16x8 qv = LEAN ? make_qfrag(*(const u32x4*)(qrow + ks * 16 + hh * 8), bv + ks * 16 + hh * 8, sc2)
+                               : Qv[LEAN ? 0 : ks];
+        stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(rr), qv, stc, 0, 0, 0);
       }
     }
     float cm = -INFINITY;
@@ -582,18 +588,30 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
           S[t] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(kfrag_fp8(kr, fp8_inv_sk), Qu8[ks], S[t], 0, 0, 0);
         }
     } else {
-      // every K fragment of the step is requested before the first MFMA waits for one
-      bf16x8 ka[KS][NCT];
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-        for (int t = 0; t < NCT; ++t) ka[ks][t] = *(const bf16x8*)(stage + k_lane[ks] + t * 32 * ROWB);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int t = 0; t < NCT; ++t)
+      if (!LEAN) {
+        // every K fragment of the step is requested before the first MFMA waits for one
+        bf16x8 ka[KS][NCT];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
-          S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][t], Qu[ks], S[t], 0, 0, 0);
+#pragma unroll
+          for (int t = 0; t < NCT; ++t) ka[ks][t] = *(const bf16x8*)(stage + k_lane[ks] + t * 32 * ROWB);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < NCT; ++t)
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks)
+            S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][t], Qu[ks], S[t], 0, 0, 0);
+      } else {
+#pragma unroll
+        for (int t = 0; t < NCT; ++t) {
+          bf16x8 ka[KS];
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) ka[ks] = *(const bf16x8*)(stage + k_lane[ks] + t * 32 * ROWB);
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks)
+            S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], Qu[ks], S[t], 0, 0, 0);
+        }
+      }
     }
     float ls = 0.f;
 #pragma unroll
