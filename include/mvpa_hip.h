@@ -155,9 +155,9 @@ typedef struct mvpa_bwd_args {
   float* dbias_chan;         /* [B,H,N,C] gradient of the table (q+z).k_chan^T, by table column */
   float* ws_delta;           /* workspace [B*H,N]      (contents after the call unspecified)  */
   float* ws_time;            /* workspace [B,H,N,T]                                           */
-  float* ws_chan;            /* workspace [B,H,N,C]                                           */
+  float* ws_chan;            /* workspace [B,H,N,C rounded up to a multiple of 4]             */
   void* ws_qu;               /* nullable workspace [B,H,N,Dh] of `dtype`, 16-byte aligned; the
-                                matrix-core kernels (bf16, Dh = 64, even C <= 64, no key_bias)
+                                matrix-core kernels (bf16, Dh = 64, C <= 128, no key_bias)
                                 run only when it is given                                     */
 } mvpa_bwd_args;
 

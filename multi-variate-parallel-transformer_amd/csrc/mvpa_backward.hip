@@ -323,12 +323,8 @@ extern "C" int mvpa_backward(const mvpa_bwd_args* a, void* stream) {
     return MVPA_ERR_NONCAUSAL_BIAS;
   if (a->dtype == MVPA_F32) return mvpa::launch_bwd_dh<float>(a, (hipStream_t)stream, true);
   if (a->dtype == MVPA_BF16) {
-    // bf16, Dh = 64, C <= 64: both passes run on MFMA
-    if (mvpa_bwd_query_mfma_supported(a)) {
-      const int st = mvpa_launch_bwd_query_mfma(a, (hipStream_t)stream);
-      if (st != MVPA_OK) return st;
-      return mvpa_launch_bwd_key_mfma(a, (hipStream_t)stream);
-    }
+    // bf16, Dh = 64, C <= 128: both passes run on MFMA
+    if (mvpa_bwd_query_mfma_supported(a)) return mvpa_launch_bwd_mfma(a, (hipStream_t)stream);
     return mvpa::launch_bwd_dh<mvpa::bf16_t>(a, (hipStream_t)stream, true);
   }
   return MVPA_ERR_DTYPE;

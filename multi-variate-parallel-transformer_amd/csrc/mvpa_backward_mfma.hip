@@ -120,10 +120,10 @@ __device__ inline int swz_row(int row) { return (row >> 1) & 7; }
 __device__ inline int swz_tr(int row) { return ((row >> 1) & 1) << 2; }
 
 template <int NCT>
-__global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_args a) {
+__global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_args a, int q0, int k0, int accum) {
   constexpr int NW = QUERY_WAVES<NCT>;
   constexpr int CP = NCT * 32, TQW = NW / NCT, TILE = CP * ROWB;
-  static_assert(CP * 32 <= WAVE_SCRATCH && 32 * (CP + 1) <= WAVE_SCRATCH, "channel tables overlay the slabs");
+  static_assert(64 * 32 <= WAVE_SCRATCH && 32 * (CP + 1) <= WAVE_SCRATCH, "channel tables overlay the slabs");
   constexpr int STAGES = QSTAGES, STAGE_BYTES = 3 * TILE;   // stage: V | K | K (transposing)
   constexpr int LPW = CP / 8 / NW;                // 1 KiB wave loads per wave and tile copy
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -138,6 +138,7 @@ __global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_ker
   float* scr = Stb;       // before the first slab [CP][32] channel table, after the last one [32][PC]
 
   const int T_ = a.T, C_ = a.C, W = a.window, N = a.T * a.C;
+  const int CW = (C_ + 3) & ~3;                   // row pitch of the Ec tiles in the workspace
   const bool has_content = a.flags & MVPA_FLAG_CONTENT;
   const bool has_time = a.flags & MVPA_FLAG_TIME_BIAS;
   const bool has_chan = a.flags & MVPA_FLAG_CHAN_BIAS;
@@ -171,7 +172,8 @@ __global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_ker
   const int tq_hi = min(T_ - 1, tq0 + TQW - 1);
   const int tq = tq0 + wave / NCT;
   const bool active = tq < T_;
-  const int cq = (wave % NCT) * 32 + ln;
+  const int cqw0 = q0 + (wave % NCT) * 32;        // first query channel of this wave
+  const int cq = cqw0 + ln;
   const bool qok = active && cq < C_;
   const int nq = active ? tq * C_ + min(cq, C_ - 1) : 0;
   const int64_t row = ((int64_t)b * a.H + h) * N + nq;
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_ker
   for (int i = 0; i < LPW; ++i) {
     const int pc = (wave + NW * i) * 64 + lane;
     const int r = pc >> 3, phys = pc & 7;
-    const int rc = min(r, C_ - 1);
+    const int rc = min(k0 + r, C_ - 1);           // key channels k0 .. of this launch
     k_off_r[i] = rc * (int)a.k_stride_n + ((phys ^ swz_row(r)) << 3);
     k_off_t[i] = rc * (int)a.k_stride_n + ((phys ^ swz_tr(r)) << 3);
     v_off[i] = rc * (int)a.v_stride_n + ((phys ^ swz_row(r)) << 3);
@@ -226,81 +228,93 @@ __global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_ker
   f32x16 Ec[NCT];            // exp2(channel bias - mc): the far steps' probabilities up to a scalar
   float delta = 0.f, mc = -INFINITY, sumEc = 0.f;
   uint32_t kbits[NCT];
-  // channel-bias tile of this lane's query from the per-wave table in the scratch; -inf where
-  // the key channel is padding or invalid
-  auto gather_bc = [&](f32x16 (&Bc)[NCT]) {
-    const uint32_t cq4 = (uint32_t)(cq - 4 * hh + 4);
-    const int gbase = ((C_ - 1) * 32 + ln) * 4;
-    const unsigned char* scr_b = (const unsigned char*)scr;
-#pragma unroll
-    for (int t = 0; t < NCT; ++t)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const uint32_t ci4 = (uint32_t)(t * 32 + (i >> 2) * 8 + (i & 3) + 4);
-        const uint32_t dist = min(max(cq4, ci4) - min(cq4, ci4), (uint32_t)(C_ - 1));
-        const float val = *(const float*)(scr_b + (gbase - (int)(dist * 128u)));
-        const bool kv = (kbits[t] >> ((i >> 2) * 8 + (i & 3))) & 1u;
-        Bc[t][i] = kv ? val : -INFINITY;
-      }
-  };
   // every global load of the set-up goes out before the first use: one round trip, not one per
   // fragment.  The log-sum-exp is among them so that its wait does not fall into the loops, where
   // it would drain the whole ring (vmcnt 0) at every key step.
-  u32x4 raw_[KS], draw_[KS], oraw_[KS], er_[KS][NCT];
+  u32x4 raw_[KS], draw_[KS], oraw_[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     const int d0 = ks * 16 + hh * 8;
     raw_[ks] = *(const u32x4*)(qrow + d0);
     draw_[ks] = *(const u32x4*)(drow + d0);
     oraw_[ks] = *(const u32x4*)(orow + d0);
-#pragma unroll
-    for (int t = 0; t < NCT; ++t)
-      er_[ks][t] = *(const u32x4*)(kchan + (int64_t)min(t * 32 + ln, C_ - 1) * DH + d0);
   }
   const float lse = a.lse[row];
-  uint64_t kmask[2];
-#pragma unroll
-  for (int w = 0; w < 2; ++w) {
-    const int ck = w * 64 + lane;
-    bool ok = ck < C_;
+  uint64_t kmask;                                 // the (up to 64) key channels of this launch
+  {
+    const int ck = k0 + lane;
+    bool ok = ck < C_ && lane < CP;
     if (valid) ok = ok && valid[min(ck, C_ - 1)] != 0;
-    kmask[w] = __ballot(ok);
+    kmask = __ballot(ok);
   }
   asm volatile("" :: "v"(lse));
   {
-    f32x16 sct[NCT];
-#pragma unroll
-    for (int t = 0; t < NCT; ++t)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) sct[t][i] = 0.f;
+    bf16x8 qz[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d0 = ks * 16 + hh * 8;
       const u32x4 raw = raw_[ks], draw = draw_[ks], oraw = oraw_[ks];
       if (qok) *(bf16x8*)((bf16_t*)a.ws_qu + row * DH + d0) = qfrag(raw, bu + d0, sc2);   // for the key pass
-      const bf16x8 qz = qfrag(raw, bz + d0, sc2);
+      qz[ks] = qfrag(raw, bz + d0, sc2);
       dOf[ks] = as_frag(draw);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         delta += __uint_as_float(draw[i] << 16) * __uint_as_float(oraw[i] << 16);
         delta += __uint_as_float(draw[i] & 0xffff0000u) * __uint_as_float(oraw[i] & 0xffff0000u);
       }
-#pragma unroll
-      for (int t = 0; t < NCT; ++t)
-        sct[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(er_[ks][t]), qz, sct[t], 0, 0, 0);
     }
     delta = xhalf_sum(delta);
 #pragma unroll
-    for (int t = 0; t < NCT; ++t)
+    for (int t = 0; t < NCT; ++t) kbits[t] = (uint32_t)(kmask >> (t * 32 + 4 * hh));
+    // Channel-bias tile, one key tile at a time: the 32 queries of this wave and the 32 keys of
+    // tile t are at most 63 channels apart in either direction, so the rows C-1-d of the table
+    // (q+z).k_chan^T they need lie in a window of 64 rows starting at jlo.  That window goes
+    // through the per-wave scratch ([64][32]), and Bc[key][q] = table[C-1-|cq-ck|][q] is
+    // gathered from it; -inf where the key channel is padding or absent.
+#pragma unroll
+    for (int t = 0; t < NCT; ++t) {
+      const int ck0 = k0 + t * 32;
+      const int dmax = max(cqw0 + 31 - ck0, ck0 + 31 - cqw0);       // > 0
+      const int jlo = max(C_ - 1 - dmax, 0);
+      f32x16 sct[2];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sct[tt][i] = 0.f;
+      u32x4 er[KS][2];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+          er[ks][tt] = *(const u32x4*)(kchan + (int64_t)min(jlo + tt * 32 + ln, C_ - 1) * DH + ks * 16 + hh * 8);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+          sct[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(er[ks][tt]), qz[ks], sct[tt], 0, 0, 0);
+      wave_sync_lds();                            // the previous tile's gather is done with the scratch
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int j = tt * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
+          scr[j * 32 + ln] = has_chan ? sct[tt][i] : 0.f;
+        }
+      wave_sync_lds();
+      // row of the window for key ck = c_i + 4hh: (C-1-jlo) - |cq - ck|, clamped into the window
+      // for padded queries / keys (their values are never used)
+      const uint32_t cq4 = (uint32_t)(cq - 4 * hh + 4);
+      const int top = C_ - 1 - jlo;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int j = t * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
-        scr[j * 32 + ln] = has_chan ? sct[t][i] : 0.f;
+        const uint32_t ci4 = (uint32_t)(ck0 + (i >> 2) * 8 + (i & 3) + 4);
+        const int dist = (int)(max(cq4, ci4) - min(cq4, ci4));
+        const int jr = min(max(top - dist, 0), 63);
+        const float val = scr[jr * 32 + ln];
+        const bool kv = (kbits[t] >> ((i >> 2) * 8 + (i & 3))) & 1u;
+        Ec[t][i] = kv ? val : -INFINITY;
       }
-#pragma unroll
-    for (int t = 0; t < NCT; ++t) kbits[t] = (uint32_t)(kmask[t >> 1] >> ((t & 1) * 32 + 4 * hh));
-    wave_sync_lds();
-    gather_bc(Ec);
+    }
 #pragma unroll
     for (int t = 0; t < NCT; ++t)
 #pragma unroll
@@ -318,20 +332,14 @@ __global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_ker
     // for the key pass: (q+u) * scale, delta, and the tile exp2(channel bias - mc) by
     // [query][key channel]; and the rows of dbias_time that no key step reaches
     if (qok) {
-      float* wc = a.ws_chan + row * C_;
+      float* wc = a.ws_chan + row * CW + k0;      // rows of CW floats: 16-byte aligned for any C
 #pragma unroll
       for (int t = 0; t < NCT; ++t)
 #pragma unroll
         for (int a4 = 0; a4 < 4; ++a4) {
           const int ci = t * 32 + a4 * 8 + hh * 4;
-          if ((C_ & 3) == 0) {
-            if (ci < C_)
-              *(float4*)(wc + ci) = make_float4(Ec[t][a4 * 4], Ec[t][a4 * 4 + 1], Ec[t][a4 * 4 + 2], Ec[t][a4 * 4 + 3]);
-          } else {
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-              if (ci + j < C_) wc[ci + j] = Ec[t][a4 * 4 + j];
-          }
+          if (k0 + ci < CW)
+            *(float4*)(wc + ci) = make_float4(Ec[t][a4 * 4], Ec[t][a4 * 4 + 1], Ec[t][a4 * 4 + 2], Ec[t][a4 * 4 + 3]);
         }
     }
     if (qok && hh == 0) a.ws_delta[row] = delta;
@@ -349,13 +357,14 @@ __global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_ker
 
   // this wave's query rows are consecutive in memory; outputs are written a row at a time (the
   // two half-waves take alternate rows) so that each store covers one contiguous run
-  const int cq0 = (wave % NCT) * 32;
+  const int cq0 = cqw0;
   const int nq_live = active ? max(0, min(32, C_ - cq0)) : 0;
   const int64_t wrow0 = ((int64_t)b * a.H + h) * N + (int64_t)(active ? tq : 0) * C_ + cq0;
 
-  // the columns of dbias_time that no key step reaches
-  for (int q = hh; q < nq_live; q += 2)
-    for (int j = ln; j < T_ - 1 - tq; j += 32) a.dbias_time[(wrow0 + q) * T_ + j] = 0.f;
+  // the columns of dbias_time that no key step reaches (once: by the launch that does not add)
+  if (!accum)
+    for (int q = hh; q < nq_live; q += 2)
+      for (int j = ln; j < T_ - 1 - tq; j += 32) a.dbias_time[(wrow0 + q) * T_ + j] = 0.f;
 
   // ---- loop-invariant fragment offsets
   int r_lane[KS], t_lane[MT];
@@ -393,7 +402,10 @@ __global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_ker
     for (int it = 0; it < 16; ++it) {
       const int q = 2 * it + hh;
       const float g = Gtb[ln * GP + q];
-      if (q < nq_live && ln < nj) a.dbias_time[(wrow0 + q) * T_ + j0 + ln] = g;
+      if (q < nq_live && ln < nj) {
+        float* dst = a.dbias_time + (wrow0 + q) * T_ + j0 + ln;
+        *dst = accum ? *dst + g : g;              // launches of one stream: the key parts add up
+      }
     }
   };
 
@@ -589,30 +601,41 @@ __global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_ker
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int a4 = 0; a4 < 4; ++a4)
-        *(float4*)(dqo + mt * 32 + a4 * 8 + hh * 4) =
-            make_float4(dq[mt][a4 * 4], dq[mt][a4 * 4 + 1], dq[mt][a4 * 4 + 2], dq[mt][a4 * 4 + 3]);
+      {
+        float4* dst = (float4*)(dqo + mt * 32 + a4 * 8 + hh * 4);
+        float4 val = make_float4(dq[mt][a4 * 4], dq[mt][a4 * 4 + 1], dq[mt][a4 * 4 + 2], dq[mt][a4 * 4 + 3]);
+        if (accum) {
+          const float4 old = *dst;
+          val = make_float4(val.x + old.x, val.y + old.y, val.z + old.z, val.w + old.w);
+        }
+        *dst = val;
+      }
   }
 
   // channel-table gradient: element (ck) of query cq goes to column C-1-|cq-ck|, so column
-  // C-1-d collects the two key channels cq-d and cq+d.  The tile goes to a per-wave table
-  // [32 queries][PC] by key channel, and each output row is gathered from it (LDS float atomics
-  // for the scatter form were measured at ~0.3 us apiece).
+  // C-1-d collects the two key channels cq-d and cq+d (those of them that this launch holds).
+  // The tile goes to a per-wave table [32 queries][PC] by local key channel, and each output row
+  // is gathered from it (LDS float atomics for the scatter form were measured at ~0.3 us apiece).
   wave_sync_lds();
 #pragma unroll
   for (int t = 0; t < NCT; ++t)
 #pragma unroll
     for (int i = 0; i < 16; ++i) scr[ln * PC + t * 32 + (i >> 2) * 8 + hh * 4 + (i & 3)] = dSc[t][i];
   wave_sync_lds();
-  {
-    const int d = C_ - 1 - lane;                  // this lane's column holds distance d
+  for (int c0 = 0; c0 < C_; c0 += 64) {
+    const int col = c0 + lane;
+    const int d = C_ - 1 - col;                   // this lane's column holds distance d
 #pragma unroll 8
     for (int q = 0; q < 32; ++q) {
-      const int lo = cq0 + q - d, hi = cq0 + q + d;
+      const int lo = cq0 + q - d - k0, hi = cq0 + q + d - k0;      // local key channels
       float g = scr[q * PC + max(0, min(lo, CP - 1))];
       const float g2 = scr[q * PC + max(0, min(hi, CP - 1))];
-      if (lo < 0 || d < 0) g = 0.f;
-      if (d > 0 && hi < C_) g += g2;
-      if (q < nq_live && lane < C_) a.dbias_chan[(wrow0 + q) * C_ + lane] = g;
+      if (lo < 0 || lo >= CP || d < 0) g = 0.f;
+      if (d > 0 && hi >= 0 && hi < CP) g += g2;
+      if (q < nq_live && col < C_) {
+        float* dst = a.dbias_chan + (wrow0 + q) * C_ + col;
+        *dst = accum ? *dst + g : g;
+      }
     }
   }
 }
@@ -622,9 +645,8 @@ __global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_ker
 
 // 1 if the MFMA query pass can serve these (already validated) arguments
 int mvpa_bwd_query_mfma_supported(const mvpa_bwd_args* a) {
-  if (a->dtype != MVPA_BF16 || a->Dh != 64 || a->C > 64) return 0;
+  if (a->dtype != MVPA_BF16 || a->Dh != 64 || a->C > 128) return 0;
   if (!(a->flags & MVPA_FLAG_CAUSAL) || a->key_bias || !a->ws_qu) return 0;
-  if (a->C & 3) return 0;      // 16-byte direct-to-LDS loads of the rows of the [C][C] Ec tiles
   const uintptr_t p = (uintptr_t)a->q | (uintptr_t)a->k | (uintptr_t)a->v | (uintptr_t)a->o |
                       (uintptr_t)a->d_o | (uintptr_t)a->bias_u | (uintptr_t)a->bias_v |
                       (uintptr_t)a->bias_z | (uintptr_t)a->k_time | (uintptr_t)a->k_chan |
@@ -638,25 +660,16 @@ int mvpa_bwd_query_mfma_supported(const mvpa_bwd_args* a) {
   return 1;
 }
 
-int mvpa_launch_bwd_query_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
+template <int NCT>
+static void launch_query(const mvpa_bwd_args* a, hipStream_t stream, int q0, int k0, int accum) {
   using namespace mvpa::bwdq;
-  const int nct = a->C <= 32 ? 1 : 2;
-  const int nw = nct == 1 ? QUERY_WAVES<1> : QUERY_WAVES<2>;
-  const int tqw = nw / nct;
+  constexpr int nw = QUERY_WAVES<NCT>, tqw = nw / NCT, cp = NCT * 32;
   const int nt = (a->T + tqw - 1) / tqw;
-  const int cp = nct * 32;
   const size_t lds = (size_t)QSTAGES * 3 * cp * ROWB + (size_t)nw * WAVE_SCRATCH * sizeof(float);
   dim3 grid((unsigned)(nt * a->B * a->H));
-  if (nct == 1) {
-    auto kern = mvpa_bwd_query_mfma_kernel<1>;
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(kern, grid, dim3(nw * 64), lds, stream, *a);
-  } else {
-    auto kern = mvpa_bwd_query_mfma_kernel<2>;
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(kern, grid, dim3(nw * 64), lds, stream, *a);
-  }
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  auto kern = mvpa_bwd_query_mfma_kernel<NCT>;
+  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  hipLaunchKernelGGL(kern, grid, dim3(nw * 64), lds, stream, *a, q0, k0, accum);
 }
 
 // ==========================================================================================
@@ -687,7 +700,7 @@ namespace bwdq {
 template <int NCT> constexpr int KEY_WAVES = NCT == 2 ? 8 : 4;
 
 template <int NCT, bool MASKED>
-__global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_args a) {
+__global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_args a, int k0, int q0, int accum) {
   constexpr int NW = KEY_WAVES<NCT>;              // shadows the query pass's wave count
   constexpr int CP = NCT * 32, KT = NW / NCT, TILE = CP * ROWB;
   constexpr int CS_BYTES = CP * CP * 4, SC_BYTES = (KT + 1) * 256;
@@ -706,6 +719,7 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
   const int ln = lane & 31, hh = lane >> 5;
   const int ktw = wave / NCT, kt = wave % NCT;    // this wave's key step and key-channel tile
   const int T_ = a.T, C_ = a.C, W = a.window, N = a.T * a.C;
+  const int CW = (C_ + 3) & ~3;                   // row pitch of the Ec tiles in the workspace
   const bool has_content = a.flags & MVPA_FLAG_CONTENT;
   const int nbg = a.B * a.Hkv, ntk = (T_ + KT - 1) / KT;
   int bg, tile;
@@ -727,7 +741,8 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
   const bool wave_on = tk < T_;
   const int tkc = min(tk, T_ - 1);
 
-  const int ck = kt * 32 + ln;
+  const int ck = k0 + kt * 32 + ln;               // key channels k0 .., query channels q0 .. in this launch
+  const int ckl = kt * 32 + ln;                   // ... local to the launch
   const bool key_live = ck < C_;                  // invalid channels have Ec = 0 already
   const int64_t nk = (int64_t)tkc * C_ + min(ck, C_ - 1);
   const bf16_t* krow = (const bf16_t*)a.k + b * a.k_stride_b + g * a.k_stride_h + nk * a.k_stride_n;
@@ -745,7 +760,7 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
   for (int i = 0; i < LPW; ++i) {
     const int pc = (wave + NW * i) * 64 + lane;
     const int r = pc >> 3, phys = pc & 7;
-    const int rc = min(r, C_ - 1);
+    const int rc = min(q0 + r, C_ - 1);
     q_off_r[i] = rc * DH + ((phys ^ swz_row(r)) << 3);
     q_off_t[i] = rc * DH + ((phys ^ swz_tr(r)) << 3);
     d_off_r[i] = rc * (int)a.do_stride_n + ((phys ^ swz_row(r)) << 3);
@@ -755,10 +770,10 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
 #pragma unroll
   for (int i = 0; i < CS_LPW; ++i) {
     const int pc = (wave + NW * i) * 64 + lane;   // 16-byte chunk: row pc / (CP/4), 4 columns
-    const int r = min(pc / (CP / 4), C_ - 1), c4 = min((pc % (CP / 4)) * 4, (C_ - 1) & ~3);
-    cs_off[i] = r * C_ + c4;
+    const int r = min(q0 + pc / (CP / 4), C_ - 1), c4 = min((pc % (CP / 4)) * 4, max(CW - k0 - 4, 0));
+    cs_off[i] = r * CW + k0 + c4;
   }
-  const int sc_lane = min(lane, C_ - 1);
+  const int sc_lane = min(q0 + lane, C_ - 1);
   const uint32_t ring_lds = (uint32_t)(uintptr_t)(BWD_LDS_PTR(unsigned char))smem;
   // a step is fetched in full when it lies inside the content window of one of the waves
   auto wg_near = [&](int tq) -> bool {
@@ -773,14 +788,14 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
   const float* p_sc = nullptr;
   const float* p_de = nullptr;
   const int64_t d_do = (int64_t)C_ * a.do_stride_n, d_sc = (int64_t)T_ * C_;
-  const int d_ec = C_ * C_, d_qu = C_ * DH;
+  const int d_ec = C_ * CW, d_qu = C_ * DH;
   auto rebase = [&](int hq) {
     const int h = g * grp + hq;
     const int64_t bhq = (int64_t)b * a.H + h;
     const int64_t r0 = bhq * N + (int64_t)(T_ - 1) * C_;    // first query row of step T-1
     p_do = (const bf16_t*)a.d_o + b * a.do_stride_b + h * a.do_stride_h + (int64_t)(T_ - 1) * d_do;
     p_qu = (const bf16_t*)a.ws_qu + r0 * DH;
-    p_ec = a.ws_chan + r0 * C_;
+    p_ec = a.ws_chan + r0 * CW;
     p_sc = a.ws_time + ((bhq * T_ + (T_ - 1)) * T_ + tkc) * C_;
     p_de = a.ws_delta + r0;
   };
@@ -867,7 +882,7 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
   // ---- a query step outside the content window: P = Ec * exp2(e), dv only
   auto far_step = [&](const unsigned char* base) {
     const unsigned char* Dtr = base + OFF_DTR;
-    const float* Ecs = (const float*)(base + OFF_EC) + ck;
+    const float* Ecs = (const float*)(base + OFF_EC) + ckl;
     const float* ET = (const float*)(base + OFF_SC) + ktw * 64;
 #pragma unroll
     for (int qt = 0; qt < NCT; ++qt) {
@@ -880,7 +895,7 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float p = Ecs[(rb + j) * CP] * es[j];
-          P[a4 * 4 + j] = (!MASKED || (key_live && rb + j < C_)) ? p : 0.f;
+          P[a4 * 4 + j] = (!MASKED || (key_live && q0 + rb + j < C_)) ? p : 0.f;
         }
       }
 #pragma unroll
@@ -899,7 +914,7 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
     const unsigned char* Drow = base + OFF_DROW;
     const unsigned char* Qrow = base + OFF_QROW;
     const unsigned char* Qtr = base + OFF_QTR;
-    const float* Ecs = (const float*)(base + OFF_EC) + ck;
+    const float* Ecs = (const float*)(base + OFF_EC) + ckl;
     const float* TL = (const float*)(base + OFF_SC) + ktw * 64;
     const float* De = (const float*)(base + OFF_SC) + KT * 64;
 #pragma unroll
@@ -923,7 +938,7 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
         for (int j = 0; j < 4; ++j) {
           const int i = a4 * 4 + j;
           float p = __builtin_amdgcn_exp2f(S[i] + tls[j]) * Ecs[(rb + j) * CP];
-          if (MASKED) p = (key_live && rb + j < C_) ? p : 0.f;
+          if (MASKED) p = (key_live && q0 + rb + j < C_) ? p : 0.f;
           S[i] = p;
           dS[i] = p * (dP[i] - des[j]) * (1.f / kLog2e);
         }
@@ -969,8 +984,15 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
 #pragma unroll
       for (int a4 = 0; a4 < 4; ++a4) {
         const int d = mt * 32 + a4 * 8 + hh * 4;
-        *(float4*)(a.dk + o + d) = make_float4(dK[mt][a4 * 4], dK[mt][a4 * 4 + 1], dK[mt][a4 * 4 + 2], dK[mt][a4 * 4 + 3]);
-        *(float4*)(a.dv + o + d) = make_float4(dV[mt][a4 * 4], dV[mt][a4 * 4 + 1], dV[mt][a4 * 4 + 2], dV[mt][a4 * 4 + 3]);
+        float4 vk = make_float4(dK[mt][a4 * 4], dK[mt][a4 * 4 + 1], dK[mt][a4 * 4 + 2], dK[mt][a4 * 4 + 3]);
+        float4 vv = make_float4(dV[mt][a4 * 4], dV[mt][a4 * 4 + 1], dV[mt][a4 * 4 + 2], dV[mt][a4 * 4 + 3]);
+        if (accum) {                              // launches of one stream: the query parts add up
+          const float4 ok = *(const float4*)(a.dk + o + d), ov = *(const float4*)(a.dv + o + d);
+          vk = make_float4(vk.x + ok.x, vk.y + ok.y, vk.z + ok.z, vk.w + ok.w);
+          vv = make_float4(vv.x + ov.x, vv.y + ov.y, vv.z + ov.z, vv.w + ov.w);
+        }
+        *(float4*)(a.dk + o + d) = vk;
+        *(float4*)(a.dv + o + d) = vv;
       }
   }
 }
@@ -979,20 +1001,37 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
 }  // namespace mvpa
 
 template <int NCT, bool MASKED>
-static void launch_key(const mvpa_bwd_args* a, hipStream_t stream) {
+static void launch_key(const mvpa_bwd_args* a, hipStream_t stream, int k0, int q0, int accum) {
   using namespace mvpa::bwdq;
   constexpr int nw = KEY_WAVES<NCT>, cp = NCT * 32, kt = nw / NCT;
   const size_t lds = (size_t)KSTAGES * (4 * cp * ROWB + cp * cp * 4 + (kt + 1) * 256);
   dim3 grid((unsigned)(((a->T + kt - 1) / kt) * a->B * a->Hkv));
   auto kern = mvpa_bwd_key_mfma_kernel<NCT, MASKED>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  hipLaunchKernelGGL(kern, grid, dim3(nw * 64), lds, stream, *a);
+  hipLaunchKernelGGL(kern, grid, dim3(nw * 64), lds, stream, *a, k0, q0, accum);
 }
 
-int mvpa_launch_bwd_key_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
-  if (a->C == 32) launch_key<1, false>(a, stream);
-  else if (a->C < 32) launch_key<1, true>(a, stream);
-  else if (a->C == 64) launch_key<2, false>(a, stream);
-  else launch_key<2, true>(a, stream);
+// Both passes.  Up to 32 channels: one launch each with one channel tile per wave; up to 64: one
+// launch each with two.  Beyond that the channels are taken in parts of 64: with the forward's
+// log-sum-exp known, the contributions of disjoint key channels (to dq and the bias-table
+// gradients) and of disjoint query channels (to dk, dv) simply add up, so every (query part, key
+// part) pair is one query-pass launch followed by the key-pass launch that consumes its
+// workspace; later launches add to what earlier ones wrote (one stream, hence ordered).
+int mvpa_launch_bwd_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
+  const int C = a->C;
+  if (C <= 32) {
+    launch_query<1>(a, stream, 0, 0, 0);
+    if (C == 32) launch_key<1, false>(a, stream, 0, 0, 0);
+    else launch_key<1, true>(a, stream, 0, 0, 0);
+  } else {
+    const int parts = (C + 63) / 64;
+    for (int kp = 0; kp < parts; ++kp)
+      for (int qp = 0; qp < parts; ++qp) {
+        const int q0 = qp * 64, k0 = kp * 64;
+        launch_query<2>(a, stream, q0, k0, kp > 0);
+        if (C - q0 >= 64 && C - k0 >= 64) launch_key<2, false>(a, stream, k0, q0, qp > 0);
+        else launch_key<2, true>(a, stream, k0, q0, qp > 0);
+      }
+  }
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }

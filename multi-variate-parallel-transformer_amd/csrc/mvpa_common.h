@@ -76,5 +76,4 @@ int mvpa_launch_mfma(const mvpa_fwd_args* a, hipStream_t stream);
 int mvpa_mfma_supported(const mvpa_fwd_args* a);
 // backward, query pass on MFMA (bf16, Dh = 64, C <= 64)
 int mvpa_bwd_query_mfma_supported(const mvpa_bwd_args* a);
-int mvpa_launch_bwd_query_mfma(const mvpa_bwd_args* a, hipStream_t stream);
-int mvpa_launch_bwd_key_mfma(const mvpa_bwd_args* a, hipStream_t stream);
+int mvpa_launch_bwd_mfma(const mvpa_bwd_args* a, hipStream_t stream);

@@ -258,7 +258,7 @@ def mvpa_backward(q, k, v, o, d_o, lse, u, vb, z, k_time, k_chan, *,
     dbc = torch.empty((B, H, N, C), **f32)
     ws_delta = torch.empty((B, H, N), **f32)
     ws_time = torch.empty((B, H, N, T), **f32)
-    ws_chan = torch.empty((B, H, N, C), **f32)
+    ws_chan = torch.empty((B, H, N, (C + 3) // 4 * 4), **f32)
     ws_qu = torch.empty((B, H, N, Dh), dtype=dt, device=q.device)
     a = MvpaBwdArgs()
     a.struct_size = ctypes.sizeof(MvpaBwdArgs)

@@ -108,7 +108,10 @@ BF16_CASES = [
     dict(B=1, C=64, T=12, H=2, Hkv=2, Dh=64, window=10),      # two waves per time step
     dict(B=1, C=40, T=37, H=2, Hkv=1, Dh=64, window=10),      # ragged channels, two 32-step slabs, GQA
     dict(B=2, C=8, T=70, H=1, Hkv=1, Dh=64, window=4),        # three slabs, narrow window
-    dict(B=1, C=33, T=9, H=2, Hkv=2, Dh=64, window=0),        # content everywhere; C % 4 != 0: generic kernels
+    dict(B=1, C=33, T=9, H=2, Hkv=2, Dh=64, window=0),        # content everywhere; odd C (workspace rows padded to 36)
+    dict(B=1, C=117, T=9, H=2, Hkv=1, Dh=64, window=2),       # two channel parts (64 + 53), four launches per pass, GQA
+    dict(B=1, C=128, T=6, H=1, Hkv=1, Dh=64, window=10),      # two full channel parts
+    dict(B=2, C=65, T=35, H=2, Hkv=2, Dh=64, window=3),       # second part of one channel; two slabs
     dict(B=1, C=36, T=9, H=2, Hkv=2, Dh=64, window=0),        # content everywhere, ragged second channel tile
     dict(B=1, C=32, T=21, H=2, Hkv=1, Dh=64, window=3),       # one channel tile, four key steps per workgroup, GQA
     dict(B=2, C=20, T=40, H=2, Hkv=2, Dh=64, window=5),       # one ragged channel tile, two slabs
@@ -124,7 +127,7 @@ def test_backward_bf16_mfma_query_pass(case):
     inp = make_mvpa_inputs(seed=13, qkv_unit=True, **cfg).round_to(torch.bfloat16)
     d_out = torch.randn(inp.q.shape, generator=torch.Generator().manual_seed(6)).bfloat16().float()
     valid = None
-    if cfg["C"] in (40, 20):
+    if cfg["C"] in (40, 20, 117):
         valid = torch.ones(cfg["B"], cfg["C"], dtype=torch.bool)
         valid[:, [3, 17, cfg["C"] - 1]] = False
     _, ref = _oracle_grads(inp, d_out, window, chan_valid=valid)
