@@ -1,4 +1,4 @@
-// MVPA backward on MFMA (bf16, Dh = 64, C <= 64): the QUERY pass (the KEY pass follows below).
+// MVPA backward on MFMA (bf16, Dh = 64, up to 64 channels per launch, 128 in parts): the QUERY pass (the KEY pass follows below).
 //
 // Same tiling as the forward kernel: queries and keys are tiled by time step, a wave owns 32
 // query channels of one time step, products are formed transposed (a lane owns one query), the

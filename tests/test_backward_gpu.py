@@ -121,7 +121,7 @@ BF16_CASES = [
 
 @pytest.mark.parametrize("case", BF16_CASES, ids=lambda c: "B{B}C{C}T{T}H{H}g{Hkv}w{window}".format(**c))
 def test_backward_bf16_mfma_query_pass(case):
-    """bf16, Dh = 64, C <= 64 takes the MFMA query pass (dq, bias-table gradients)."""
+    """bf16, Dh = 64, C <= 128 takes the MFMA passes (dq, dk, dv, bias-table gradients)."""
     cfg = dict(case)
     window = cfg.pop("window")
     inp = make_mvpa_inputs(seed=13, qkv_unit=True, **cfg).round_to(torch.bfloat16)
