@@ -164,7 +164,7 @@ def main():
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "kernel": "mvpa_mfma_kernel",
                      "kernel_ms": round(kern_ms, 4)},
     }
-    if not args.no_backward and C <= 64 and C % 4 == 0:   # shapes the matrix-core backward serves
+    if not args.no_backward and C <= 128:   # shapes the matrix-core backward serves
         # the backward of the same workload (reported beside the headline, never part of `value`):
         # both passes of mvpa_backward, gradients and workspace allocated outside the timed region
         # by torch's caching allocator after the first call

@@ -119,3 +119,19 @@ def test_layer_state_dict_names():
     cfg.hidden_size = 66
     with pytest.raises(ValueError):
         MVPFormerGQAAttention(cfg)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: with --gpus above 1 (or under a multi-rank launcher) it exits
+    with a message that says so, before touching any device."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                         capture_output=True, text=True, timeout=120)
+    assert res.returncode == 2
+    assert "ONE GPU" in res.stderr and res.stdout.strip() == ""
+    env = dict(os.environ, WORLD_SIZE="2")
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py")], capture_output=True,
+                         text=True, timeout=120, env=env)
+    assert res.returncode == 2 and "ONE GPU" in res.stderr
