@@ -205,3 +205,23 @@ def test_backward_bf16_full_size_invariants():
     n_q = cfg["T"] * cfg["C"] * (cfg["H"] // cfg["Hkv"])
     tot = dv1.sum(2)                                  # [B,Hkv,Dh]
     assert (tot / n_q - 1).abs().max().item() <= 2e-3, (tot / n_q - 1).abs().max().item()
+
+
+def test_backward_bf16_strided_inputs_match_contiguous():
+    """q, k, v, o, d_o as head-interleaved views ([B,N,H,Dh] buffers, the layout the layer's fused
+    projection produces): the same gradients, bit for bit, as from contiguous copies."""
+    import mvpa_hip
+    cfg = dict(B=2, C=48, T=20, H=4, Hkv=2, Dh=64)
+    inp = make_mvpa_inputs(seed=4, qkv_unit=True, **cfg).to("cuda", torch.bfloat16)
+    tabs = (inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan)
+    out, lse = mvpa_hip.mvpa_forward(inp.q, inp.k, inp.v, *tabs, return_lse=True)
+    d_o = torch.randn(out.shape, device="cuda", generator=torch.Generator("cuda").manual_seed(1)).bfloat16()
+    ref = mvpa_hip.mvpa_backward(inp.q, inp.k, inp.v, out, d_o, lse, *tabs)
+
+    def interleave(t):                      # [B,h,N,Dh] -> view of a [B,N,h,Dh] buffer
+        return t.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    q, k, v, o, g = (interleave(t) for t in (inp.q, inp.k, inp.v, out, d_o))
+    assert not q.is_contiguous() and q.stride(-1) == 1
+    got = mvpa_hip.mvpa_backward(q, k, v, o, g, lse, *tabs)
+    for a, b in zip(got, ref):
+        assert torch.equal(a, b)
