@@ -657,6 +657,12 @@ int mvpa_bwd_query_mfma_supported(const mvpa_bwd_args* a) {
                     a->o_stride_b | a->o_stride_h | a->o_stride_n | a->do_stride_b |
                     a->do_stride_h | a->do_stride_n;
   if ((p & 15) || (s & 7)) return 0;
+  // row offsets within one time step are kept in 32 bits inside the kernels
+  const int64_t big = (int64_t)1 << 31;
+  if (a->C * a->q_stride_n >= big || a->C * a->k_stride_n >= big || a->C * a->v_stride_n >= big ||
+      a->C * a->do_stride_n >= big || a->q_stride_n < 0 || a->k_stride_n < 0 || a->v_stride_n < 0 ||
+      a->do_stride_n < 0)
+    return 0;
   return 1;
 }
 
