@@ -55,6 +55,11 @@ enum {
 #define MVPA_FLAG_TIME_BIAS 4u  /* (q+v).r[T-1-(tq-tk)]      (layers/mvpa.py:223,225)      */
 #define MVPA_FLAG_CHAN_BIAS 8u  /* (q+z).e[C-1-|cq-ck|]      (layers/mvpa.py:224,226)      */
 #define MVPA_FLAG_FP8_QK 16u    /* content term QK^T in fp8 e4m3 with per-head scales      */
+#define MVPA_FLAG_LAST_STEP 32u /* q, o (and lse) hold only the C rows of the LAST time step,
+                                   tq = T-1; k and v hold all T*C rows.  One step of incremental
+                                   decoding against cached keys and values (the use the
+                                   layer_past / use_cache arguments of layers/mvpa.py:314-321
+                                   are for).  Needs MVPA_FLAG_CAUSAL.                        */
 
 /*
  * Arguments of the fused MVPA forward.  Replaces the pair

@@ -38,6 +38,7 @@ extern "C" int mvpa_validate(const mvpa_fwd_args* a) {
   if (!a->bias_u || !a->bias_v || !a->bias_z || !a->k_time || !a->k_chan) return MVPA_ERR_NULL;
   if ((a->flags & (MVPA_FLAG_TIME_BIAS | MVPA_FLAG_CHAN_BIAS)) && !(a->flags & MVPA_FLAG_CAUSAL))
     return MVPA_ERR_NONCAUSAL_BIAS;
+  if ((a->flags & MVPA_FLAG_LAST_STEP) && !(a->flags & MVPA_FLAG_CAUSAL)) return MVPA_ERR_UNSUPPORTED;
   const int64_t n = (int64_t)a->T * a->C;
   // a token stride smaller than Dh (or a head/batch stride of 0 with more than one head)
   // means the caller's N does not match T*C or the view is wrong

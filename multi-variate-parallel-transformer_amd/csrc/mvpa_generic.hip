@@ -34,12 +34,17 @@ __global__ __launch_bounds__(GEN_THREADS) void mvpa_generic_kernel(mvpa_fwd_args
   const bool has_time = a.flags & MVPA_FLAG_TIME_BIAS;
   const bool has_chan = a.flags & MVPA_FLAG_CHAN_BIAS;
 
+  // MVPA_FLAG_LAST_STEP: only the C queries of the last time step exist; rq is the row of q / o,
+  // nq the query's place in the full sequence
+  const bool last_only = a.flags & MVPA_FLAG_LAST_STEP;
+  const int Nq = last_only ? C_ : N;
   const int nq_raw = blockIdx.x * GEN_THREADS + tid;
-  const bool live = nq_raw < N;
-  const int nq = live ? nq_raw : N - 1;           // clamp: dead lanes still take part in barriers
+  const bool live = nq_raw < Nq;
+  const int rq = live ? nq_raw : Nq - 1;          // clamp: dead lanes still take part in barriers
+  const int nq = last_only ? (T_ - 1) * C_ + rq : rq;
   const int tq = nq / C_, cq = nq % C_;
 
-  const T* qrow = (const T*)a.q + b * a.q_stride_b + h * a.q_stride_h + (int64_t)nq * a.q_stride_n;
+  const T* qrow = (const T*)a.q + b * a.q_stride_b + h * a.q_stride_h + (int64_t)rq * a.q_stride_n;
   const T* kbase = (const T*)a.k + b * a.k_stride_b + g * a.k_stride_h;
   const T* vbase = (const T*)a.v + b * a.v_stride_b + g * a.v_stride_h;
   const T* bu = (const T*)a.bias_u + g * DH;
@@ -67,7 +72,7 @@ __global__ __launch_bounds__(GEN_THREADS) void mvpa_generic_kernel(mvpa_fwd_args
   }
 
   const int q_last = min(N - 1, (int)blockIdx.x * GEN_THREADS + GEN_THREADS - 1);
-  const int hi = causal ? (q_last / C_ + 1) * C_ : N;
+  const int hi = (causal && !last_only) ? (q_last / C_ + 1) * C_ : N;   // last step: every key
 
   float m = -INFINITY, l = 0.f;
   float acc[DH];
@@ -156,11 +161,11 @@ __global__ __launch_bounds__(GEN_THREADS) void mvpa_generic_kernel(mvpa_fwd_args
   }
 
   if (live) {
-    T* orow = (T*)a.o + b * a.o_stride_b + h * a.o_stride_h + (int64_t)nq * a.o_stride_n;
+    T* orow = (T*)a.o + b * a.o_stride_b + h * a.o_stride_h + (int64_t)rq * a.o_stride_n;
     const float inv = 1.f / l;
 #pragma unroll
     for (int d = 0; d < DH; ++d) io<T>::store(orow + d, acc[d] * inv);
-    if (a.lse) a.lse[((int64_t)b * a.H + h) * N + nq] = (m + logf(l)) * kLog2e;
+    if (a.lse) a.lse[((int64_t)b * a.H + h) * Nq + rq] = (m + logf(l)) * kLog2e;
   }
 }
 
@@ -190,7 +195,8 @@ static int launch_generic_t(const mvpa_fwd_args* a, hipStream_t stream) {
   const size_t lds = base + (chan_table ? table : 0);
   auto kern = mvpa_generic_kernel<T, DH>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  dim3 grid((N + GEN_THREADS - 1) / GEN_THREADS, a->B * a->H);
+  const int n_rows = (a->flags & MVPA_FLAG_LAST_STEP) ? a->C : N;
+  dim3 grid((n_rows + GEN_THREADS - 1) / GEN_THREADS, a->B * a->H);
   hipLaunchKernelGGL(kern, grid, dim3(GEN_THREADS), lds, stream, *a, chan_table);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }

@@ -235,10 +235,16 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   const int nt = SPLIT ? 1 + T_ / 2 : (T_ + G::TQW - 1) / G::TQW;
   const int nbh = a.B * a.H;
   constexpr int TAIL_MERGE = 2;
+  // MVPA_FLAG_LAST_STEP: only the workgroup of the last time step runs, one per (b, h); q, o and
+  // lse are indexed by channel alone
+  const bool last_only = a.flags & MVPA_FLAG_LAST_STEP;
   int bh, tile;
   {
     const int L = blockIdx.x;
-    if ((nbh & 7) == 0 && nt > 1) {
+    if (last_only) {
+      bh = L;
+      tile = nt - 1;
+    } else if ((nbh & 7) == 0 && nt > 1) {
       if (L < nbh) {
         bh = L;                          // L & 7 is the XCD, the same one as below for this (b, h)
         tile = nt - 1;
@@ -284,14 +290,14 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   const int tq0 = split_last ? T_ - 1 : tile * G::TQW;
   const int tq_hi = split_last ? T_ - 1 : min(T_ - 1 - (SPLIT ? 1 : 0), tq0 + G::TQW - 1);
   const int tq = split_last ? T_ - 1 : tq0 + wave / G::WPT;
-  const bool active = tq <= tq_hi;
+  const bool active = tq <= tq_hi && (!last_only || tq == T_ - 1);
   const int cq = (wave % G::QT) * 32 + ln;         // this lane's query channel
   const bool qok = active && cq < C_;
 
   // Loads below are unconditional: rows that do not exist (padded channels, time steps past the
   // end) are redirected to an existing row and their results are never used.
   const bf16_t* qrow = (const bf16_t*)a.q + b * a.q_stride_b + h * a.q_stride_h +
-                       (int64_t)(active ? tq * C_ + min(cq, C_ - 1) : 0) * a.q_stride_n;
+                       (int64_t)(active ? (last_only ? 0 : tq * C_) + min(cq, C_ - 1) : 0) * a.q_stride_n;
   const bf16_t* kbase = (const bf16_t*)a.k + b * a.k_stride_b + g * a.k_stride_h;
   const bf16_t* vbase = (const bf16_t*)a.v + b * a.v_stride_b + g * a.v_stride_h;
   const bf16_t* ktime = (const bf16_t*)a.k_time + (int64_t)g * T_ * DH;
@@ -817,7 +823,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     const float ltot = l_run + __shfl_xor(l_run, 32);
     if (qok) {
       const float inv = 1.f / ltot;
-      const int64_t n = (int64_t)tq * C_ + cq;
+      const int64_t n = (last_only ? 0 : (int64_t)tq * C_) + cq;
       bf16_t* orow = (bf16_t*)a.o + b * a.o_stride_b + h * a.o_stride_h + n * a.o_stride_n;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
@@ -830,7 +836,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
           *(bf16x4*)(orow + d0) = w;
         }
       if (a.lse && hh == 0)
-        a.lse[((int64_t)b * a.H + h) * ((int64_t)T_ * C_) + n] = m_run + log2f(ltot);
+        a.lse[((int64_t)b * a.H + h) * (last_only ? (int64_t)C_ : (int64_t)T_ * C_) + n] = m_run + log2f(ltot);
     }
   }
 }
@@ -844,7 +850,7 @@ static int launch_one(const mvpa_fwd_args* a, hipStream_t stream) {
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)G::LDS_BYTES);
   const int nt = (G::TQW == 2 && STAGES == 4 && KH == 1) ? 1 + a->T / 2 : (a->T + G::TQW - 1) / G::TQW;   // as in the kernel
-  dim3 grid((unsigned)(nt * a->B * a->H));
+  dim3 grid((unsigned)(((a->flags & MVPA_FLAG_LAST_STEP) ? 1 : nt) * a->B * a->H));
   hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), G::LDS_BYTES, stream, *a);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }

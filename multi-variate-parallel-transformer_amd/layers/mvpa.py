@@ -195,7 +195,7 @@ class MVPFormerGQAAttention(torch.nn.Module):
         return s
 
     def _attend(self, hidden_states, positional_embedding, channel_embedding, attention_mask,
-                head_mask, use_cache, window):
+                head_mask, use_cache, window, layer_past=None):
         if self.training and (self.attn_dropout.p > 0 or self.resid_dropout.p > 0):
             raise NotImplementedError("MVPA HIP layer: dropout/training is not implemented; call .eval()")
         if self.is_cross_attention:
@@ -206,6 +206,9 @@ class MVPFormerGQAAttention(torch.nn.Module):
         h, hkv, dh, kv = self.num_heads, self.num_kv_heads, self.head_dim, self.embed_kv_dim
         n = t_len * c_len
         dt = hidden_states.dtype
+        if layer_past is not None:
+            return self._attend_step(hidden_states, positional_embedding, channel_embedding,
+                                     attention_mask, head_mask, use_cache, window, layer_past)
         with torch.no_grad():
             qkv = _linear(hidden_states, self._qkv_weight(dt))          # [B,T,C,E+2kvE]
             row = e + 2 * kv
@@ -236,6 +239,51 @@ class MVPFormerGQAAttention(torch.nn.Module):
             present = (k.reshape(bsz, hkv, t_len, c_len, dh), v.reshape(bsz, hkv, t_len, c_len, dh))
         return out, present
 
+    def _attend_step(self, hidden_states, positional_embedding, channel_embedding, attention_mask,
+                     head_mask, use_cache, window, layer_past):
+        """One step of incremental decoding: hidden_states holds the new time step only
+        ([B,1,C,E]), layer_past the keys and values of the steps before it ([B,Hkv,Tp,C,Dh] each,
+        as returned in `present`), positional_embedding all Tp+1 positions.  The new keys and
+        values are appended along the TIME axis; the reference's cache path concatenates along
+        dim -2, the channel axis (layers/mvpa.py:314-317), which does not continue the sequence,
+        and is not reproduced."""
+        bsz, t_new, c_len, e = hidden_states.shape
+        h, hkv, dh, kv = self.num_heads, self.num_kv_heads, self.head_dim, self.embed_kv_dim
+        past_k, past_v = layer_past
+        if t_new != 1:
+            raise NotImplementedError("MVPA HIP layer: with layer_past, hidden_states holds one new time step")
+        t_len = past_k.shape[2] + 1
+        if positional_embedding.shape[-2] != t_len or past_k.shape[3] != c_len:
+            raise ValueError("layer_past, positional_embedding and hidden_states disagree on T or C")
+        dt = hidden_states.dtype
+        with torch.no_grad():
+            qkv = _linear(hidden_states, self._qkv_weight(dt)).view(bsz, c_len, e + 2 * kv)
+            q = qkv[:, :, :e].view(bsz, c_len, h, dh).permute(0, 2, 1, 3)           # [B,H,C,Dh]
+            k_new = qkv[:, :, e:e + kv].view(bsz, c_len, hkv, dh).permute(0, 2, 1, 3)
+            v_new = qkv[:, :, e + kv:].view(bsz, c_len, hkv, dh).permute(0, 2, 1, 3)
+            k = torch.cat([past_k.to(dt), k_new.unsqueeze(2)], dim=2)                # [B,Hkv,T,C,Dh]
+            v = torch.cat([past_v.to(dt), v_new.unsqueeze(2)], dim=2)
+            k_time, k_chan = self._key_tables(positional_embedding, channel_embedding)
+            u, vb, z = (b.view(hkv, dh) for b in self.attn_bias.split(kv, dim=0))
+            chan_valid, key_bias = None, None
+            if attention_mask is not None:
+                chan_valid = self._as_channel_validity(attention_mask, bsz, t_len, c_len)
+                if chan_valid is None:
+                    key_bias = attention_mask.reshape(bsz, t_len * c_len).to(torch.float32)
+            merged = torch.empty((bsz, c_len, h, dh), dtype=dt, device=hidden_states.device)
+            mvpa_hip.mvpa_forward(
+                q, k.view(bsz, hkv, t_len * c_len, dh), v.view(bsz, hkv, t_len * c_len, dh),
+                u, vb, z, k_time, k_chan, sm_scale=self._scale(), window=window, causal=True,
+                content=bool(self.global_att), chan_valid=chan_valid, key_bias=key_bias,
+                out=merged.permute(0, 2, 1, 3), last_step_only=True,
+                fp8_qk=self.fp8_qk and dt == torch.bfloat16 and key_bias is None)
+            if head_mask is not None:
+                if head_mask.numel() != h:
+                    raise NotImplementedError("head_mask must hold one factor per head")
+                merged = merged * head_mask.to(dt).reshape(1, 1, h, 1)
+            out = _linear(merged.view(bsz, 1, c_len, e), self.c_proj.weight)
+        return out, ((k, v) if use_cache is True else None)
+
     def forward(
         self,
         hidden_states,
@@ -251,15 +299,14 @@ class MVPFormerGQAAttention(torch.nn.Module):
     ):
         if encoder_hidden_states is not None:
             raise NotImplementedError("MVPA HIP layer: cross attention is not implemented")
-        if layer_past is not None:
-            raise NotImplementedError("MVPA HIP layer: incremental decoding (layer_past) is not implemented")
         if not self._honours_masks:
             attention_mask, head_mask = None, None
         elif output_attentions:
             raise NotImplementedError(
                 "MVPA HIP layer: the fused kernel never forms the [B,H,N,N] attention weights")
         out, present = self._attend(hidden_states, positional_embedding, channel_embedding,
-                                    attention_mask, head_mask, use_cache, window=10)
+                                    attention_mask, head_mask, use_cache, window=10,
+                                    layer_past=layer_past)
         outputs = (out, present)
         if output_attentions:
             outputs += (None,)                            # layers/mvpa.py:407-408
@@ -267,8 +314,9 @@ class MVPFormerGQAAttention(torch.nn.Module):
 
 
 class MVPFormerGQAFlashAttention(MVPFormerGQAAttention):
-    """Interface of layers/mvpa.py:340-409: same parameters, attention_mask / head_mask /
-    layer_past ignored, `None` in place of attention weights."""
+    """Interface of layers/mvpa.py:340-409: same parameters, attention_mask / head_mask ignored,
+    `None` in place of attention weights.  layer_past continues the sequence by one time step
+    (see _attend_step)."""
 
     _honours_masks = False
 
@@ -276,7 +324,7 @@ class MVPFormerGQAFlashAttention(MVPFormerGQAAttention):
                 attention_mask=None, head_mask=None, encoder_hidden_states=None,
                 encoder_attention_mask=None, use_cache=False, output_attentions=False):
         out, present = self._attend(hidden_states, positional_embedding, channel_embedding,
-                                    None, None, use_cache, window=10)
+                                    None, None, use_cache, window=10, layer_past=layer_past)
         outputs = (out, present)
         if output_attentions:
             outputs += (None,)

@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libmvpa_hip.so")
 
 MVPA_F32, MVPA_BF16 = 0, 1
 KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA = 0, 1, 2
+FLAG_LAST_STEP = 32
 FLAG_CAUSAL, FLAG_CONTENT, FLAG_TIME_BIAS, FLAG_CHAN_BIAS, FLAG_FP8_QK = 1, 2, 4, 8, 16
 
 ERR_HEAD_DIM, ERR_HEAD_RATIO, ERR_CTX, ERR_SHAPE = -2, -3, -4, -5
@@ -182,34 +183,42 @@ def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float]
                  chan_valid: Optional[torch.Tensor] = None,
                  key_bias: Optional[torch.Tensor] = None, return_lse: bool = False,
                  kernel: int = KERNEL_AUTO, out: Optional[torch.Tensor] = None,
-                 fp8_qk: bool = False):
+                 fp8_qk: bool = False, last_step_only: bool = False):
     """Fused MVPA forward on the GPU.
 
     q [B,H,N,Dh]; k, v [B,Hkv,N,Dh]; u, vb, z [Hkv,Dh]; k_time [Hkv,T,Dh]; k_chan [Hkv,C,Dh];
     chan_valid [B,C] bool/uint8; key_bias [B,N] float32 additive.  Returns out [B,H,N,Dh] in
     q's dtype (and the base-2 log-sum-exp [B,H,N] float32 if asked).
+
+    last_step_only: q holds only the C queries of the last time step ([B,H,C,Dh]) while k, v hold
+    all T*C rows (cached steps followed by the new one); out is [B,H,C,Dh].  One step of
+    incremental decoding.
     """
     lib = load_library()
     _need_cuda(q, k, v, u, vb, z, k_time, k_chan, chan_valid, key_bias)
-    B, H, N, Dh = q.shape
+    B, H, Nq, Dh = q.shape
     assert k.shape[-1] == Dh and v.shape[-1] == Dh, "head dims of q, k, v differ"
     T, C = k_time.shape[-2], k_chan.shape[-2]
-    assert N == T * C, "N must equal T*C"
+    N = T * C
+    assert k.shape[2] == N and v.shape[2] == N, "k and v must hold T*C rows"
+    assert Nq == (C if last_step_only else N), "q must hold T*C rows (C with last_step_only)"
+    if last_step_only and not causal:
+        raise ValueError("last_step_only needs the time-causal mask")
     dt = q.dtype
     u, vb, z = (t.to(dt).contiguous() for t in (u, vb, z))
     k_time, k_chan = k_time.to(dt).contiguous(), k_chan.to(dt).contiguous()
     if out is None:
-        out = torch.empty((B, H, N, Dh), dtype=dt, device=q.device)
+        out = torch.empty((B, H, Nq, Dh), dtype=dt, device=q.device)
     if chan_valid is not None:
         chan_valid = chan_valid.to(torch.uint8).contiguous()
         assert chan_valid.shape == (B, C)
     if key_bias is not None:
         key_bias = key_bias.to(torch.float32).contiguous()
         assert key_bias.shape == (B, N)
-    lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device) if return_lse else None
+    lse = torch.empty((B, H, Nq), dtype=torch.float32, device=q.device) if return_lse else None
     flags = ((FLAG_CAUSAL if causal else 0) | (FLAG_CONTENT if content else 0) |
              (FLAG_TIME_BIAS if time_bias else 0) | (FLAG_CHAN_BIAS if chan_bias else 0) |
-             (FLAG_FP8_QK if fp8_qk else 0))
+             (FLAG_FP8_QK if fp8_qk else 0) | (FLAG_LAST_STEP if last_step_only else 0))
     s = (1.0 / Dh ** 0.5) if sm_scale is None else float(sm_scale)
     q_scale = k_scale = None
     if fp8_qk:

@@ -143,3 +143,28 @@ def test_base_classification_bf16_then_fp8():
     e8 = (logits[True] - ref).abs().max().item() / spread
     print(f"base-size logits: ref {ref.flatten().tolist()}, bf16 err {e16:.3e}, fp8 err {e8:.3e} (relative to spread)")
     assert e16 <= 3e-2 and e8 <= 6e-2
+
+
+@pytest.mark.parametrize("flash", [True, False], ids=["flash", "masked"])
+def test_layer_incremental_step_matches_full_forward(flash):
+    """use_cache / layer_past: the layer run on T-1 time steps with use_cache, then on the last
+    step alone with layer_past, gives the last step of the layer run on all T steps (bf16: the
+    projections are row-wise and the attention kernel runs the same code on the same operands, so
+    the results are identical)."""
+    from layers import MVPFormerGQAAttention, MVPFormerGQAFlashAttention
+    from models.mvpformer import MVPFormerConfig
+    torch.manual_seed(5)
+    cfg = MVPFormerConfig(n_embd=256, n_head=4, n_head_kv=2, n_layer=1, n_positions=16, n_channels=24)
+    cls = MVPFormerGQAFlashAttention if flash else MVPFormerGQAAttention
+    layer = cls(cfg, layer_idx=0).to("cuda", torch.bfloat16).eval()
+    B, T, C, E = 2, 11, 24, 256
+    x = torch.randn(B, T, C, E, device="cuda").bfloat16()
+    pos = torch.randn(1, T, E, device="cuda").bfloat16() * 0.02
+    chan = torch.randn(1, C, E, device="cuda").bfloat16() * 0.02
+    full = layer(x, pos, chan)[0]
+    # the first T-1 steps see the last T-1 rows of the relative-time table: positions 1 .. T-1
+    _, present = layer(x[:, :T - 1], pos[:, 1:], chan, use_cache=True)[:2]
+    assert present[0].shape == (B, 2, T - 1, C, 64)
+    step, present2 = layer(x[:, T - 1:], pos, chan, layer_past=present, use_cache=True)[:2]
+    assert step.shape == (B, 1, C, E) and present2[0].shape == (B, 2, T, C, 64)
+    assert torch.equal(step[:, 0], full[:, T - 1])

@@ -354,3 +354,30 @@ def test_fp8_needs_mfma_kernel():
     d = inp.to("cuda", torch.float32)
     with pytest.raises(mvpa_hip.MvpaError):
         mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, fp8_qk=True)
+
+
+LAST_STEP_SHAPES = [
+    dict(B=2, C=64, T=17, H=4, Hkv=2, Dh=64),      # split last step (two key steps per barrier), odd T
+    dict(B=1, C=117, T=12, H=2, Hkv=2, Dh=64),     # keys in two parts
+    dict(B=2, C=20, T=40, H=2, Hkv=1, Dh=64),      # 8 waves = 8 time steps per workgroup: 7 of them idle
+    dict(B=1, C=64, T=9, H=2, Hkv=2, Dh=128),
+    dict(B=3, C=8, T=1, H=1, Hkv=1, Dh=32),        # nothing cached yet
+]
+
+
+@pytest.mark.parametrize("cfg", LAST_STEP_SHAPES, ids=lambda c: "B{B}C{C}T{T}H{H}D{Dh}".format(**c))
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_last_step_only_equals_last_rows_of_full_forward(cfg, dtype):
+    """MVPA_FLAG_LAST_STEP (one step of incremental decoding: C queries against T*C cached keys)
+    gives the rows of the last time step of the full forward: the same kernel code runs on the
+    same operands, so bit for bit, output and log-sum-exp."""
+    inp = make_mvpa_inputs(seed=17, qkv_unit=True, **cfg).to("cuda", dtype)
+    C = cfg["C"]
+    tabs = (inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan)
+    full, lse_full = mvpa_hip.mvpa_forward(inp.q, inp.k, inp.v, *tabs, return_lse=True)
+    q_last = inp.q[:, :, -C:]
+    step, lse_step = mvpa_hip.mvpa_forward(q_last, inp.k, inp.v, *tabs, return_lse=True,
+                                           last_step_only=True)
+    assert step.shape == q_last.shape and lse_step.shape == q_last.shape[:3]
+    assert torch.equal(step, full[:, :, -C:])
+    assert torch.equal(lse_step, lse_full[:, :, -C:])
