@@ -2,13 +2,16 @@
 """Benchmark of the MVPA forward hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3] [--no-cpu] [--no-model]
+                    [--no-backward] [--base-model] [--copy-probe]
 
 A step is one fused MVPA forward (one kernel launch) over one batch of synthetic inputs that
 are already resident in HBM.  The default workload is the configuration the headline metric
 is quoted on: B=4, C=64, T=128, H=16, Dh=64, bf16, time-causal, window 10.  Prints ONE JSON
 line with the metric, the roofline of the attention kernel (achieved = algorithmic flops per
 launch / HIP-event time per launch) and a bounded CPU baseline (the oracle's op-by-op
-restatement of the reference PyTorch path on this box's host cores).
+restatement of the reference PyTorch path on this box's host cores).  Beside them, never part
+of `value`: `backward` (one mvpa_backward call on the same workload), `mvpformer_s` (the
+MVPFormer-S forward in windows per second) and, on request, `mvpformer_base`.
 """
 from __future__ import annotations
 
