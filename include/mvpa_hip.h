@@ -11,13 +11,14 @@
 #ifndef MVPA_HIP_H
 #define MVPA_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
 extern "C" {
 #endif
 
-#define MVPA_ABI_VERSION 1
+#define MVPA_ABI_VERSION 2
 
 /* ---- status codes ---------------------------------------------------------------- */
 enum {
@@ -106,6 +107,16 @@ typedef struct mvpa_fwd_args {
                                 (the reference's L, attentions/attn.py:327-333)         */
   const float* fp8_q_scale;  /* nullable [H]   per-head amax scales for MVPA_FLAG_FP8_QK */
   const float* fp8_k_scale;  /* nullable [Hkv]                                          */
+  void* split_ws;            /* nullable; MVPA_FLAG_LAST_STEP on the bf16 MFMA kernel only: with
+                                n_split > 1 the T key steps are cut into n_split runs, each run
+                                goes to a workgroup of its own per (b, h) and the partial results
+                                (soft-max over the run, its log-sum-exp) are merged by a second
+                                small kernel.  Without it one workgroup per (b, h) walks the whole
+                                cache.  Holds mvpa_split_ws_bytes(args) bytes, 16-byte aligned.
+                                No counterpart in the reference (its cache path,
+                                layers/mvpa.py:314-321, re-enters the full kernel).           */
+  int32_t n_split;           /* 0 or 1 = no split; at most T                              */
+  int32_t reserved0;
 } mvpa_fwd_args;
 
 /* ABI version of the loaded library. */
@@ -117,6 +128,10 @@ const char* mvpa_error_string(int status);
 /* Host-only check of an argument block; touches no device memory and needs no GPU.
  * Mirrors the asserts of attentions/attn.py:1041-1045, 1339, 1344. */
 int mvpa_validate(const mvpa_fwd_args* args);
+
+/* Bytes of mvpa_fwd_args.split_ws for args->n_split runs: n_split * B * H * C partial output
+ * rows of Dh bf16 values followed by as many float log-sum-exps.  0 if n_split <= 1. */
+size_t mvpa_split_ws_bytes(const mvpa_fwd_args* args);
 
 /* Fused forward; replaces attentions/attn.py:1064-1123 + 1305-1314 and
  * layers/mvpa.py:173-278.  Validates, then enqueues on `stream`. */

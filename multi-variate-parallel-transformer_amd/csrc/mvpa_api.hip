@@ -50,6 +50,14 @@ extern "C" int mvpa_validate(const mvpa_fwd_args* a) {
     if (a->dtype != MVPA_BF16) return MVPA_ERR_UNSUPPORTED;
     if (!a->fp8_q_scale || !a->fp8_k_scale) return MVPA_ERR_NULL;
   }
+  if (a->n_split < 0 || a->n_split > a->T) return MVPA_ERR_SHAPE;
+  if (a->n_split > 1) {
+    if (!(a->flags & MVPA_FLAG_LAST_STEP)) return MVPA_ERR_UNSUPPORTED;
+    if (!a->split_ws) return MVPA_ERR_NULL;
+    if ((uintptr_t)a->split_ws & 15) return MVPA_ERR_ALIGN;
+    const int len = (a->T + a->n_split - 1) / a->n_split;
+    if ((int64_t)(a->n_split - 1) * len >= a->T) return MVPA_ERR_SHAPE;   // an empty run
+  }
   if (a->kernel == MVPA_KERNEL_MFMA && !mvpa_mfma_supported(a)) {
     if (a->dtype == MVPA_BF16) {
       const uintptr_t p = (uintptr_t)a->q | (uintptr_t)a->k | (uintptr_t)a->v | (uintptr_t)a->o;
@@ -61,6 +69,11 @@ extern "C" int mvpa_validate(const mvpa_fwd_args* a) {
     return MVPA_ERR_UNSUPPORTED;
   }
   return MVPA_OK;
+}
+
+extern "C" size_t mvpa_split_ws_bytes(const mvpa_fwd_args* a) {
+  if (!a || a->n_split <= 1) return 0;
+  return (size_t)a->n_split * a->B * a->H * a->C * ((size_t)a->Dh * 2 + sizeof(float));
 }
 
 extern "C" int mvpa_select_kernel(const mvpa_fwd_args* a) {

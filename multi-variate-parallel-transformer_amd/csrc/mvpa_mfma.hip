@@ -201,7 +201,7 @@ struct Cfg {
   static_assert(WLOADS % NW == 0 || WLOADS < NW, "every loading wave issues the same number of loads");
 };
 
-template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8, int KH>
+template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8, int KH, bool RUNS>
 __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args a) {
   using G = Cfg<DH, NCT, NW, STAGES, KH>;
   constexpr int CP = G::CP, KS = G::KS, MT = G::MT, ROWB = G::ROWB, CHUNKS = G::CHUNKS;
@@ -215,7 +215,18 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   // compiler branch on everything derived from it (tq, far/near, ...) without exec masking
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 31, hh = lane >> 5;
-  const int T_ = a.T, C_ = a.C, W = a.window;
+  const int C_ = a.C, W = a.window;
+  // MVPA_FLAG_LAST_STEP with a split workspace: block L works on run L / (B*H) of the key steps,
+  // steps [t_lo, t_lo + T_).  Seen from the queries of the last step a run is a problem of its
+  // own (content term everywhere, every key visible, table row of key step tk is tk), so the rest
+  // of the kernel just takes T_ steps from pointers moved on by t_lo; its normalised output and
+  // log-sum-exp go to the workspace, from where mvpa_split_merge_kernel combines the runs.
+  // (RUNS: a build of the kernel of its own, so that the usual launch carries none of this.)
+  const int n_split = RUNS ? a.n_split : 1;
+  const int split_len = (a.T + n_split - 1) / n_split;
+  const int run = n_split > 1 ? (int)blockIdx.x / (a.B * a.H) : 0;
+  const int t_lo = run * split_len;
+  const int T_ = n_split > 1 ? min(split_len, a.T - t_lo) : a.T;
   const bool has_content = a.flags & MVPA_FLAG_CONTENT;
   const bool has_time = a.flags & MVPA_FLAG_TIME_BIAS;
   const bool has_chan = a.flags & MVPA_FLAG_CHAN_BIAS;
@@ -242,7 +253,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   {
     const int L = blockIdx.x;
     if (last_only) {
-      bh = L;
+      bh = n_split > 1 ? L % nbh : L;
       tile = nt - 1;
     } else if ((nbh & 7) == 0 && nt > 1) {
       if (L < nbh) {
@@ -298,9 +309,9 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   // end) are redirected to an existing row and their results are never used.
   const bf16_t* qrow = (const bf16_t*)a.q + b * a.q_stride_b + h * a.q_stride_h +
                        (int64_t)(active ? (last_only ? 0 : tq * C_) + min(cq, C_ - 1) : 0) * a.q_stride_n;
-  const bf16_t* kbase = (const bf16_t*)a.k + b * a.k_stride_b + g * a.k_stride_h;
-  const bf16_t* vbase = (const bf16_t*)a.v + b * a.v_stride_b + g * a.v_stride_h;
-  const bf16_t* ktime = (const bf16_t*)a.k_time + (int64_t)g * T_ * DH;
+  const bf16_t* kbase = (const bf16_t*)a.k + b * a.k_stride_b + g * a.k_stride_h + (int64_t)t_lo * C_ * a.k_stride_n;
+  const bf16_t* vbase = (const bf16_t*)a.v + b * a.v_stride_b + g * a.v_stride_h + (int64_t)t_lo * C_ * a.v_stride_n;
+  const bf16_t* ktime = (const bf16_t*)a.k_time + ((int64_t)g * a.T + t_lo) * DH;
   const bf16_t* kchan = (const bf16_t*)a.k_chan + (int64_t)g * C_ * DH;
   const bf16_t* bu = (const bf16_t*)a.bias_u + g * DH;
   const bf16_t* bv = (const bf16_t*)a.bias_v + g * DH;
@@ -824,7 +835,9 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     if (qok) {
       const float inv = 1.f / ltot;
       const int64_t n = (last_only ? 0 : (int64_t)tq * C_) + cq;
-      bf16_t* orow = (bf16_t*)a.o + b * a.o_stride_b + h * a.o_stride_h + n * a.o_stride_n;
+      const int64_t prow = ((int64_t)run * nbh + bh) * C_ + cq;      // row of the split workspace
+      bf16_t* orow = n_split > 1 ? (bf16_t*)a.split_ws + prow * DH
+                                 : (bf16_t*)a.o + b * a.o_stride_b + h * a.o_stride_h + n * a.o_stride_n;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -835,10 +848,46 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
           for (int r = 0; r < 4; ++r) w[r] = (__bf16)(acc[mt][a4 * 4 + r] * inv);
           *(bf16x4*)(orow + d0) = w;
         }
-      if (a.lse && hh == 0)
+      if (n_split > 1) {
+        float* plse = (float*)((bf16_t*)a.split_ws + (int64_t)n_split * nbh * C_ * DH);
+        if (hh == 0) plse[prow] = m_run + log2f(ltot);
+      } else if (a.lse && hh == 0) {
         a.lse[((int64_t)b * a.H + h) * (last_only ? (int64_t)C_ : (int64_t)T_ * C_) + n] = m_run + log2f(ltot);
+      }
     }
   }
+}
+
+// Combines the runs of a split last-step launch: out = sum_r 2^(lse_r - lse) o_r with
+// lse = log2 sum_r 2^lse_r.  One wave per output row, lane = pair of head-dim elements.
+template <int DH>
+__global__ __launch_bounds__(256) void mvpa_split_merge_kernel(mvpa_fwd_args a) {
+  const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int nbh = a.B * a.H, C_ = a.C, rows = nbh * C_;
+  if (row >= rows) return;
+  const bf16_t* po = (const bf16_t*)a.split_ws;
+  const float* plse = (const float*)(po + (int64_t)a.n_split * rows * DH);
+  float m = -INFINITY;
+  for (int r = 0; r < a.n_split; ++r) m = fmaxf(m, plse[(int64_t)r * rows + row]);
+  float l = 0.f, acc[2] = {0.f, 0.f};
+  for (int r = 0; r < a.n_split; ++r) {
+    const float w = fast_exp2(plse[(int64_t)r * rows + row] - m);
+    l += w;
+    if (2 * lane < DH) {
+      const bf16x2 v = *(const bf16x2*)(po + ((int64_t)r * rows + row) * DH + 2 * lane);
+      acc[0] += w * (float)v[0];
+      acc[1] += w * (float)v[1];
+    }
+  }
+  const int bh = row / C_, cq = row % C_, b = bh / a.H, h = bh % a.H;
+  if (2 * lane < DH) {
+    const float inv = 1.f / l;
+    bf16x2 w2;
+    w2[0] = (__bf16)(acc[0] * inv);
+    w2[1] = (__bf16)(acc[1] * inv);
+    *(bf16x2*)((bf16_t*)a.o + b * a.o_stride_b + h * a.o_stride_h + (int64_t)cq * a.o_stride_n + 2 * lane) = w2;
+  }
+  if (a.lse && lane == 0) a.lse[row] = m + log2f(l);
 }
 
 template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8, int KH>
@@ -846,12 +895,19 @@ static int launch_one(const mvpa_fwd_args* a, hipStream_t stream) {
   using G = Cfg<DH, NCT, NW, STAGES, KH>;
   static_assert(KH <= 2 && (KH == 1 || G::TQW * G::QT * (2 + G::MT * 16) * 256 <= G::RING_BYTES), "merge buffer");
   static_assert(G::LDS_BYTES <= 160 * 1024, "LDS budget");
-  auto kern = mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH>;
+  const bool last = a->flags & MVPA_FLAG_LAST_STEP;
+  const int n_split = (last && a->split_ws && a->n_split > 1) ? a->n_split : 1;
+  auto kern = n_split > 1 ? mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH, true>
+                          : mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH, false>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)G::LDS_BYTES);
   const int nt = (G::TQW == 2 && STAGES == 4 && KH == 1) ? 1 + a->T / 2 : (a->T + G::TQW - 1) / G::TQW;   // as in the kernel
-  dim3 grid((unsigned)(((a->flags & MVPA_FLAG_LAST_STEP) ? 1 : nt) * a->B * a->H));
+  dim3 grid((unsigned)((last ? n_split : nt) * a->B * a->H));
   hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), G::LDS_BYTES, stream, *a);
+  if (n_split > 1) {
+    const int rows = a->B * a->H * a->C;
+    hipLaunchKernelGGL(mvpa_split_merge_kernel<DH>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, *a);
+  }
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 

@@ -24,7 +24,7 @@ def test_exports_every_declared_symbol(lib):
     assert "mvpa_forward" in names and "mvpa_linear_bf16" in names
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/mvpa_hip.h but not exported"
-    assert lib.mvpa_version() == 1
+    assert lib.mvpa_version() == 2
 
 
 def _args(B=2, H=4, Hkv=4, T=4, C=3, Dh=32, dtype=torch.float32, **kw):
@@ -60,6 +60,35 @@ def test_validate_rejects(lib, mutate, code):
     assert lib.mvpa_validate(ctypes.byref(a)) == code
     assert lib.mvpa_forward(ctypes.byref(a), None) == code      # rejected before any launch
     assert len(lib.mvpa_error_string(code)) > 3
+
+
+def test_validate_key_split_arguments(lib):
+    """n_split cuts the key steps of a MVPA_FLAG_LAST_STEP launch into runs: it needs that flag, a
+    16-byte aligned workspace of mvpa_split_ws_bytes and no empty run."""
+    a, keep = _args(T=6)
+    assert lib.mvpa_split_ws_bytes(ctypes.byref(a)) == 0
+    a.n_split = 3
+    assert lib.mvpa_split_ws_bytes(ctypes.byref(a)) == 3 * 2 * 4 * 3 * (32 * 2 + 4)
+    assert lib.mvpa_validate(ctypes.byref(a)) == -8              # not a last-step launch
+    a.flags |= mvpa_hip.FLAG_LAST_STEP
+    assert lib.mvpa_validate(ctypes.byref(a)) == -1              # no workspace
+    buf = ctypes.create_string_buffer(64)
+    p16 = (ctypes.addressof(buf) + 15) & ~15
+    a.split_ws = p16 + 4
+    assert lib.mvpa_validate(ctypes.byref(a)) == -7
+    a.split_ws = p16
+    assert lib.mvpa_validate(ctypes.byref(a)) == 0
+    a.n_split = 4                                                # runs of 2: the fourth is empty
+    assert lib.mvpa_validate(ctypes.byref(a)) == -5
+    a.n_split = 7                                                # more runs than key steps
+    assert lib.mvpa_validate(ctypes.byref(a)) == -5
+    a.n_split = -1
+    assert lib.mvpa_validate(ctypes.byref(a)) == -5
+    assert mvpa_hip.default_key_splits(1, 16, 512) == 16
+    assert mvpa_hip.default_key_splits(8, 64, 512) == 1
+    for T in range(1, 200):                                      # never an empty run
+        n = mvpa_hip.default_key_splits(1, 2, T)
+        assert n >= 1 and (n - 1) * ((T + n - 1) // n) < T
 
 
 def test_null_block(lib):

@@ -377,7 +377,50 @@ def test_last_step_only_equals_last_rows_of_full_forward(cfg, dtype):
     full, lse_full = mvpa_hip.mvpa_forward(inp.q, inp.k, inp.v, *tabs, return_lse=True)
     q_last = inp.q[:, :, -C:]
     step, lse_step = mvpa_hip.mvpa_forward(q_last, inp.k, inp.v, *tabs, return_lse=True,
-                                           last_step_only=True)
+                                           last_step_only=True, key_splits=1)
     assert step.shape == q_last.shape and lse_step.shape == q_last.shape[:3]
     assert torch.equal(step, full[:, :, -C:])
     assert torch.equal(lse_step, lse_full[:, :, -C:])
+
+
+SPLIT_CASES = [
+    (dict(B=2, C=64, T=17, H=4, Hkv=2, Dh=64), 2),      # runs of 9 and 8 steps
+    (dict(B=2, C=64, T=17, H=4, Hkv=2, Dh=64), 17),     # one key step per run
+    (dict(B=1, C=117, T=45, H=2, Hkv=2, Dh=64), 4),     # keys in two parts, runs 12+12+12+9
+    (dict(B=2, C=20, T=70, H=2, Hkv=1, Dh=64), 3),      # runs longer than a 32-step slab
+    (dict(B=1, C=128, T=40, H=2, Hkv=1, Dh=128), 5),
+    (dict(B=1, C=64, T=33, H=2, Hkv=2, Dh=128), None),  # the binding's own choice
+    (dict(B=3, C=8, T=24, H=2, Hkv=1, Dh=32), 6),
+]
+
+
+@pytest.mark.parametrize("cfg,n", SPLIT_CASES, ids=lambda c: "B{B}C{C}T{T}H{H}D{Dh}".format(**c) if isinstance(c, dict) else f"n{c}")
+@pytest.mark.parametrize("fp8", [False, True], ids=["bf16", "fp8qk"])
+def test_last_step_key_splits_match_unsplit(cfg, n, fp8):
+    """The key steps of a last-step launch cut into runs, each on its own workgroups, merged by the
+    second kernel: within bf16 rounding of the one-workgroup result (the partial outputs pass
+    through bf16), log-sum-exp to 1e-3, with some channels absent."""
+    inp = make_mvpa_inputs(seed=23, qkv_unit=True, **cfg).to("cuda", torch.bfloat16)
+    C = cfg["C"]
+    valid = torch.ones(cfg["B"], C, dtype=torch.bool, device="cuda")
+    valid[:, 1::5] = False
+    tabs = (inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan)
+    q_last = inp.q[:, :, -C:]
+    kw = dict(return_lse=True, last_step_only=True, chan_valid=valid, fp8_qk=fp8)
+    ref, lse_ref = mvpa_hip.mvpa_forward(q_last, inp.k, inp.v, *tabs, key_splits=1, **kw)
+    got, lse_got = mvpa_hip.mvpa_forward(q_last, inp.k, inp.v, *tabs, key_splits=n, **kw)
+    if n is None:
+        assert mvpa_hip.default_key_splits(cfg["B"], cfg["H"], cfg["T"]) > 1
+    err = (got.float() - ref.float()).abs().max().item()
+    rel = ((got.float() - ref.float()).norm() / ref.float().norm()).item()
+    assert err <= 2e-2 and rel <= 5e-3, (err, rel)
+    assert (lse_got - lse_ref).abs().max().item() <= 1e-3
+
+
+def test_key_splits_rejected_where_they_make_no_sense():
+    d = make_mvpa_inputs(seed=1, B=1, C=8, T=6, H=1, Hkv=1, Dh=64).to("cuda", torch.bfloat16)
+    tabs = (d.u, d.vb, d.z, d.k_time, d.k_chan)
+    with pytest.raises(AssertionError):    # 4 runs of ceil(6/4) = 2 steps: the last one is empty
+        mvpa_hip.mvpa_forward(d.q[:, :, -8:], d.k, d.v, *tabs, last_step_only=True, key_splits=4)
+    with pytest.raises(AssertionError):    # more runs than key steps
+        mvpa_hip.mvpa_forward(d.q[:, :, -8:], d.k, d.v, *tabs, last_step_only=True, key_splits=7)
