@@ -11,7 +11,9 @@ line with the metric, the roofline of the attention kernel (achieved = algorithm
 launch / HIP-event time per launch) and a bounded CPU baseline (the oracle's op-by-op
 restatement of the reference PyTorch path on this box's host cores).  Beside them, never part
 of `value`: `backward` (one mvpa_backward call on the same workload), `mvpformer_s` (the
-MVPFormer-S forward in windows per second) and, on request, `mvpformer_base`.
+MVPFormer-S forward in windows per second), `mvpformer_s_stream` (one new segment of a stream
+against cached keys and values, beside the full forward over the same window) and, on request,
+`mvpformer_base`.
 """
 from __future__ import annotations
 
@@ -194,6 +196,8 @@ def main():
         try:
             from models.bench_model import mvpformer_s_windows_per_s
             line["mvpformer_s"] = mvpformer_s_windows_per_s()
+            from models.bench_model import mvpformer_s_stream_step_ms
+            line["mvpformer_s_stream"] = mvpformer_s_stream_step_ms()
         except ImportError:
             line["mvpformer_s"] = None
     if args.base_model:

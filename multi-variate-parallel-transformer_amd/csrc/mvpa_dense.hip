@@ -158,6 +158,135 @@ __global__ __launch_bounds__(256) void linear_bf16_kernel(const bf16_t* __restri
 }
 
 // -----------------------------------------------------------------------------------------
+// Skinny variant for at most 128 rows of x (one decoding step: a time step of C <= 128 channels):
+// the work is reading w once, so it is spread over as many workgroups as there are 32-column
+// slices of the output, and inside a workgroup over 8 waves that split K (wave v takes the
+// 16-wide k-steps v, v+8, ...).  Fragments go from global memory straight into the MFMA operands
+// (A = 32 rows of w, B = 32 rows of x, so a lane owns one x row and 4 consecutive output columns
+// per accumulator quad), several k-steps are requested before the first is used, and the 8
+// partial tiles are summed through LDS.  XT = 32-row tiles of x (2 or 4).  EPI == 1: gate rows n
+// and up rows N + n of w side by side.
+// -----------------------------------------------------------------------------------------
+constexpr int SK_WAVES = 8;
+
+__device__ inline bf16x8 chunk_as_bf16x8(u32x4 v) {
+  union { u32x4 u; bf16x8 b; } c;
+  c.u = v;
+  return c.b;
+}
+
+template <int EPI, int XT>
+__global__ __launch_bounds__(SK_WAVES * 64) void linear_bf16_skinny_kernel(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, bf16_t* __restrict__ Y, int64_t M,
+    int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldy) {
+  constexpr int NA = EPI == 1 ? 2 : 1;            // w tiles per workgroup (gate, up)
+  constexpr int UNROLL = XT == 2 ? 4 : 2;         // k-steps in flight per wave
+  extern __shared__ __attribute__((aligned(16))) float sk_red[];   // [SK_WAVES][XT][16][64]
+  const int tid = threadIdx.x, lane = tid & 63, ln = lane & 31, hh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t n0 = (int64_t)blockIdx.x * 32;
+  const int xt_live = (int)((M + 31) / 32);       // tiles of x rows in use
+
+  const bf16_t* wrow[NA];
+  bool wok[NA];
+#pragma unroll
+  for (int a = 0; a < NA; ++a) {
+    const int64_t n = n0 + ln;
+    wok[a] = n < N;
+    wrow[a] = W + ((wok[a] ? n : 0) + (a ? N : 0)) * ldw;
+  }
+  const bf16_t* xrow[XT];
+  bool xok[XT];
+#pragma unroll
+  for (int t = 0; t < XT; ++t) {
+    const int64_t m = t * 32 + ln;
+    xok[t] = m < M;
+    xrow[t] = X + (xok[t] ? m : 0) * ldx;
+  }
+
+  f32x16 acc[NA][XT];
+#pragma unroll
+  for (int a = 0; a < NA; ++a)
+#pragma unroll
+    for (int t = 0; t < XT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][t][r] = 0.f;
+
+  const int nks = (int)((K + 15) / 16);
+  for (int s0 = wave; s0 < nks; s0 += SK_WAVES * UNROLL) {
+    u32x4 wf[UNROLL][NA], xf[UNROLL][XT];
+#pragma unroll
+    for (int j = 0; j < UNROLL; ++j) {
+      const int64_t k = (int64_t)(s0 + j * SK_WAVES) * 16 + hh * 8;     // past K: zeros
+#pragma unroll
+      for (int a = 0; a < NA; ++a) wf[j][a] = load_chunk(wrow[a], k, K, wok[a]);
+#pragma unroll
+      for (int t = 0; t < XT; ++t)
+        if (t < xt_live) xf[j][t] = load_chunk(xrow[t], k, K, xok[t]);
+    }
+#pragma unroll
+    for (int j = 0; j < UNROLL; ++j)
+#pragma unroll
+      for (int a = 0; a < NA; ++a)
+#pragma unroll
+        for (int t = 0; t < XT; ++t)
+          if (t < xt_live)
+            acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chunk_as_bf16x8(wf[j][a]), chunk_as_bf16x8(xf[j][t]), acc[a][t], 0, 0, 0);
+  }
+
+  // reduction over the waves, one w tile at a time through the same buffer.  Item -> (x tile t,
+  // accumulator quad q, lane l): x row t*32 + l%32, columns 8q + 4(l/32) + 0..3
+  constexpr int ITEMS = XT * 256 / (SK_WAVES * 64);
+  float sum[NA][ITEMS][4];
+#pragma unroll
+  for (int a = 0; a < NA; ++a) {
+    if (a) __syncthreads();
+#pragma unroll
+    for (int t = 0; t < XT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sk_red[((wave * XT + t) * 16 + r) * 64 + lane] = acc[a][t][r];
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int item = tid + it * SK_WAVES * 64;
+      const int t = item >> 8, q = (item >> 6) & 3, l = item & 63;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < SK_WAVES; ++w) v += sk_red[((w * XT + t) * 16 + 4 * q + r) * 64 + l];
+        sum[a][it][r] = v;
+      }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < ITEMS; ++it) {
+    const int item = tid + it * SK_WAVES * 64;
+    const int t = item >> 8, q = (item >> 6) & 3, l = item & 63;
+    const int64_t m = t * 32 + (l & 31);
+    const int64_t n = n0 + 8 * q + 4 * (l >> 5);
+    if (m >= M || n >= N) continue;
+    bf16_t out[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float g = sum[0][it][r];
+      out[r] = f32_to_bf16(EPI == 1 ? g / (1.f + __expf(-g)) * sum[NA - 1][it][r] : g);
+    }
+    bf16_t* yp = Y + m * ldy + n;
+    if (n + 3 < N && (((uintptr_t)yp) & 7) == 0) {
+      uint2 pk;
+      pk.x = out[0] | ((uint32_t)out[1] << 16);
+      pk.y = out[2] | ((uint32_t)out[3] << 16);
+      *(uint2*)yp = pk;
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n + r < N) yp[r] = out[r];
+    }
+  }
+}
+
+// -----------------------------------------------------------------------------------------
 // Large-tile variant for the big projections (M >= 256, K a multiple of 8):
 //   workgroup tile 256 (rows of x) x BN (rows of w) x 64, 8 waves as 4 (x) x 2 (w), 2 waves/SIMD;
 //   tiles go HBM/L2 -> LDS with direct-to-LDS loads (no staging registers) into two buffers,
@@ -555,6 +684,17 @@ __global__ __launch_bounds__(256) void wavedec_db4_kernel(const float* __restric
 
 using namespace mvpa;
 
+template <int EPI, int XT>
+static int launch_skinny(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, int64_t N, int64_t K,
+                         int64_t ldx, int64_t ldw, int64_t ldy, hipStream_t s) {
+  constexpr int lds = SK_WAVES * XT * 16 * 64 * (int)sizeof(float);
+  auto kern = linear_bf16_skinny_kernel<EPI, XT>;
+  if (lds > 64 * 1024)
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  hipLaunchKernelGGL(kern, dim3((unsigned)((N + 31) / 32)), dim3(SK_WAVES * 64), lds, s, x, w, y, M, N, K, ldx, ldw, ldy);
+  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+}
+
 extern "C" int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M, int64_t N,
                                 int64_t K, int64_t ldx, int64_t ldw, int64_t ldy,
                                 int32_t epilogue, void* stream) {
@@ -581,6 +721,13 @@ extern "C" int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M
     if (c256 <= c192 && c256 <= c128) return launch_big<256, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
     if (c192 <= c128) return launch_big<192, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
     return launch_big<128, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
+  }
+  if (M <= 128) {
+    // one decoding step's worth of rows: weight-read bound, spread over N/32 workgroups
+    return M <= 64 ? (epilogue == 1 ? launch_skinny<1, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+                                    : launch_skinny<0, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s))
+                   : (epilogue == 1 ? launch_skinny<1, 4>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+                                    : launch_skinny<0, 4>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s));
   }
   if (epilogue == 1) {
     dim3 grid((unsigned)((N + GBN / 2 - 1) / (GBN / 2)), (unsigned)((M + GBM - 1) / GBM));

@@ -1,3 +1,3 @@
-from .mvpa import MVPFormerGQAAttention, MVPFormerGQAFlashAttention
+from .mvpa import MvpaKVCache, MVPFormerGQAAttention, MVPFormerGQAFlashAttention
 
-__all__ = ["MVPFormerGQAAttention", "MVPFormerGQAFlashAttention"]
+__all__ = ["MvpaKVCache", "MVPFormerGQAAttention", "MVPFormerGQAFlashAttention"]

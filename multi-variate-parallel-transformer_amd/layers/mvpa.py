@@ -23,6 +23,56 @@ import torch
 import mvpa_hip
 
 
+class MvpaKVCache:
+    """Keys and values of one layer for step-by-step decoding, kept in place.
+
+    The `(k, v)` tuple of the reference's `layer_past` / `present` (layers/mvpa.py:314-321) grows
+    by a concatenation per step, i.e. a copy of the whole cache.  This holder owns two buffers
+    [B,Hkv,capacity,C,Dh] instead; a step writes its C new rows behind the cached ones and the
+    attention kernel reads the live time steps through a strided view.  At most `max_steps` time
+    steps are live (the new one included): once that many are cached the oldest drops out, which
+    is the sliding window of a stream - the biases are relative, so the remaining steps keep their
+    meaning.  The live steps move back to the front of the buffer once every `capacity -
+    max_steps + 1` steps, so the copy is amortised.  Pass it wherever `layer_past` goes; the layer
+    returns the same object as `present`."""
+
+    def __init__(self, batch: int, kv_heads: int, channels: int, head_dim: int, max_steps: int,
+                 dtype=torch.bfloat16, device="cuda", slack: Optional[int] = None):
+        if max_steps < 1:
+            raise ValueError("max_steps must be at least 1")
+        slack = max(1, max_steps // 4) if slack is None else max(0, int(slack))
+        self.max_steps = max_steps
+        self.capacity = max_steps + slack
+        self.k = torch.empty((batch, kv_heads, self.capacity, channels, head_dim), dtype=dtype, device=device)
+        self.v = torch.empty_like(self.k)
+        self.start = 0            # first live time step in the buffers
+        self.length = 0           # live time steps
+
+    def append(self, k_new: torch.Tensor, v_new: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Add one time step ([B,Hkv,C,Dh] each); returns views [B,Hkv,T,C,Dh] of the live steps."""
+        if self.length == self.max_steps:                 # the oldest step leaves the window
+            self.start += 1
+            self.length -= 1
+        if self.start + self.length == self.capacity:     # out of room: live steps back to the front
+            live_k = self.k[:, :, self.start:self.start + self.length].clone()
+            live_v = self.v[:, :, self.start:self.start + self.length].clone()
+            self.k[:, :, :self.length] = live_k
+            self.v[:, :, :self.length] = live_v
+            self.start = 0
+        pos = self.start + self.length
+        self.k[:, :, pos] = k_new
+        self.v[:, :, pos] = v_new
+        self.length += 1
+        return self.views()
+
+    def views(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        sl = slice(self.start, self.start + self.length)
+        return self.k[:, :, sl], self.v[:, :, sl]
+
+    def reset(self) -> None:
+        self.start = self.length = 0
+
+
 class _LoRALinear(torch.nn.Linear):
     """Bias-free Linear with low-rank adapters under the parameter names the reference's
     adapter library uses (lora_A, lora_B; layers/mvpa.py:43-62, 86-93).  `enable` marks which
@@ -243,16 +293,23 @@ class MVPFormerGQAAttention(torch.nn.Module):
                      head_mask, use_cache, window, layer_past):
         """One step of incremental decoding: hidden_states holds the new time step only
         ([B,1,C,E]), layer_past the keys and values of the steps before it ([B,Hkv,Tp,C,Dh] each,
-        as returned in `present`), positional_embedding all Tp+1 positions.  The new keys and
+        as returned in `present`, or an MvpaKVCache that is appended to in place),
+        positional_embedding all Tp+1 positions.  The new keys and
         values are appended along the TIME axis; the reference's cache path concatenates along
         dim -2, the channel axis (layers/mvpa.py:314-317), which does not continue the sequence,
         and is not reproduced."""
         bsz, t_new, c_len, e = hidden_states.shape
         h, hkv, dh, kv = self.num_heads, self.num_kv_heads, self.head_dim, self.embed_kv_dim
-        past_k, past_v = layer_past
+        cache = layer_past if isinstance(layer_past, MvpaKVCache) else None
+        if cache is not None:
+            t_past = min(cache.length, cache.max_steps - 1)
+            past_k = cache.k
+        else:
+            past_k, past_v = layer_past
+            t_past = past_k.shape[2]
         if t_new != 1:
             raise NotImplementedError("MVPA HIP layer: with layer_past, hidden_states holds one new time step")
-        t_len = past_k.shape[2] + 1
+        t_len = t_past + 1
         if positional_embedding.shape[-2] != t_len or past_k.shape[3] != c_len:
             raise ValueError("layer_past, positional_embedding and hidden_states disagree on T or C")
         dt = hidden_states.dtype
@@ -261,8 +318,13 @@ class MVPFormerGQAAttention(torch.nn.Module):
             q = qkv[:, :, :e].view(bsz, c_len, h, dh).permute(0, 2, 1, 3)           # [B,H,C,Dh]
             k_new = qkv[:, :, e:e + kv].view(bsz, c_len, hkv, dh).permute(0, 2, 1, 3)
             v_new = qkv[:, :, e + kv:].view(bsz, c_len, hkv, dh).permute(0, 2, 1, 3)
-            k = torch.cat([past_k.to(dt), k_new.unsqueeze(2)], dim=2)                # [B,Hkv,T,C,Dh]
-            v = torch.cat([past_v.to(dt), v_new.unsqueeze(2)], dim=2)
+            if cache is not None:
+                if cache.k.dtype != dt:
+                    raise ValueError("MvpaKVCache and hidden_states differ in dtype")
+                k, v = cache.append(k_new, v_new)                                    # views, in place
+            else:
+                k = torch.cat([past_k.to(dt), k_new.unsqueeze(2)], dim=2)            # [B,Hkv,T,C,Dh]
+                v = torch.cat([past_v.to(dt), v_new.unsqueeze(2)], dim=2)
             k_time, k_chan = self._key_tables(positional_embedding, channel_embedding)
             u, vb, z = (b.view(hkv, dh) for b in self.attn_bias.split(kv, dim=0))
             chan_valid, key_bias = None, None
@@ -272,7 +334,7 @@ class MVPFormerGQAAttention(torch.nn.Module):
                     key_bias = attention_mask.reshape(bsz, t_len * c_len).to(torch.float32)
             merged = torch.empty((bsz, c_len, h, dh), dtype=dt, device=hidden_states.device)
             mvpa_hip.mvpa_forward(
-                q, k.view(bsz, hkv, t_len * c_len, dh), v.view(bsz, hkv, t_len * c_len, dh),
+                q, k.reshape(bsz, hkv, t_len * c_len, dh), v.reshape(bsz, hkv, t_len * c_len, dh),
                 u, vb, z, k_time, k_chan, sm_scale=self._scale(), window=window, causal=True,
                 content=bool(self.global_att), chan_valid=chan_valid, key_bias=key_bias,
                 out=merged.permute(0, 2, 1, 3), last_step_only=True,
@@ -282,6 +344,8 @@ class MVPFormerGQAAttention(torch.nn.Module):
                     raise NotImplementedError("head_mask must hold one factor per head")
                 merged = merged * head_mask.to(dt).reshape(1, 1, h, 1)
             out = _linear(merged.view(bsz, 1, c_len, e), self.c_proj.weight)
+        if cache is not None:
+            return out, cache
         return out, ((k, v) if use_cache is True else None)
 
     def forward(

@@ -42,6 +42,33 @@ def mvpformer_s_windows_per_s(B: int = 4, C: int = 64, T: int = 64, seg: int = 5
                       f"segments of {seg} samples, bf16, random-init weights, synthetic iEEG"}
 
 
+def mvpformer_s_stream_step_ms(C: int = 64, T: int = 64, seg: int = 512, steps: int = 40) -> dict:
+    """One window of C channels as a stream: the steady-state cost of one new segment
+    (classify_step: encoder on the segment, one decoding step per block against caches holding the
+    last T segments) beside the full forward over the same T segments."""
+    model = build_mvpformer_s(seg, n_positions=T)
+    x = make_ieeg(1, C, T + steps, seg, seed=1).to("cuda:0")
+    past = None
+    for t in range(T):                       # fill the window; the caches slide from here on
+        _, past = model.classify_step(x[:, t], past)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t in range(T, T + steps):
+        _, past = model.classify_step(x[:, t], past)
+    torch.cuda.synchronize()
+    step_ms = (time.perf_counter() - t0) * 1e3 / steps
+    for _ in range(5):
+        model.classify(x[:, :T])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        model.classify(x[:, :T])
+    torch.cuda.synchronize()
+    full_ms = (time.perf_counter() - t0) * 1e3 / 10
+    return {"ms_per_segment": round(step_ms, 3), "ms_full_forward_same_window": round(full_ms, 3),
+            "config": f"MVPFormer-S, B=1 C={C}, window of {T} segments of {seg} samples, bf16"}
+
+
 def mvpformer_base_forward_ms(C: int = 128, T: int = 512, seg: int = 512, steps: int = 3,
                               warmup: int = 2) -> dict:
     """Random-init base-size classification forward (E2048 L24 H16 Hkv8 Dh128 n_inner5632, binary
@@ -66,6 +93,18 @@ def mvpformer_base_forward_ms(C: int = 128, T: int = 512, seg: int = 512, steps:
         res["ms_per_forward_fp8_qk" if fp8 else "ms_per_forward_bf16"] = round(
             (time.perf_counter() - t0) * 1e3 / steps, 1)
         logits[fp8] = y.float().cpu()
+        if not fp8:
+            # the same window as a stream: fill the caches, then time segments that slide it
+            past = None
+            for t in range(T):
+                _, past = model.classify_step(x[:, t], past)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for t in range(10):
+                _, past = model.classify_step(x[:, t], past)
+            torch.cuda.synchronize()
+            res["ms_per_streamed_segment_bf16"] = round((time.perf_counter() - t0) * 1e3 / 10, 2)
+            del past
         del model
         torch.cuda.empty_cache()
     res["logits_bf16"] = [round(v, 5) for v in logits[False].flatten().tolist()]

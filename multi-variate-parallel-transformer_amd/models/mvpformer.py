@@ -11,7 +11,7 @@ import torch
 from torch import nn
 
 import mvpa_hip
-from layers import MVPFormerGQAAttention, MVPFormerGQAFlashAttention
+from layers import MvpaKVCache, MVPFormerGQAAttention, MVPFormerGQAFlashAttention
 from models import BrainDecider, BrainEncoder, BrainModel
 from models.fftencoder import RMSNorm
 
@@ -178,14 +178,48 @@ class MVPFormerModel(nn.Module):
         if isinstance(module, (nn.Linear, nn.Embedding)):
             module.weight.data.normal_(mean=0.0, std=std)
 
+    def new_cache(self, batch: int, channels: int, max_steps: Optional[int] = None,
+                  dtype=torch.bfloat16, device="cuda"):
+        """One MvpaKVCache per block for step-by-step decoding (`past_key_values` of forward);
+        max_steps defaults to the number of position embeddings."""
+        max_steps = self.positional_embedding.num_embeddings if max_steps is None else max_steps
+        if max_steps > self.positional_embedding.num_embeddings:
+            raise IndexError("more time steps than embedding rows (n_positions)")
+        return tuple(MvpaKVCache(batch, self.num_kv_heads, channels, self.head_dim, max_steps,
+                                 dtype=dtype, device=device) for _ in self.h)
+
     @torch.no_grad()
-    def forward(self, input_ids=None, inputs_embeds=None, attention_mask=None, head_mask=None,
-                use_cache=None, output_attentions=None, **unused):
+    def forward(self, input_ids=None, past_key_values=None, inputs_embeds=None, attention_mask=None,
+                head_mask=None, use_cache=None, output_attentions=None, position_end=None, **unused):
+        """forward(inputs_embeds=[B,T,C,E]) -> last_hidden_state [B,T,C,E]; with use_cache also the
+        per-block `present`s, as the reference returns them in `past_key_values`
+        (models/mvpformer.py:290-398).  With past_key_values (one entry per block: the (k, v)
+        tuples a use_cache call returned, or the MvpaKVCache objects of new_cache) inputs_embeds
+        holds ONE new time step [B,1,C,E] that continues the cached sequence.
+
+        position_end: the T time steps use rows [position_end - T, position_end) of the position
+        embedding instead of rows [0, T).  Row j of the T rows in use stands for the distance
+        T-1-j between query and key step (layers/mvpa.py:223), so with rows [0, T) the row of a
+        given distance moves as a sequence grows; a stream keeps it in place by always ending at
+        the same row (MvpaKVCache entries imply position_end = their max_steps)."""
         if inputs_embeds is None:
             raise NotImplementedError
         if self.training:
             raise NotImplementedError("MVPFormer HIP stack: inference only; call .eval()")
+        use_cache = bool(use_cache)      # None = off whatever config.use_cache says: a tensor comes back
         bsz, t_len, c_len, _ = inputs_embeds.shape
+        if past_key_values is not None:
+            if len(past_key_values) != len(self.h):
+                raise ValueError("past_key_values needs one entry per block")
+            if t_len != 1:
+                raise NotImplementedError("with past_key_values, inputs_embeds holds one new time step")
+            first = past_key_values[0]
+            past_len = (min(first.length, first.max_steps - 1) if isinstance(first, MvpaKVCache)
+                        else first[0].shape[2])                  # models/mvpformer.py:241-245
+            t_len = past_len + 1
+            use_cache = True
+            if position_end is None and isinstance(first, MvpaKVCache):
+                position_end = first.max_steps
         if attention_mask is not None:                           # models/mvpformer.py:262-268
             dt = inputs_embeds.dtype
             attention_mask = attention_mask.view(bsz, -1)[:, None, None, :].to(dtype=dt)
@@ -194,19 +228,27 @@ class MVPFormerModel(nn.Module):
         # (models/mvpformer.py:282-283) are leading slices of the embedding tables
         if t_len > self.positional_embedding.num_embeddings or c_len > self.channel_embedding.num_embeddings:
             raise IndexError("more time steps / channels than embedding rows (n_positions / n_channels)")
-        position_embeds = self.positional_embedding.weight[:t_len][None]
+        pos_lo = 0 if position_end is None else position_end - t_len
+        if pos_lo < 0 or pos_lo + t_len > self.positional_embedding.num_embeddings:
+            raise IndexError("position_end leaves fewer than T rows of the position embedding")
+        position_embeds = self.positional_embedding.weight[pos_lo:pos_lo + t_len][None]
         channel_embeds = self.channel_embedding.weight[:c_len][None]
         hidden_states, normed = inputs_embeds, None
         n_layers = len(self.h)
+        presents = () if use_cache else None
         for i, block in enumerate(self.h):
             next_norm = self.h[i + 1].ln_1 if i + 1 < n_layers else self.ln_f
+            layer_past = past_key_values[i] if past_key_values is not None else None
             outputs, normed = block.forward_fused(hidden_states, normed, next_norm, position_embeds,
-                                                  channel_embeds, attention_mask=attention_mask,
-                                                  use_cache=False)
+                                                  channel_embeds, layer_past=layer_past,
+                                                  attention_mask=attention_mask, use_cache=use_cache)
             hidden_states = outputs[0]
+            if use_cache:
+                presents = presents + (outputs[1],)              # models/mvpformer.py:366-367
         if normed is None:                                       # no blocks
             normed = self.ln_f(hidden_states)
-        return normed.view(bsz, t_len, c_len, -1)
+        out = normed.view(bsz, inputs_embeds.shape[1], c_len, -1)
+        return (out, presents) if use_cache else out
 
 
 class MVPFormerHead(BrainDecider):
@@ -244,6 +286,34 @@ class HMVPFormer(BrainModel):
         input_embeds = out_enc.view(bsz, seg_n, ch, -1)
         out = self.mvpformer(inputs_embeds=input_embeds, attention_mask=attention_mask)
         return out, input_embeds
+
+    @torch.no_grad()
+    def classify_step(self, segment: torch.Tensor, past=None, max_steps: Optional[int] = None):
+        """Classification score of a stream, one segment at a time: segment [B, ch, len] is the
+        newest one, `past` what the previous call returned (None at the start of a stream).
+        Returns (logits, past).  Each call runs the encoder on the new segment only and one
+        decoding step of every block against the cached keys and values; as long as the stream is
+        no longer than max_steps (default: the number of position embeddings) every step sees what
+        the full forward over the segments so far sees when its position rows end at max_steps
+        (forward(position_end=max_steps)); at step max_steps that is classify() on the whole
+        window.  After that the oldest segment drops out of the attention window at every step."""
+        bsz, ch, seg = segment.shape
+        embeds = self.encoder(segment.reshape(bsz * ch, seg)).view(bsz, 1, ch, -1)
+        if past is None:
+            past = self.mvpformer.new_cache(bsz, ch, max_steps, dtype=embeds.dtype, device=embeds.device)
+            out, past = self._first_step(embeds, past)
+        else:
+            out, past = self.mvpformer(inputs_embeds=embeds, past_key_values=past)
+        return self.head(out[:, -1].float().mean(dim=1).to(out.dtype)), past
+
+    def _first_step(self, embeds, caches):
+        """The first segment of a stream through the full forward; its keys and values seed the
+        caches."""
+        out, presents = self.mvpformer(inputs_embeds=embeds, use_cache=True,
+                                       position_end=caches[0].max_steps)
+        for cache, (k, v) in zip(caches, presents):
+            cache.append(k[:, :, 0], v[:, :, 0])
+        return out, caches
 
     @torch.no_grad()
     def predict_next_segment(self, batch: torch.Tensor):

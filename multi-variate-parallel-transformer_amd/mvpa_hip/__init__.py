@@ -129,7 +129,14 @@ def _check(status: int) -> None:
     raise MvpaError(status, text)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """Handle of torch's current stream on the current device (the raw getter skips building a
+    Stream object: this runs once per launch)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 

@@ -10,7 +10,10 @@ pytestmark = pytest.mark.gpu
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 200, 72), (1000, 768, 550), (64, 2304, 768), (17, 33, 8),
                                    (2048, 768, 768), (1024, 1280, 768), (600, 130, 72), (4100, 2048, 552),
-                                   (16384, 768, 1728)])
+                                   (16384, 768, 1728),
+                                   # at most 128 rows: the K-split kernel of a decoding step
+                                   (64, 1280, 768), (64, 768, 1728), (33, 130, 550), (1, 768, 768), (20, 100, 72),
+                                   (32, 2048, 5632), (128, 2048, 2048), (100, 3072, 2048), (65, 96, 24)])
 def test_linear_bf16(M, N, K):
     g = torch.Generator().manual_seed(M + N + K)
     ldk = (K + 7) // 8 * 8
@@ -26,7 +29,8 @@ def test_linear_bf16(M, N, K):
     assert (y.double() - ref).abs().max().item() <= 2 ** -8 * ref.abs().max().item() + 1e-6
 
 
-@pytest.mark.parametrize("M,N,K", [(200, 96, 64), (1024, 1728, 768), (700, 200, 136), (4096, 64, 768)])
+@pytest.mark.parametrize("M,N,K", [(200, 96, 64), (1024, 1728, 768), (700, 200, 136), (4096, 64, 768),
+                                   (64, 1728, 768), (20, 70, 136), (40, 33, 552), (7, 5632, 2048), (128, 5632, 2048), (97, 40, 72)])
 def test_linear_gated(M, N, K):
     g = torch.Generator().manual_seed(3)
     x = torch.randn(M, K, generator=g).bfloat16()
