@@ -2,7 +2,7 @@
 """Benchmark of the MVPA forward hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3] [--no-cpu] [--no-model]
-                    [--no-backward] [--base-model] [--copy-probe]
+                    [--no-stream] [--no-backward] [--base-model] [--copy-probe]
 
 A step is one fused MVPA forward (one kernel launch) over one batch of synthetic inputs that
 are already resident in HBM.  The default workload is the configuration the headline metric
@@ -103,6 +103,7 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-model", action="store_true", help="skip the MVPFormer-S forward leg")
+    ap.add_argument("--no-stream", action="store_true", help="skip the MVPFormer-S streamed-segment leg")
     ap.add_argument("--no-backward", action="store_true", help="skip the MVPA backward leg")
     ap.add_argument("--base-model", action="store_true",
                     help="also time the base-size classification forward (B1 C128 T512, bf16 and fp8 QK^T)")
@@ -196,8 +197,9 @@ def main():
         try:
             from models.bench_model import mvpformer_s_windows_per_s
             line["mvpformer_s"] = mvpformer_s_windows_per_s()
-            from models.bench_model import mvpformer_s_stream_step_ms
-            line["mvpformer_s_stream"] = mvpformer_s_stream_step_ms()
+            if not args.no_stream:
+                from models.bench_model import mvpformer_s_stream_step_ms
+                line["mvpformer_s_stream"] = mvpformer_s_stream_step_ms()
         except ImportError:
             line["mvpformer_s"] = None
     if args.base_model:
