@@ -2,7 +2,7 @@
 """Benchmark of the MVPA forward hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3] [--no-cpu] [--no-model]
-                    [--no-stream] [--no-backward] [--base-model] [--copy-probe]
+                    [--no-stream] [--no-backward] [--base-model] [--copy-probe] [--no-mfma-probe]
 
 A step is one fused MVPA forward (one kernel launch) over one batch of synthetic inputs that
 are already resident in HBM.  The default workload is the configuration the headline metric
@@ -13,7 +13,8 @@ restatement of the reference PyTorch path on this box's host cores).  Beside the
 of `value`: `backward` (one mvpa_backward call on the same workload), `mvpformer_s` (the
 MVPFormer-S forward in windows per second), `mvpformer_s_stream` (one new segment of a stream
 against cached keys and values, beside the full forward over the same window) and, on request,
-`mvpformer_base`.
+`mvpformer_base` and `mfma_probe` (what a stream of nothing but bf16 MFMAs reaches on this box,
+on smooth and on random operands).
 """
 from __future__ import annotations
 
@@ -103,6 +104,8 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-model", action="store_true", help="skip the MVPFormer-S forward leg")
+    ap.add_argument("--no-mfma-probe", action="store_true",
+                    help="skip the pure MFMA stream on smooth and on random operands")
     ap.add_argument("--no-stream", action="store_true", help="skip the MVPFormer-S streamed-segment leg")
     ap.add_argument("--no-backward", action="store_true", help="skip the MVPA backward leg")
     ap.add_argument("--base-model", action="store_true",
@@ -193,6 +196,11 @@ def main():
         line["backward"] = {"ms_per_step": round(ev0.elapsed_time(ev1) / n_bwd, 4), "steps": n_bwd,
                             "kernels": "mvpa_bwd_query_mfma_kernel + mvpa_bwd_key_mfma_kernel",
                             "outputs": "dq (content share), dk, dv, dbias_time, dbias_chan (fp32)"}
+    if not args.no_mfma_probe:
+        line["mfma_probe"] = {
+            "smooth_operands_tflops": round(mvpa_hip.mfma_probe_tflops(False), 1),
+            "random_operands_tflops": round(mvpa_hip.mfma_probe_tflops(True), 1),
+            "what": "a stream of nothing but v_mfma_f32_32x32x16_bf16 on every SIMD, two waves each"}
     if not args.no_model:
         try:
             from models.bench_model import mvpformer_s_windows_per_s
@@ -204,7 +212,7 @@ def main():
             line["mvpformer_s"] = None
     if args.base_model:
         from models.bench_model import mvpformer_base_forward_ms
-        line["mvpformer_base"] = mvpformer_base_forward_ms()
+        line["mvpformer_base"] = mvpformer_base_forward_ms(stream=not args.no_stream)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(line))

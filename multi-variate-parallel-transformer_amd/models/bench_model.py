@@ -70,7 +70,7 @@ def mvpformer_s_stream_step_ms(C: int = 64, T: int = 64, seg: int = 512, steps: 
 
 
 def mvpformer_base_forward_ms(C: int = 128, T: int = 512, seg: int = 512, steps: int = 3,
-                              warmup: int = 2) -> dict:
+                              warmup: int = 2, stream: bool = True) -> dict:
     """Random-init base-size classification forward (E2048 L24 H16 Hkv8 Dh128 n_inner5632, binary
     head) on one window of C channels x T segments: bf16, then fp8 e4m3 QK^T."""
     from models.configs import MVPFORMER_BASE
@@ -93,7 +93,7 @@ def mvpformer_base_forward_ms(C: int = 128, T: int = 512, seg: int = 512, steps:
         res["ms_per_forward_fp8_qk" if fp8 else "ms_per_forward_bf16"] = round(
             (time.perf_counter() - t0) * 1e3 / steps, 1)
         logits[fp8] = y.float().cpu()
-        if not fp8:
+        if not fp8 and stream:
             # the same window as a stream: fill the caches, then time segments that slide it
             past = None
             for t in range(T):
