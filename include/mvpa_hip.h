@@ -61,6 +61,12 @@ enum {
                                    decoding against cached keys and values (the use the
                                    layer_past / use_cache arguments of layers/mvpa.py:314-321
                                    are for).  Needs MVPA_FLAG_CAUSAL.                        */
+#define MVPA_FLAG_RING 64u      /* with MVPA_FLAG_LAST_STEP on the bf16 MFMA kernel: the T time
+                                   steps of k and v are the slots of a ring; *ring_head (device
+                                   memory, read by the kernel) is the slot of the newest step and
+                                   slot s holds the step (ring_head - s) mod T steps older.  Lets
+                                   a caller keep a sliding window of keys and values in place and
+                                   replay one decoding step as a fixed sequence of launches.  */
 
 /*
  * Arguments of the fused MVPA forward.  Replaces the pair
@@ -117,6 +123,7 @@ typedef struct mvpa_fwd_args {
                                 layers/mvpa.py:314-321, re-enters the full kernel).           */
   int32_t n_split;           /* 0 or 1 = no split; at most T                              */
   int32_t reserved0;
+  const int32_t* ring_head;  /* MVPA_FLAG_RING: device pointer to the newest slot, in [0, T)  */
 } mvpa_fwd_args;
 
 /* ABI version of the loaded library. */

@@ -50,6 +50,10 @@ extern "C" int mvpa_validate(const mvpa_fwd_args* a) {
     if (a->dtype != MVPA_BF16) return MVPA_ERR_UNSUPPORTED;
     if (!a->fp8_q_scale || !a->fp8_k_scale) return MVPA_ERR_NULL;
   }
+  if (a->flags & MVPA_FLAG_RING) {
+    if (!(a->flags & MVPA_FLAG_LAST_STEP)) return MVPA_ERR_UNSUPPORTED;
+    if (!a->ring_head) return MVPA_ERR_NULL;
+  }
   if (a->n_split < 0 || a->n_split > a->T) return MVPA_ERR_SHAPE;
   if (a->n_split > 1) {
     if (!(a->flags & MVPA_FLAG_LAST_STEP)) return MVPA_ERR_UNSUPPORTED;
@@ -88,6 +92,6 @@ extern "C" int mvpa_forward(const mvpa_fwd_args* a, void* stream) {
   const int sel = mvpa_select_kernel(a);
   if (sel < 0) return sel;
   if (sel == MVPA_KERNEL_MFMA) return mvpa_launch_mfma(a, (hipStream_t)stream);
-  if (a->flags & MVPA_FLAG_FP8_QK) return MVPA_ERR_UNSUPPORTED;
+  if (a->flags & (MVPA_FLAG_FP8_QK | MVPA_FLAG_RING)) return MVPA_ERR_UNSUPPORTED;
   return mvpa_launch_generic(a, (hipStream_t)stream);
 }

@@ -222,7 +222,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   // of the kernel just takes T_ steps from pointers moved on by t_lo; its normalised output and
   // log-sum-exp go to the workspace, from where mvpa_split_merge_kernel combines the runs.
   // (RUNS: a build of the kernel of its own, so that the usual launch carries none of this.)
-  const int n_split = RUNS ? a.n_split : 1;
+  const int n_split = RUNS ? max(a.n_split, 1) : 1;
   const int split_len = (a.T + n_split - 1) / n_split;
   const int run = n_split > 1 ? (int)blockIdx.x / (a.B * a.H) : 0;
   const int t_lo = run * split_len;
@@ -311,7 +311,10 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
                        (int64_t)(active ? (last_only ? 0 : tq * C_) + min(cq, C_ - 1) : 0) * a.q_stride_n;
   const bf16_t* kbase = (const bf16_t*)a.k + b * a.k_stride_b + g * a.k_stride_h + (int64_t)t_lo * C_ * a.k_stride_n;
   const bf16_t* vbase = (const bf16_t*)a.v + b * a.v_stride_b + g * a.v_stride_h + (int64_t)t_lo * C_ * a.v_stride_n;
-  const bf16_t* ktime = (const bf16_t*)a.k_time + ((int64_t)g * a.T + t_lo) * DH;
+  // MVPA_FLAG_RING: slot s holds the step whose table row is (s + ring_rot) mod T
+  const bool ring = RUNS && (a.flags & MVPA_FLAG_RING);
+  const int ring_rot = ring ? a.T - 1 - __builtin_amdgcn_readfirstlane(*a.ring_head) : 0;
+  const bf16_t* ktime = (const bf16_t*)a.k_time + ((int64_t)g * a.T + (ring ? 0 : t_lo)) * DH;
   const bf16_t* kchan = (const bf16_t*)a.k_chan + (int64_t)g * C_ * DH;
   const bf16_t* bu = (const bf16_t*)a.bias_u + g * DH;
   const bf16_t* bv = (const bf16_t*)a.bias_v + g * DH;
@@ -534,7 +537,8 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 #pragma unroll
     for (int i = 0; i < 16; ++i) stc[i] = 0.f;
     if (has_time) {
-      const int j = min(j0 + ln, T_ - 1);          // rows past T-1 belong to tk > tq: never used
+      int j = min(j0 + ln, T_ - 1);                // rows past T-1 belong to tk > tq: never used
+      if (ring) j = (t_lo + tk + ln + ring_rot) % a.T;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const u32x4 rr = *(const u32x4*)(ktime + (int64_t)j * DH + ks * 16 + hh * 8);
@@ -897,7 +901,8 @@ static int launch_one(const mvpa_fwd_args* a, hipStream_t stream) {
   static_assert(G::LDS_BYTES <= 160 * 1024, "LDS budget");
   const bool last = a->flags & MVPA_FLAG_LAST_STEP;
   const int n_split = (last && a->split_ws && a->n_split > 1) ? a->n_split : 1;
-  auto kern = n_split > 1 ? mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH, true>
+  const bool ring = last && (a->flags & MVPA_FLAG_RING);
+  auto kern = (n_split > 1 || ring) ? mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH, true>
                           : mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH, false>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)G::LDS_BYTES);

@@ -18,6 +18,7 @@ LIB_PATH = os.path.join(_HERE, "libmvpa_hip.so")
 MVPA_F32, MVPA_BF16 = 0, 1
 KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA = 0, 1, 2
 FLAG_LAST_STEP = 32
+FLAG_RING = 64
 FLAG_CAUSAL, FLAG_CONTENT, FLAG_TIME_BIAS, FLAG_CHAN_BIAS, FLAG_FP8_QK = 1, 2, 4, 8, 16
 
 ERR_HEAD_DIM, ERR_HEAD_RATIO, ERR_CTX, ERR_SHAPE = -2, -3, -4, -5
@@ -43,6 +44,7 @@ class MvpaFwdArgs(ctypes.Structure):
         ("lse", ctypes.c_void_p),
         ("fp8_q_scale", ctypes.c_void_p), ("fp8_k_scale", ctypes.c_void_p),
         ("split_ws", ctypes.c_void_p), ("n_split", ctypes.c_int32), ("reserved0", ctypes.c_int32),
+        ("ring_head", ctypes.c_void_p),
     ]
 
 
@@ -161,7 +163,8 @@ def _need_cuda(*tensors) -> None:
 def make_args(q, k, v, out, u, vb, z, k_time, k_chan, *, T: int, C: int,
               sm_scale: float, window: int = 10, flags: int = 15,
               chan_valid=None, key_bias=None, lse=None, kernel: int = KERNEL_AUTO,
-              fp8_q_scale=None, fp8_k_scale=None, split_ws=None, n_split: int = 0) -> MvpaFwdArgs:
+              fp8_q_scale=None, fp8_k_scale=None, split_ws=None, n_split: int = 0,
+              ring_head=None) -> MvpaFwdArgs:
     """Fill the argument block from [B,H,N,Dh]-indexable tensors (any strides with a unit
     last stride).  Accepts meta/CPU tensors too so validation can be exercised without a GPU."""
     a = MvpaFwdArgs()
@@ -190,6 +193,7 @@ def make_args(q, k, v, out, u, vb, z, k_time, k_chan, *, T: int, C: int,
     a.fp8_k_scale = fp8_k_scale.data_ptr() if fp8_k_scale is not None else None
     a.split_ws = split_ws.data_ptr() if split_ws is not None else None
     a.n_split = n_split
+    a.ring_head = ring_head.data_ptr() if ring_head is not None else None
     return a
 
 
@@ -210,7 +214,7 @@ def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float]
                  key_bias: Optional[torch.Tensor] = None, return_lse: bool = False,
                  kernel: int = KERNEL_AUTO, out: Optional[torch.Tensor] = None,
                  fp8_qk: bool = False, last_step_only: bool = False,
-                 key_splits: Optional[int] = None):
+                 key_splits: Optional[int] = None, ring_head: Optional[torch.Tensor] = None):
     """Fused MVPA forward on the GPU.
 
     q [B,H,N,Dh]; k, v [B,Hkv,N,Dh]; u, vb, z [Hkv,Dh]; k_time [Hkv,T,Dh]; k_chan [Hkv,C,Dh];
@@ -222,6 +226,10 @@ def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float]
     incremental decoding.  key_splits: the number of runs the T key steps are cut into, each run
     on workgroups of its own, merged by a second kernel (bf16 MFMA kernel only; None picks
     default_key_splits, 1 keeps one workgroup per (b, h) on the whole cache).
+    ring_head (with last_step_only, bf16): a one-element int32 device tensor; the T time steps of
+    k and v are then the slots of a ring, slot ring_head holding the newest step and slot s the one
+    (ring_head - s) mod T steps older.  The kernel reads it from device memory, so a captured
+    graph of the call follows a cache that moves on.
     """
     lib = load_library()
     _need_cuda(q, k, v, u, vb, z, k_time, k_chan, chan_valid, key_bias)
@@ -247,7 +255,13 @@ def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float]
     lse = torch.empty((B, H, Nq), dtype=torch.float32, device=q.device) if return_lse else None
     flags = ((FLAG_CAUSAL if causal else 0) | (FLAG_CONTENT if content else 0) |
              (FLAG_TIME_BIAS if time_bias else 0) | (FLAG_CHAN_BIAS if chan_bias else 0) |
-             (FLAG_FP8_QK if fp8_qk else 0) | (FLAG_LAST_STEP if last_step_only else 0))
+             (FLAG_FP8_QK if fp8_qk else 0) | (FLAG_LAST_STEP if last_step_only else 0) |
+             (FLAG_RING if ring_head is not None else 0))
+    if ring_head is not None:
+        if not last_step_only:
+            raise ValueError("ring_head needs last_step_only")
+        if ring_head.dtype != torch.int32 or not ring_head.is_cuda or ring_head.numel() != 1:
+            raise TypeError("ring_head: one int32 element on the GPU")
     s = (1.0 / Dh ** 0.5) if sm_scale is None else float(sm_scale)
     q_scale = k_scale = None
     if fp8_qk:
@@ -259,7 +273,7 @@ def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float]
         k_scale = (k.float().abs().amax(dim=(0, 2, 3)) / 224.0).clamp_min(1e-20).contiguous()
     a = make_args(q, k, v, out, u, vb, z, k_time, k_chan, T=T, C=C, sm_scale=s, window=window,
                   flags=flags, chan_valid=chan_valid, key_bias=key_bias, lse=lse, kernel=kernel,
-                  fp8_q_scale=q_scale, fp8_k_scale=k_scale)
+                  fp8_q_scale=q_scale, fp8_k_scale=k_scale, ring_head=ring_head)
     if last_step_only and lib.mvpa_select_kernel(ctypes.byref(a)) == KERNEL_MFMA:
         n = default_key_splits(B, H, T) if key_splits is None else int(key_splits)
         if n > 1:

@@ -424,3 +424,41 @@ def test_key_splits_rejected_where_they_make_no_sense():
         mvpa_hip.mvpa_forward(d.q[:, :, -8:], d.k, d.v, *tabs, last_step_only=True, key_splits=4)
     with pytest.raises(AssertionError):    # more runs than key steps
         mvpa_hip.mvpa_forward(d.q[:, :, -8:], d.k, d.v, *tabs, last_step_only=True, key_splits=7)
+
+
+@pytest.mark.parametrize("cfg,n,head", [
+    (dict(B=2, C=64, T=17, H=4, Hkv=2, Dh=64), 1, 5),
+    (dict(B=2, C=64, T=40, H=4, Hkv=2, Dh=64), 4, 39),      # head on the last slot: ring order = time order
+    (dict(B=1, C=117, T=45, H=2, Hkv=2, Dh=64), 4, 0),
+    (dict(B=1, C=128, T=70, H=2, Hkv=1, Dh=128), 5, 33),    # runs longer than a 32-step slab, wrap inside a run
+    (dict(B=3, C=8, T=24, H=2, Hkv=1, Dh=32), None, 23),
+])
+def test_last_step_on_a_ring_of_slots(cfg, n, head):
+    """MVPA_FLAG_RING: the cached time steps sit in the slots of a ring, the newest one in slot
+    `head` (read from device memory by the kernel).  Same result as the same steps in time order,
+    to bf16 rounding (the key steps are visited in another order)."""
+    inp = make_mvpa_inputs(seed=29, qkv_unit=True, **cfg).to("cuda", torch.bfloat16)
+    B, C, T, Hkv, Dh = cfg["B"], cfg["C"], cfg["T"], cfg["Hkv"], cfg["Dh"]
+    tabs = (inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan)
+    q_last = inp.q[:, :, -C:]
+    ref, lse_ref = mvpa_hip.mvpa_forward(q_last, inp.k, inp.v, *tabs, return_lse=True, last_step_only=True, key_splits=1)
+    # slot s holds the step that is (head - s) mod T steps older than the newest one (time index T-1)
+    slot = torch.arange(T, device="cuda")
+    step_of_slot = T - 1 - (head - slot) % T
+    k5, v5 = inp.k.view(B, Hkv, T, C, Dh), inp.v.view(B, Hkv, T, C, Dh)
+    k_ring = k5[:, :, step_of_slot].reshape(B, Hkv, T * C, Dh).contiguous()
+    v_ring = v5[:, :, step_of_slot].reshape(B, Hkv, T * C, Dh).contiguous()
+    head_t = torch.tensor([head], dtype=torch.int32, device="cuda")
+    got, lse_got = mvpa_hip.mvpa_forward(q_last, k_ring, v_ring, *tabs, return_lse=True, last_step_only=True,
+                                         key_splits=n, ring_head=head_t)
+    err = (got.float() - ref.float()).abs().max().item()
+    rel = ((got.float() - ref.float()).norm() / ref.float().norm()).item()
+    assert err <= 2e-2 and rel <= 5e-3, (err, rel)
+    assert (lse_got - lse_ref).abs().max().item() <= 1e-3
+    # the head is read at run time: moving it (and the slots with it) needs no new arguments
+    head_t.fill_((head + 3) % T)
+    step_of_slot = T - 1 - ((head + 3) % T - slot) % T
+    k_ring.copy_(k5[:, :, step_of_slot].reshape(B, Hkv, T * C, Dh))
+    v_ring.copy_(v5[:, :, step_of_slot].reshape(B, Hkv, T * C, Dh))
+    got2 = mvpa_hip.mvpa_forward(q_last, k_ring, v_ring, *tabs, last_step_only=True, key_splits=n, ring_head=head_t)
+    assert (got2.float() - ref.float()).abs().max().item() <= 2e-2
