@@ -1,3 +1,3 @@
-from .mvpa import MvpaKVCache, MVPFormerGQAAttention, MVPFormerGQAFlashAttention
+from .mvpa import MvpaKVCache, MvpaRingCache, MVPFormerGQAAttention, MVPFormerGQAFlashAttention
 
-__all__ = ["MvpaKVCache", "MVPFormerGQAAttention", "MVPFormerGQAFlashAttention"]
+__all__ = ["MvpaKVCache", "MvpaRingCache", "MVPFormerGQAAttention", "MVPFormerGQAFlashAttention"]

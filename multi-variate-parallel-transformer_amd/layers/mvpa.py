@@ -73,6 +73,37 @@ class MvpaKVCache:
         self.start = self.length = 0
 
 
+class MvpaRingCache:
+    """A full window of keys and values as a ring: `steps` slots [B,Hkv,steps,C,Dh], the newest
+    time step in slot `head` (a device counter), the one before it in slot head-1, and so on
+    around the ring.  Appending overwrites the oldest slot, so nothing ever moves, every pointer
+    stays where it is and the position of the newest step lives in device memory: one decoding step
+    is then a fixed sequence of launches that a HIP graph can replay (MVPA_FLAG_RING tells the
+    attention kernel which table row each slot stands for).  Always full: build it from a filled
+    MvpaKVCache with `from_cache`."""
+
+    def __init__(self, k: torch.Tensor, v: torch.Tensor, head: int):
+        self.k, self.v = k, v                    # [B,Hkv,steps,C,Dh]
+        self.steps = k.shape[2]
+        self.head64 = torch.tensor([head], dtype=torch.int64, device=k.device)
+        self.head32 = torch.tensor([head], dtype=torch.int32, device=k.device)
+
+    @classmethod
+    def from_cache(cls, cache: "MvpaKVCache") -> "MvpaRingCache":
+        if cache.length != cache.max_steps:
+            raise ValueError("the window is not full yet: keep appending to the MvpaKVCache")
+        k, v = cache.views()
+        return cls(k.clone(), v.clone(), cache.max_steps - 1)      # time order: the newest step is last
+
+    def append(self, k_new: torch.Tensor, v_new: torch.Tensor) -> None:
+        """Overwrite the oldest slot with one new time step ([B,Hkv,C,Dh] each).  Device-side only:
+        may run under graph capture."""
+        self.head64.add_(1).remainder_(self.steps)
+        self.head32.copy_(self.head64)
+        self.k.index_copy_(2, self.head64, k_new.unsqueeze(2))
+        self.v.index_copy_(2, self.head64, v_new.unsqueeze(2))
+
+
 class _LoRALinear(torch.nn.Linear):
     """Bias-free Linear with low-rank adapters under the parameter names the reference's
     adapter library uses (lora_A, lora_B; layers/mvpa.py:43-62, 86-93).  `enable` marks which
@@ -301,7 +332,11 @@ class MVPFormerGQAAttention(torch.nn.Module):
         bsz, t_new, c_len, e = hidden_states.shape
         h, hkv, dh, kv = self.num_heads, self.num_kv_heads, self.head_dim, self.embed_kv_dim
         cache = layer_past if isinstance(layer_past, MvpaKVCache) else None
-        if cache is not None:
+        ring = layer_past if isinstance(layer_past, MvpaRingCache) else None
+        if ring is not None:
+            t_past = ring.steps - 1
+            past_k = ring.k
+        elif cache is not None:
             t_past = min(cache.length, cache.max_steps - 1)
             past_k = cache.k
         else:
@@ -318,7 +353,12 @@ class MVPFormerGQAAttention(torch.nn.Module):
             q = qkv[:, :, :e].view(bsz, c_len, h, dh).permute(0, 2, 1, 3)           # [B,H,C,Dh]
             k_new = qkv[:, :, e:e + kv].view(bsz, c_len, hkv, dh).permute(0, 2, 1, 3)
             v_new = qkv[:, :, e + kv:].view(bsz, c_len, hkv, dh).permute(0, 2, 1, 3)
-            if cache is not None:
+            if ring is not None:
+                if ring.k.dtype != dt:
+                    raise ValueError("MvpaRingCache and hidden_states differ in dtype")
+                ring.append(k_new, v_new)                                            # oldest slot overwritten
+                k, v = ring.k, ring.v
+            elif cache is not None:
                 if cache.k.dtype != dt:
                     raise ValueError("MvpaKVCache and hidden_states differ in dtype")
                 k, v = cache.append(k_new, v_new)                                    # views, in place
@@ -338,12 +378,15 @@ class MVPFormerGQAAttention(torch.nn.Module):
                 u, vb, z, k_time, k_chan, sm_scale=self._scale(), window=window, causal=True,
                 content=bool(self.global_att), chan_valid=chan_valid, key_bias=key_bias,
                 out=merged.permute(0, 2, 1, 3), last_step_only=True,
+                ring_head=ring.head32 if ring is not None else None,
                 fp8_qk=self.fp8_qk and dt == torch.bfloat16 and key_bias is None)
             if head_mask is not None:
                 if head_mask.numel() != h:
                     raise NotImplementedError("head_mask must hold one factor per head")
                 merged = merged * head_mask.to(dt).reshape(1, 1, h, 1)
             out = _linear(merged.view(bsz, 1, c_len, e), self.c_proj.weight)
+        if ring is not None:
+            return out, ring
         if cache is not None:
             return out, cache
         return out, ((k, v) if use_cache is True else None)

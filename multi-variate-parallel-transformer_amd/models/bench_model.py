@@ -57,6 +57,16 @@ def mvpformer_s_stream_step_ms(C: int = 64, T: int = 64, seg: int = 512, steps: 
         _, past = model.classify_step(x[:, t], past)
     torch.cuda.synchronize()
     step_ms = (time.perf_counter() - t0) * 1e3 / steps
+    # the same step on ring caches, replayed as one HIP graph
+    graph_step = model.capture_stream(past, x[:, 0])
+    for t in range(5):
+        graph_step(x[:, t])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t in range(steps):
+        graph_step(x[:, T + t])
+    torch.cuda.synchronize()
+    graph_ms = (time.perf_counter() - t0) * 1e3 / steps
     for _ in range(5):
         model.classify(x[:, :T])
     torch.cuda.synchronize()
@@ -65,7 +75,8 @@ def mvpformer_s_stream_step_ms(C: int = 64, T: int = 64, seg: int = 512, steps: 
         model.classify(x[:, :T])
     torch.cuda.synchronize()
     full_ms = (time.perf_counter() - t0) * 1e3 / 10
-    return {"ms_per_segment": round(step_ms, 3), "ms_full_forward_same_window": round(full_ms, 3),
+    return {"ms_per_segment": round(step_ms, 3), "ms_per_segment_graph_replay": round(graph_ms, 3),
+            "ms_full_forward_same_window": round(full_ms, 3),
             "config": f"MVPFormer-S, B=1 C={C}, window of {T} segments of {seg} samples, bf16"}
 
 
@@ -104,7 +115,16 @@ def mvpformer_base_forward_ms(C: int = 128, T: int = 512, seg: int = 512, steps:
                 _, past = model.classify_step(x[:, t], past)
             torch.cuda.synchronize()
             res["ms_per_streamed_segment_bf16"] = round((time.perf_counter() - t0) * 1e3 / 10, 2)
-            del past
+            graph_step = model.capture_stream(past, x[:, 0])
+            for t in range(3):
+                graph_step(x[:, t])
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for t in range(10):
+                graph_step(x[:, t])
+            torch.cuda.synchronize()
+            res["ms_per_streamed_segment_graph_replay_bf16"] = round((time.perf_counter() - t0) * 1e3 / 10, 2)
+            del past, graph_step
         del model
         torch.cuda.empty_cache()
     res["logits_bf16"] = [round(v, 5) for v in logits[False].flatten().tolist()]

@@ -11,7 +11,7 @@ import torch
 from torch import nn
 
 import mvpa_hip
-from layers import MvpaKVCache, MVPFormerGQAAttention, MVPFormerGQAFlashAttention
+from layers import MvpaKVCache, MvpaRingCache, MVPFormerGQAAttention, MVPFormerGQAFlashAttention
 from models import BrainDecider, BrainEncoder, BrainModel
 from models.fftencoder import RMSNorm
 
@@ -215,11 +215,14 @@ class MVPFormerModel(nn.Module):
                 raise NotImplementedError("with past_key_values, inputs_embeds holds one new time step")
             first = past_key_values[0]
             past_len = (min(first.length, first.max_steps - 1) if isinstance(first, MvpaKVCache)
+                        else first.steps - 1 if isinstance(first, MvpaRingCache)
                         else first[0].shape[2])                  # models/mvpformer.py:241-245
             t_len = past_len + 1
             use_cache = True
             if position_end is None and isinstance(first, MvpaKVCache):
                 position_end = first.max_steps
+            if position_end is None and isinstance(first, MvpaRingCache):
+                position_end = first.steps
         if attention_mask is not None:                           # models/mvpformer.py:262-268
             dt = inputs_embeds.dtype
             attention_mask = attention_mask.view(bsz, -1)[:, None, None, :].to(dtype=dt)
@@ -305,6 +308,47 @@ class HMVPFormer(BrainModel):
         else:
             out, past = self.mvpformer(inputs_embeds=embeds, past_key_values=past)
         return self.head(out[:, -1].float().mean(dim=1).to(out.dtype)), past
+
+    def capture_stream(self, past, segment_like: torch.Tensor):
+        """Turn a stream whose window is full into a replayable HIP graph.  `past` is what
+        classify_step returned once max_steps segments were in (MvpaKVCache per block);
+        segment_like a tensor shaped like one segment batch [B, ch, len].  Returns a callable
+        step(segment) -> logits that copies the segment into a fixed buffer and replays the graph
+        of one classify_step on ring caches (the caches are copied; `past` is left alone).  The
+        returned logits tensor is overwritten by the next call."""
+        rings = tuple(MvpaRingCache.from_cache(c) for c in past)
+        inp = segment_like.clone()
+
+        def one_step():
+            bsz, ch, seg = inp.shape
+            embeds = self.encoder(inp.reshape(bsz * ch, seg)).view(bsz, 1, ch, -1)
+            out, _ = self.mvpformer(inputs_embeds=embeds, past_key_values=rings)
+            return self.head(out[:, -1].float().mean(dim=1).to(out.dtype))
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        saved = [(r.k.clone(), r.v.clone(), r.head64.clone(), r.head32.clone()) for r in rings]
+        with torch.cuda.stream(side):
+            for _ in range(2):                      # warm-up: fills every host-side cache of the path
+                one_step()
+        torch.cuda.current_stream().wait_stream(side)
+        for r, (k0, v0, h64, h32) in zip(rings, saved):     # the warm-up steps wrote into the rings
+            r.k.copy_(k0)
+            r.v.copy_(v0)
+            r.head64.copy_(h64)
+            r.head32.copy_(h32)
+        del saved
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = one_step()
+
+        def step(segment: torch.Tensor) -> torch.Tensor:
+            inp.copy_(segment)
+            graph.replay()
+            return logits
+
+        step.rings, step.graph = rings, graph
+        return step
 
     def _first_step(self, embeds, caches):
         """The first segment of a stream through the full forward; its keys and values seed the

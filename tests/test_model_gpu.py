@@ -239,3 +239,24 @@ def test_model_use_cache_returns_presents_like_the_reference():
     assert presents2[0][0].shape == (B, 2, T, C, 64)
     err = (step[:, 0].float() - full[:, T - 1].float()).abs().max().item()
     assert err <= 3e-2 * full.float().abs().max().item(), err
+
+
+def test_graph_replayed_stream_step_matches_eager_steps():
+    """capture_stream: once the window is full, one classify_step on ring caches is captured into a
+    HIP graph; every replay (with eager work of the same model between replays) gives the logits
+    of the eager classify_step on the in-place caches, to bf16 rounding - the ring visits the key
+    steps in another order."""
+    model, cfg = _small_harness()
+    B, T, C = 2, cfg.n_positions, 20
+    n_more = 2 * T + 3                                   # the ring wraps more than twice
+    batch = torch.randn(B, T + n_more, C, 512, device="cuda")
+    past = None
+    for t in range(T):
+        _, past = model.classify_step(batch[:, t], past)
+    step = model.capture_stream(past, batch[:, 0])
+    for t in range(T, T + n_more):
+        want, past = model.classify_step(batch[:, t], past)          # eager, in-place caches
+        model.classify(batch[:, t - T + 1:t + 1])                    # unrelated eager work in between
+        got = step(batch[:, t])
+        spread = want.float().abs().max().item() + 1e-3
+        assert (got.float() - want.float()).abs().max().item() <= 3e-2 * spread, t
