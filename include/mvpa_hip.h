@@ -250,6 +250,15 @@ int mvpa_add3_rmsnorm_bf16(const void* a, const void* b, const void* c, const fl
 int mvpa_wavedec_db4(const float* x, float* coeffs, int64_t M, int32_t L, int32_t levels,
                      int32_t dwt_size, int64_t ldc, void* stream);
 
+/* One new time step of keys and values ([B,Hkv,C,Dh] views with element strides
+ * stride_b/h/c and unit last stride, e.g. slices of the fused projection output) into slot *head
+ * (device memory) of the ring buffers [B,Hkv,steps,C,Dh] that MVPA_FLAG_RING reads: the in-place
+ * form of the cache concatenation of layers/mvpa.py:314-317, both tensors in one launch. */
+int mvpa_ring_append_bf16(const void* k_new, const void* v_new, void* k_ring, void* v_ring,
+                          const int32_t* head, int32_t B, int32_t Hkv, int32_t C, int32_t Dh,
+                          int32_t steps, int64_t stride_b, int64_t stride_h, int64_t stride_c,
+                          void* stream);
+
 /* Measurement aid with no counterpart in the reference: a stream of nothing but
  * v_mfma_f32_32x32x16_bf16 on every SIMD (512 workgroups x 4 waves x iters x 8 instructions,
  * mvpa_probe_mfma_flops(iters) flop in all), on smooth operands (the same small value in every

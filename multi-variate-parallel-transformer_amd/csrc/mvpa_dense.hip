@@ -180,7 +180,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void linear_bf16_skinny_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, bf16_t* __restrict__ Y, int64_t M,
     int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldy) {
   constexpr int NA = EPI == 1 ? 2 : 1;            // w tiles per workgroup (gate, up)
-  constexpr int UNROLL = XT == 2 ? 4 : 2;         // k-steps in flight per wave
+  constexpr int UNROLL = XT == 2 ? 8 : 4;         // k-steps in flight per wave
   extern __shared__ __attribute__((aligned(16))) float sk_red[];   // [SK_WAVES][XT][16][64]
   const int tid = threadIdx.x, lane = tid & 63, ln = lane & 31, hh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -680,6 +680,27 @@ __global__ __launch_bounds__(256) void wavedec_db4_kernel(const float* __restric
   for (int k = threadIdx.x; k < n; k += 256) out[row * ldc + k] = cur[k];
 }
 
+// One new time step of keys and values into the slot *head of two ring buffers
+// [B,Hkv,steps,C,Dh]: k_new / v_new are [B,Hkv,C,Dh] views (element strides sb, sh, sc, unit
+// last stride) of the projection output.  One thread per 16 bytes.
+__global__ __launch_bounds__(256) void ring_append_bf16_kernel(
+    const bf16_t* __restrict__ k_new, const bf16_t* __restrict__ v_new, bf16_t* __restrict__ k_ring,
+    bf16_t* __restrict__ v_ring, const int32_t* __restrict__ head, int Hkv, int C, int Dh, int steps,
+    int64_t sb, int64_t sh, int64_t sc, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int d8 = Dh / 8;
+  const int d = (int)(i % d8) * 8;
+  const int c = (int)((i / d8) % C);
+  const int h = (int)((i / ((int64_t)d8 * C)) % Hkv);
+  const int64_t b = i / ((int64_t)d8 * C * Hkv);
+  const int slot = *head;
+  const int64_t src = b * sb + h * sh + c * sc + d;
+  const int64_t dst = (((b * Hkv + h) * steps + slot) * C + c) * Dh + d;
+  *(u32x4*)(k_ring + dst) = *(const u32x4*)(k_new + src);
+  *(u32x4*)(v_ring + dst) = *(const u32x4*)(v_new + src);
+}
+
 }  // namespace mvpa
 
 using namespace mvpa;
@@ -790,6 +811,22 @@ extern "C" int mvpa_add3_bf16(const void* a, const void* b, const void* c, void*
   hipLaunchKernelGGL(add3_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)c,
                      (bf16_t*)out, n);
+  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+}
+
+extern "C" int mvpa_ring_append_bf16(const void* k_new, const void* v_new, void* k_ring, void* v_ring,
+                                     const int32_t* head, int32_t B, int32_t Hkv, int32_t C, int32_t Dh,
+                                     int32_t steps, int64_t stride_b, int64_t stride_h, int64_t stride_c,
+                                     void* stream) {
+  if (!k_new || !v_new || !k_ring || !v_ring || !head) return MVPA_ERR_NULL;
+  if (B <= 0 || Hkv <= 0 || C <= 0 || Dh <= 0 || steps <= 0) return MVPA_ERR_SHAPE;
+  if (Dh % 8 != 0 || ((stride_b | stride_h | stride_c) & 7) ||
+      (((uintptr_t)k_new | (uintptr_t)v_new | (uintptr_t)k_ring | (uintptr_t)v_ring) & 15))
+    return MVPA_ERR_ALIGN;
+  const int64_t total = (int64_t)B * Hkv * C * (Dh / 8);
+  hipLaunchKernelGGL(ring_append_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, (const bf16_t*)k_new, (const bf16_t*)v_new, (bf16_t*)k_ring,
+                     (bf16_t*)v_ring, head, Hkv, C, Dh, steps, stride_b, stride_h, stride_c, total);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 

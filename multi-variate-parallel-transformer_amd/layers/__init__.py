@@ -1,3 +1,5 @@
-from .mvpa import MvpaKVCache, MvpaRingCache, MVPFormerGQAAttention, MVPFormerGQAFlashAttention
+from .mvpa import (MvpaKVCache, MvpaRingCache, MvpaRingClock, MVPFormerGQAAttention,
+                   MVPFormerGQAFlashAttention)
 
-__all__ = ["MvpaKVCache", "MvpaRingCache", "MVPFormerGQAAttention", "MVPFormerGQAFlashAttention"]
+__all__ = ["MvpaKVCache", "MvpaRingCache", "MvpaRingClock", "MVPFormerGQAAttention",
+           "MVPFormerGQAFlashAttention"]

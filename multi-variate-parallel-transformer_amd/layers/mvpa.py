@@ -73,6 +73,20 @@ class MvpaKVCache:
         self.start = self.length = 0
 
 
+class MvpaRingClock:
+    """The slot of the newest time step of one or several MvpaRingCaches, as a device counter (the
+    attention kernel and the append kernel read it there).  The caches of all blocks of a stack
+    move together, so they share one clock that advances once per step."""
+
+    def __init__(self, steps: int, head: int, device):
+        self.steps = steps
+        self.head32 = torch.tensor([head], dtype=torch.int32, device=device)
+
+    def advance(self) -> None:
+        """On to the next slot (the oldest step's).  Device-side only: may run under graph capture."""
+        self.head32.add_(1).remainder_(self.steps)
+
+
 class MvpaRingCache:
     """A full window of keys and values as a ring: `steps` slots [B,Hkv,steps,C,Dh], the newest
     time step in slot `head` (a device counter), the one before it in slot head-1, and so on
@@ -80,28 +94,35 @@ class MvpaRingCache:
     stays where it is and the position of the newest step lives in device memory: one decoding step
     is then a fixed sequence of launches that a HIP graph can replay (MVPA_FLAG_RING tells the
     attention kernel which table row each slot stands for).  Always full: build it from a filled
-    MvpaKVCache with `from_cache`."""
+    MvpaKVCache with `from_cache`.  With a clock of its own (the default) append() moves on to the
+    next slot by itself; caches that share a clock write where the clock stands and whoever drives
+    them advances it once per step."""
 
-    def __init__(self, k: torch.Tensor, v: torch.Tensor, head: int):
-        self.k, self.v = k, v                    # [B,Hkv,steps,C,Dh]
+    def __init__(self, k: torch.Tensor, v: torch.Tensor, head: int = 0, clock: Optional[MvpaRingClock] = None):
+        self.k, self.v = k.contiguous(), v.contiguous()      # [B,Hkv,steps,C,Dh]
         self.steps = k.shape[2]
-        self.head64 = torch.tensor([head], dtype=torch.int64, device=k.device)
-        self.head32 = torch.tensor([head], dtype=torch.int32, device=k.device)
+        self.own_clock = clock is None
+        self.clock = MvpaRingClock(self.steps, head, k.device) if clock is None else clock
+        if self.clock.steps != self.steps:
+            raise ValueError("clock and cache disagree on the number of slots")
+
+    @property
+    def head32(self) -> torch.Tensor:
+        return self.clock.head32
 
     @classmethod
-    def from_cache(cls, cache: "MvpaKVCache") -> "MvpaRingCache":
+    def from_cache(cls, cache: "MvpaKVCache", clock: Optional[MvpaRingClock] = None) -> "MvpaRingCache":
         if cache.length != cache.max_steps:
             raise ValueError("the window is not full yet: keep appending to the MvpaKVCache")
         k, v = cache.views()
-        return cls(k.clone(), v.clone(), cache.max_steps - 1)      # time order: the newest step is last
+        return cls(k.clone(), v.clone(), cache.max_steps - 1, clock)   # time order: the newest step is last
 
     def append(self, k_new: torch.Tensor, v_new: torch.Tensor) -> None:
-        """Overwrite the oldest slot with one new time step ([B,Hkv,C,Dh] each).  Device-side only:
-        may run under graph capture."""
-        self.head64.add_(1).remainder_(self.steps)
-        self.head32.copy_(self.head64)
-        self.k.index_copy_(2, self.head64, k_new.unsqueeze(2))
-        self.v.index_copy_(2, self.head64, v_new.unsqueeze(2))
+        """One new time step ([B,Hkv,C,Dh] each) over the oldest slot.  Device-side only: may run
+        under graph capture."""
+        if self.own_clock:
+            self.clock.advance()
+        mvpa_hip.ring_append(k_new, v_new, self.k, self.v, self.clock.head32)
 
 
 class _LoRALinear(torch.nn.Linear):

@@ -11,7 +11,8 @@ import torch
 from torch import nn
 
 import mvpa_hip
-from layers import MvpaKVCache, MvpaRingCache, MVPFormerGQAAttention, MVPFormerGQAFlashAttention
+from layers import (MvpaKVCache, MvpaRingCache, MvpaRingClock, MVPFormerGQAAttention,
+                    MVPFormerGQAFlashAttention)
 from models import BrainDecider, BrainEncoder, BrainModel
 from models.fftencoder import RMSNorm
 
@@ -316,10 +317,12 @@ class HMVPFormer(BrainModel):
         step(segment) -> logits that copies the segment into a fixed buffer and replays the graph
         of one classify_step on ring caches (the caches are copied; `past` is left alone).  The
         returned logits tensor is overwritten by the next call."""
-        rings = tuple(MvpaRingCache.from_cache(c) for c in past)
+        clock = MvpaRingClock(past[0].max_steps, past[0].max_steps - 1, segment_like.device)
+        rings = tuple(MvpaRingCache.from_cache(c, clock) for c in past)     # one clock for all blocks
         inp = segment_like.clone()
 
         def one_step():
+            clock.advance()
             bsz, ch, seg = inp.shape
             embeds = self.encoder(inp.reshape(bsz * ch, seg)).view(bsz, 1, ch, -1)
             out, _ = self.mvpformer(inputs_embeds=embeds, past_key_values=rings)
@@ -327,16 +330,16 @@ class HMVPFormer(BrainModel):
 
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
-        saved = [(r.k.clone(), r.v.clone(), r.head64.clone(), r.head32.clone()) for r in rings]
+        saved = [(r.k.clone(), r.v.clone()) for r in rings]
+        head0 = clock.head32.clone()
         with torch.cuda.stream(side):
             for _ in range(2):                      # warm-up: fills every host-side cache of the path
                 one_step()
         torch.cuda.current_stream().wait_stream(side)
-        for r, (k0, v0, h64, h32) in zip(rings, saved):     # the warm-up steps wrote into the rings
+        for r, (k0, v0) in zip(rings, saved):       # the warm-up steps wrote into the rings
             r.k.copy_(k0)
             r.v.copy_(v0)
-            r.head64.copy_(h64)
-            r.head32.copy_(h32)
+        clock.head32.copy_(head0)
         del saved
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):

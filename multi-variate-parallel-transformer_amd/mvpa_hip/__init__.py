@@ -92,6 +92,8 @@ def load_library() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(MvpaFwdArgs)]
+    lib.mvpa_ring_append_bf16.restype = ctypes.c_int
+    lib.mvpa_ring_append_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i64, i64, i64, vp]
     lib.mvpa_probe_mfma.restype = ctypes.c_int
     lib.mvpa_probe_mfma.argtypes = [i32, i32, vp, vp]
     lib.mvpa_probe_mfma_flops.restype = ctypes.c_int64
@@ -439,6 +441,23 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5,
                             x2.stride(0), y2.stride(0), eps, _dtype_code(x.dtype), _dtype_code(od),
                             _stream()))
     return y
+
+
+def ring_append(k_new: torch.Tensor, v_new: torch.Tensor, k_ring: torch.Tensor, v_ring: torch.Tensor,
+                head32: torch.Tensor) -> None:
+    """Write one time step ([B,Hkv,C,Dh] views of equal strides, bf16) into slot head32[0] of the
+    contiguous ring buffers [B,Hkv,steps,C,Dh]; the slot is read on the device."""
+    lib = load_library()
+    _need_cuda(k_new, v_new, k_ring, v_ring, head32)
+    B, Hkv, C, Dh = k_new.shape
+    assert v_new.shape == k_new.shape and k_new.stride() == v_new.stride() and k_new.stride(3) == 1
+    assert k_ring.is_contiguous() and v_ring.is_contiguous() and k_ring.shape == v_ring.shape
+    assert k_ring.shape[0] == B and k_ring.shape[1] == Hkv and tuple(k_ring.shape[3:]) == (C, Dh)
+    assert k_new.dtype == v_new.dtype == k_ring.dtype == v_ring.dtype == torch.bfloat16
+    assert head32.dtype == torch.int32
+    _check(lib.mvpa_ring_append_bf16(k_new.data_ptr(), v_new.data_ptr(), k_ring.data_ptr(), v_ring.data_ptr(),
+                                     head32.data_ptr(), B, Hkv, C, Dh, k_ring.shape[2],
+                                     k_new.stride(0), k_new.stride(1), k_new.stride(2), _stream()))
 
 
 def add3(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor) -> torch.Tensor:

@@ -107,3 +107,20 @@ def test_mfma_probe_runs_and_reads_plausibly():
     rand = mvpa_hip.mfma_probe_tflops(True, iters=4000, reps=2)
     assert 800.0 < smooth < 2700.0, smooth
     assert 500.0 < rand <= smooth * 1.05, (rand, smooth)
+
+
+def test_ring_append_writes_the_slot_the_device_counter_names():
+    """mvpa_ring_append_bf16: keys and values of one step, given as strided views of a fused
+    projection output, land in slot head[0] of both rings; everything else stays."""
+    B, Hkv, C, Dh, steps = 2, 3, 5, 16, 7
+    row = 4 * Dh + 2 * Hkv * Dh
+    qkv = torch.randn(B, C, row, device="cuda").bfloat16()
+    k_new = qkv[:, :, 4 * Dh:4 * Dh + Hkv * Dh].view(B, C, Hkv, Dh).permute(0, 2, 1, 3)
+    v_new = qkv[:, :, 4 * Dh + Hkv * Dh:].view(B, C, Hkv, Dh).permute(0, 2, 1, 3)
+    k_ring = torch.randn(B, Hkv, steps, C, Dh, device="cuda").bfloat16()
+    v_ring = torch.randn(B, Hkv, steps, C, Dh, device="cuda").bfloat16()
+    k0, v0 = k_ring.clone(), v_ring.clone()
+    head = torch.tensor([4], dtype=torch.int32, device="cuda")
+    mvpa_hip.ring_append(k_new, v_new, k_ring, v_ring, head)
+    k0[:, :, 4], v0[:, :, 4] = k_new, v_new
+    assert torch.equal(k_ring, k0) and torch.equal(v_ring, v0)
