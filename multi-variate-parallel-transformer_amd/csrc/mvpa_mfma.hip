@@ -504,7 +504,9 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 
   float* Stb = Stb_all + wave * (32 * 32);
   // key steps 0 .. far_max are "far" for this wave's queries (content term absent or zeroed)
-  const int far_max = !has_content ? tq : (W > 0 && tq != T_ - 1) ? tq - W - 1 : -1;
+  // (RUNS launches are last-step launches with the content term on: no far steps at all, and the
+  // far path is compiled out of that build of the kernel)
+  const int far_max = RUNS ? -1 : !has_content ? tq : (W > 0 && tq != T_ - 1) ? tq - W - 1 : -1;
   auto is_far = [&](int tk) -> bool { return tk <= far_max; };
 
   // ---- per-lane pieces of the LDS fragment addresses (loop invariant)
@@ -704,7 +706,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
         const int tkw = t0 + par;
         if (tkw <= T_ - 1) {
           const unsigned char* stage = smem_raw + (2 * u) * G::STAGE_BYTES + par * G::STAGE_BYTES;
-          if (is_far(tkw)) far_step(stage, tkw);
+          if (!RUNS && is_far(tkw)) far_step(stage, tkw);
           else near_step(stage, tkw);
         }
       }
@@ -721,7 +723,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   {
     // uniform over the workgroup (every wave must reach the same barriers): all of these steps
     // are at or before tq0, hence visible to every query of the workgroup
-    const int fast_end = min(tk_near - (STAGES - 1), tq0 + 1);
+    const int fast_end = RUNS ? 0 : min(tk_near - (STAGES - 1), tq0 + 1);
     const int n_groups = fast_end > 0 ? fast_end / STAGES : 0;
     f32x16 ptmp[MT];                       // V^T Ec^T of the previous step, not yet accumulated
     float pet = 0.f;                       // its weight
@@ -797,7 +799,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
       if ((tk & 31) == 0 && active) time_slab(tk);
       if (active && tk <= tq) {
         const unsigned char* stage = smem_raw + s * G::STAGE_BYTES + key_off;
-        if (is_far(tk)) far_step(stage, tk);
+        if (!RUNS && is_far(tk)) far_step(stage, tk);
         else near_step(stage, tk);
       }
     }
@@ -900,8 +902,11 @@ static int launch_one(const mvpa_fwd_args* a, hipStream_t stream) {
   static_assert(KH <= 2 && (KH == 1 || G::TQW * G::QT * (2 + G::MT * 16) * 256 <= G::RING_BYTES), "merge buffer");
   static_assert(G::LDS_BYTES <= 160 * 1024, "LDS budget");
   const bool last = a->flags & MVPA_FLAG_LAST_STEP;
-  const int n_split = (last && a->split_ws && a->n_split > 1) ? a->n_split : 1;
+  int n_split = (last && a->split_ws && a->n_split > 1) ? a->n_split : 1;
   const bool ring = last && (a->flags & MVPA_FLAG_RING);
+  const bool content = a->flags & MVPA_FLAG_CONTENT;
+  if (ring && !content) return MVPA_ERR_UNSUPPORTED;      // the run build has no far path
+  if (!content) n_split = 1;
   auto kern = (n_split > 1 || ring) ? mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH, true>
                           : mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH, false>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -960,6 +965,11 @@ int mvpa_launch_mfma(const mvpa_fwd_args* a, hipStream_t stream) {
     case 128:
       if (nct == 1) return launch_cfg<128, 1, 4, 4>(a, stream);
       if (nct == 2) return launch_cfg<128, 2, 4, 3>(a, stream);
+      // key-run (decoding) launches of 97..128 channels: the keys of a step in two parts, 8 waves,
+      // two per SIMD (that build has no far path and fits the registers)
+      if ((a->flags & MVPA_FLAG_LAST_STEP) && (a->flags & MVPA_FLAG_CONTENT) &&
+          ((a->split_ws && a->n_split > 1) || (a->flags & MVPA_FLAG_RING)))
+        return launch_cfg<128, 2, 8, 2, 1, 2>(a, stream);
       return launch_cfg<128, 4, 4, 2>(a, stream);
   }
   return MVPA_ERR_UNSUPPORTED;

@@ -201,8 +201,8 @@ def make_args(q, k, v, out, u, vb, z, k_time, k_chan, *, T: int, C: int,
 
 def default_key_splits(B: int, H: int, T: int) -> int:
     """Runs of key steps a last-step launch is cut into: about one workgroup per CU (256), at
-    least 8 key steps per run, no empty run.  Measured: B1 H16 C128 T512 Dh128 2.60 ms unsplit,
-    0.24 ms at 16 runs, 0.26 at 32; B4 H16 C64 T128 0.071 ms unsplit, 0.034 at 4 runs, 0.050 at 16."""
+    least 8 key steps per run, no empty run.  Measured: B1 H16 C128 T512 Dh128 2.50 ms unsplit,
+    0.11 ms at 16 runs, 0.14 at 32; B4 H16 C64 T128 0.071 ms unsplit, 0.034 at 4 runs, 0.050 at 16."""
     n = max(1, min(T // 8, 256 // max(1, B * H)))
     while n > 1 and (n - 1) * ((T + n - 1) // n) >= T:
         n -= 1
