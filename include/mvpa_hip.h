@@ -223,6 +223,16 @@ int mvpa_debug_maps(int32_t T, int32_t C, int32_t window, uint32_t flags,
 int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M, int64_t N, int64_t K,
                      int64_t ldx, int64_t ldw, int64_t ldy, int32_t epilogue, void* stream);
 
+/* The same product for at most 128 rows of x against a large weight (the projections of one
+ * decoding step of a wide model), with K split over workgroups: fp32 partial tiles go through the
+ * caller's workspace ws (mvpa_linear_splitk_ws_bytes(M, N, K, epilogue) bytes, 16-byte aligned)
+ * and a second kernel sums them and applies the epilogue.  Same arguments and results (to fp32
+ * summation order) as mvpa_linear_bf16. */
+int mvpa_linear_bf16_splitk(const void* x, const void* w, void* y, int64_t M, int64_t N, int64_t K,
+                            int64_t ldx, int64_t ldw, int64_t ldy, int32_t epilogue, void* ws,
+                            size_t ws_bytes, void* stream);
+size_t mvpa_linear_splitk_ws_bytes(int64_t M, int64_t N, int64_t K, int32_t epilogue);
+
 /* RMSNorm over the last dim: y = x * rsqrt(mean(x^2)+eps) * weight
  * (models/mvpformer.py:108,133,167,380; models/fftencoder.py:67,93).
  * in_dtype/out_dtype: MVPA_F32 | MVPA_BF16; weight is fp32; ldx/ldy are row pitches in

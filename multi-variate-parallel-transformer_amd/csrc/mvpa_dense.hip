@@ -287,6 +287,130 @@ __global__ __launch_bounds__(SK_WAVES * 64) void linear_bf16_skinny_kernel(
 }
 
 // -----------------------------------------------------------------------------------------
+// K-split variant for at most 128 rows of x against a large weight (the projections of one decoding
+// step of a wide model): workgroup (c, s) multiplies the 64 rows of w from 64c on with all rows of
+// x over the K slice [256 s, 256 s + 256).  Both slices are fetched once, coalesced, into LDS (row
+// pitch 528 bytes, so the 16-byte fragment reads of 32 rows spread over the banks), each of the
+// 4 waves takes 32 rows of x, and the fp32 partial tile goes to a workspace [slices][M][rows of w];
+// linear_splitk_reduce_kernel sums the slices and applies the epilogue.  Against the kernel above
+// this reads x once per 64 columns instead of once per 32 with one access per 128-byte line
+// instead of four, and has enough workgroups for every CU whatever N is.
+// -----------------------------------------------------------------------------------------
+constexpr int SPK_KS = 256, SPK_COLS = 64, SPK_PITCH = SPK_KS + 8, SPK_XROWS = 128;
+constexpr int SPK_LDS_BYTES = (SPK_XROWS + SPK_COLS) * SPK_PITCH * 2;
+
+__global__ __launch_bounds__(256) void linear_splitk_kernel(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* __restrict__ P, int64_t M,
+    int64_t NW, int64_t K, int64_t ldx, int64_t ldw, int per_group) {
+  extern __shared__ __attribute__((aligned(16))) bf16_t spk_lds[];
+  bf16_t* Xs = spk_lds;                               // [128][SPK_PITCH]
+  bf16_t* Ws = spk_lds + SPK_XROWS * SPK_PITCH;       // [64][SPK_PITCH]
+  const int tid = threadIdx.x, lane = tid & 63, ln = lane & 31, hh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t n0 = (int64_t)blockIdx.x * SPK_COLS;
+  const int xrows = (int)((M + 31) / 32) * 32;        // rows of x staged (whole 32-row tiles)
+  f32x16 acc[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+
+  // a workgroup takes per_group consecutive K slices, one after the other through the same buffer
+  for (int sl = 0; sl < per_group; ++sl) {
+  const int64_t k0 = ((int64_t)blockIdx.y * per_group + sl) * SPK_KS;
+  if (k0 >= K) break;
+  if (sl) __syncthreads();
+
+  // stage both slices: 32 chunks of 16 bytes per row, consecutive lanes on consecutive chunks
+  u32x4 xr[SPK_XROWS * 32 / 256], wr[SPK_COLS * 32 / 256];
+#pragma unroll
+  for (int i = 0; i < SPK_XROWS * 32 / 256; ++i) {
+    const int c = tid + 256 * i, r = c >> 5, kc = (c & 31) * 8;
+    if (r < xrows) xr[i] = load_chunk(X + (r < M ? r : 0) * ldx, k0 + kc, K, r < M);
+  }
+#pragma unroll
+  for (int i = 0; i < SPK_COLS * 32 / 256; ++i) {
+    const int c = tid + 256 * i, r = c >> 5, kc = (c & 31) * 8;
+    const int64_t n = n0 + r;
+    wr[i] = load_chunk(W + (n < NW ? n : 0) * ldw, k0 + kc, K, n < NW);
+  }
+#pragma unroll
+  for (int i = 0; i < SPK_XROWS * 32 / 256; ++i) {
+    const int c = tid + 256 * i, r = c >> 5, kc = (c & 31) * 8;
+    if (r < xrows) *(u32x4*)(Xs + r * SPK_PITCH + kc) = xr[i];
+  }
+#pragma unroll
+  for (int i = 0; i < SPK_COLS * 32 / 256; ++i) {
+    const int c = tid + 256 * i, r = c >> 5, kc = (c & 31) * 8;
+    *(u32x4*)(Ws + r * SPK_PITCH + kc) = wr[i];
+  }
+  __syncthreads();
+  if (wave * 32 < M) {                                // else this wave's rows of x do not exist
+#pragma unroll 4
+  for (int ks = 0; ks < SPK_KS / 16; ++ks) {
+    const bf16x8 xf = *(const bf16x8*)(Xs + (wave * 32 + ln) * SPK_PITCH + ks * 16 + hh * 8);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const bf16x8 wf = *(const bf16x8*)(Ws + (j * 32 + ln) * SPK_PITCH + ks * 16 + hh * 8);
+      acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf, acc[j], 0, 0, 0);   // [w row][x row]
+    }
+  }
+  }
+  }   // K slices of this workgroup
+  // lane: x row wave*32 + ln, rows of w n0 + 32j + 8q + 4hh + 0..3 -> 16-byte stores
+  const int64_t m = wave * 32 + ln;
+  if (m >= M) return;
+  float* prow = P + ((int64_t)blockIdx.y * M + m) * NW;
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int64_t n = n0 + j * 32 + q * 8 + hh * 4;
+      if (n + 3 < NW && (NW & 3) == 0) {
+        *(float4*)(prow + n) = make_float4(acc[j][4 * q], acc[j][4 * q + 1], acc[j][4 * q + 2], acc[j][4 * q + 3]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < NW) prow[n + r] = acc[j][4 * q + r];
+      }
+    }
+}
+
+// Sums the K slices of linear_splitk_kernel and writes bf16: one thread per 4 output columns.
+template <int EPI>
+__global__ __launch_bounds__(256) void linear_splitk_reduce_kernel(
+    const float* __restrict__ P, bf16_t* __restrict__ Y, int64_t M, int64_t N, int64_t NW,
+    int slices, int64_t ldy) {
+  const int64_t n4 = (N + 3) / 4;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= M * n4) return;
+  const int64_t m = i / n4, n = (i % n4) * 4;
+  float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool vec = n + 3 < N && (NW & 3) == 0 && (N & 3) == 0;
+  for (int s = 0; s < slices; ++s) {
+    const float* row = P + ((int64_t)s * M + m) * NW;
+    if (vec) {
+      const float4 a = *(const float4*)(row + n);
+      g[0] += a.x; g[1] += a.y; g[2] += a.z; g[3] += a.w;
+      if (EPI == 1) {
+        const float4 b = *(const float4*)(row + N + n);
+        u[0] += b.x; u[1] += b.y; u[2] += b.z; u[3] += b.w;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n + r < N) {
+          g[r] += row[n + r];
+          if (EPI == 1) u[r] += row[N + n + r];
+        }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    if (n + r < N) Y[m * ldy + n + r] = f32_to_bf16(EPI == 1 ? g[r] / (1.f + __expf(-g[r])) * u[r] : g[r]);
+}
+
+// -----------------------------------------------------------------------------------------
 // Large-tile variant for the big projections (M >= 256, K a multiple of 8):
 //   workgroup tile 256 (rows of x) x BN (rows of w) x 64, 8 waves as 4 (x) x 2 (w), 2 waves/SIMD;
 //   tiles go HBM/L2 -> LDS with direct-to-LDS loads (no staging registers) into two buffers,
@@ -713,6 +837,51 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M,
   if (lds > 64 * 1024)
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   hipLaunchKernelGGL(kern, dim3((unsigned)((N + 31) / 32)), dim3(SK_WAVES * 64), lds, s, x, w, y, M, N, K, ldx, ldw, ldy);
+  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+}
+
+// K slices per workgroup and the number of workgroup rows that follows: as few partial tiles as
+// still give every CU a workgroup (about 256 in all)
+static void splitk_groups(int64_t nw, int64_t K, int* per_group, int* groups) {
+  const int64_t slices = (K + SPK_KS - 1) / SPK_KS, col_tiles = (nw + SPK_COLS - 1) / SPK_COLS;
+  int64_t g = (256 + col_tiles - 1) / col_tiles;          // workgroup rows wanted
+  if (g > slices) g = slices;
+  if (g < 1) g = 1;
+  *per_group = (int)((slices + g - 1) / g);
+  *groups = (int)((slices + *per_group - 1) / *per_group);
+}
+
+extern "C" size_t mvpa_linear_splitk_ws_bytes(int64_t M, int64_t N, int64_t K, int32_t epilogue) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  const int64_t nw = epilogue == 1 ? 2 * N : N;
+  int per_group, groups;
+  splitk_groups(nw, K, &per_group, &groups);
+  return (size_t)((int64_t)groups * M * nw) * sizeof(float);
+}
+
+extern "C" int mvpa_linear_bf16_splitk(const void* x, const void* w, void* y, int64_t M, int64_t N,
+                                       int64_t K, int64_t ldx, int64_t ldw, int64_t ldy,
+                                       int32_t epilogue, void* ws, size_t ws_bytes, void* stream) {
+  if (!x || !w || !y || !ws) return MVPA_ERR_NULL;
+  if (M <= 0 || M > SPK_XROWS || N <= 0 || K <= 0 || ldx < K || ldw < K || ldy < N) return MVPA_ERR_SHAPE;
+  if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)ws & 15) || (ldx & 7) || (ldw & 7))
+    return MVPA_ERR_ALIGN;
+  if (epilogue != 0 && epilogue != 1) return MVPA_ERR_UNSUPPORTED;
+  if (ws_bytes < mvpa_linear_splitk_ws_bytes(M, N, K, epilogue)) return MVPA_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t nw = epilogue == 1 ? 2 * N : N;
+  int per_group, slices;          // slices: partial tiles per output tile = workgroup rows
+  splitk_groups(nw, K, &per_group, &slices);
+  (void)hipFuncSetAttribute((const void*)linear_splitk_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SPK_LDS_BYTES);
+  hipLaunchKernelGGL(linear_splitk_kernel, dim3((unsigned)((nw + SPK_COLS - 1) / SPK_COLS), (unsigned)slices), dim3(256),
+                     SPK_LDS_BYTES, s, (const bf16_t*)x, (const bf16_t*)w, (float*)ws, M, nw, K, ldx, ldw, per_group);
+  const int64_t items = M * ((N + 3) / 4);
+  if (epilogue == 1)
+    hipLaunchKernelGGL(linear_splitk_reduce_kernel<1>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
+                       (const float*)ws, (bf16_t*)y, M, N, nw, slices, ldy);
+  else
+    hipLaunchKernelGGL(linear_splitk_reduce_kernel<0>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
+                       (const float*)ws, (bf16_t*)y, M, N, nw, slices, ldy);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 

@@ -124,3 +124,28 @@ def test_ring_append_writes_the_slot_the_device_counter_names():
     mvpa_hip.ring_append(k_new, v_new, k_ring, v_ring, head)
     k0[:, :, 4], v0[:, :, 4] = k_new, v_new
     assert torch.equal(k_ring, k0) and torch.equal(v_ring, v0)
+
+
+@pytest.mark.parametrize("M,N,K,gated", [(128, 2048, 2048, False), (128, 4096, 2048, False), (100, 2048, 5632, False),
+                                         (128, 5632, 2048, True), (65, 96, 24, False), (33, 130, 550, False),
+                                         (7, 70, 136, True), (128, 33, 300, True), (1, 64, 256, False)])
+def test_linear_split_k_pair(M, N, K, gated):
+    """mvpa_linear_bf16_splitk (K slices of 256 on separate workgroups, fp32 partial tiles through a
+    workspace, second kernel sums and applies the epilogue) against float64, and against the
+    one-kernel path to fp32 summation order."""
+    g = torch.Generator().manual_seed(M * 7 + N + K)
+    ldk = (K + 7) // 8 * 8
+    x = torch.zeros(M, ldk).bfloat16()
+    w = torch.zeros((2 if gated else 1) * N, ldk).bfloat16()
+    x[:, :K] = torch.randn(M, K, generator=g).bfloat16()
+    w[:, :K] = (torch.randn(w.shape[0], K, generator=g) * 0.05).bfloat16()
+    xg, wg = x.cuda(), w.cuda()
+    y = mvpa_hip.linear(xg[:, :K], wg[:, :K], gated=gated, split_k=True).float().cpu()
+    y1 = mvpa_hip.linear(xg[:, :K], wg[:, :K], gated=gated, split_k=False).float().cpu()
+    if gated:
+        ref = torch.nn.functional.silu(x[:, :K].double() @ w[:N, :K].double().T) * (x[:, :K].double() @ w[N:, :K].double().T)
+    else:
+        ref = x[:, :K].double() @ w[:, :K].double().T
+    tol = (2 ** -7 if gated else 2 ** -8) * ref.abs().max().item() + 1e-5
+    assert (y.double() - ref).abs().max().item() <= tol
+    assert (y - y1).abs().max().item() <= 2 * tol
