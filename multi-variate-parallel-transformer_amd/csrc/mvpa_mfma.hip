@@ -865,35 +865,35 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 }
 
 // Combines the runs of a split last-step launch: out = sum_r 2^(lse_r - lse) o_r with
-// lse = log2 sum_r 2^lse_r.  One wave per output row, lane = pair of head-dim elements.
+// lse = log2 sum_r 2^lse_r.  DH/8 lanes per output row, 16 bytes each.
 template <int DH>
 __global__ __launch_bounds__(256) void mvpa_split_merge_kernel(mvpa_fwd_args a) {
-  const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  constexpr int LPR = DH / 8, RPB = 256 / LPR;         // lanes per row (8 elements each), rows per block
+  const int sub = threadIdx.x % LPR;
   const int nbh = a.B * a.H, C_ = a.C, rows = nbh * C_;
+  const int row = blockIdx.x * RPB + threadIdx.x / LPR;
   if (row >= rows) return;
   const bf16_t* po = (const bf16_t*)a.split_ws;
   const float* plse = (const float*)(po + (int64_t)a.n_split * rows * DH);
   float m = -INFINITY;
   for (int r = 0; r < a.n_split; ++r) m = fmaxf(m, plse[(int64_t)r * rows + row]);
-  float l = 0.f, acc[2] = {0.f, 0.f};
+  float l = 0.f, acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
   for (int r = 0; r < a.n_split; ++r) {
     const float w = fast_exp2(plse[(int64_t)r * rows + row] - m);
     l += w;
-    if (2 * lane < DH) {
-      const bf16x2 v = *(const bf16x2*)(po + ((int64_t)r * rows + row) * DH + 2 * lane);
-      acc[0] += w * (float)v[0];
-      acc[1] += w * (float)v[1];
-    }
+    const bf16x8 v = *(const bf16x8*)(po + ((int64_t)r * rows + row) * DH + 8 * sub);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] += w * (float)v[i];
   }
   const int bh = row / C_, cq = row % C_, b = bh / a.H, h = bh % a.H;
-  if (2 * lane < DH) {
-    const float inv = 1.f / l;
-    bf16x2 w2;
-    w2[0] = (__bf16)(acc[0] * inv);
-    w2[1] = (__bf16)(acc[1] * inv);
-    *(bf16x2*)((bf16_t*)a.o + b * a.o_stride_b + h * a.o_stride_h + (int64_t)cq * a.o_stride_n + 2 * lane) = w2;
-  }
-  if (a.lse && lane == 0) a.lse[row] = m + log2f(l);
+  const float inv = 1.f / l;
+  bf16x8 w8;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) w8[i] = (__bf16)(acc[i] * inv);
+  *(bf16x8*)((bf16_t*)a.o + b * a.o_stride_b + h * a.o_stride_h + (int64_t)cq * a.o_stride_n + 8 * sub) = w8;
+  if (a.lse && sub == 0) a.lse[row] = m + log2f(l);
 }
 
 template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8, int KH>
@@ -916,7 +916,7 @@ static int launch_one(const mvpa_fwd_args* a, hipStream_t stream) {
   hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), G::LDS_BYTES, stream, *a);
   if (n_split > 1) {
     const int rows = a->B * a->H * a->C;
-    hipLaunchKernelGGL(mvpa_split_merge_kernel<DH>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, *a);
+    hipLaunchKernelGGL(mvpa_split_merge_kernel<DH>, dim3((unsigned)((rows + 2048 / DH - 1) / (2048 / DH))), dim3(256), 0, stream, *a);
   }
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
