@@ -371,6 +371,28 @@ class HMVPFormer(BrainModel):
         return torch.cosine_similarity(enc[:, 1:].float(), out[:, :-1].float(), dim=-1)
 
     @torch.no_grad()
+    def predict_step(self, segment: torch.Tensor, past=None, max_steps: Optional[int] = None):
+        """predict_next_segment for a stream, one segment [B, ch, len] at a time.  Returns
+        (similarity, prediction, past): `prediction` [B, ch, E] is the head's forecast of the NEXT
+        segment's encoding, `similarity` [B, ch] the cosine similarity between this segment's
+        encoding and the forecast the previous call made for it (None on the first call) - the
+        column of predict_next_segment's result that this segment closes.  `past` carries the
+        caches and the last forecast from call to call."""
+        bsz, ch, seg = segment.shape
+        embeds = self.encoder(segment.reshape(bsz * ch, seg)).view(bsz, 1, ch, -1)
+        caches, forecast = (None, None) if past is None else past
+        if caches is None:
+            caches = self.mvpformer.new_cache(bsz, ch, max_steps, dtype=embeds.dtype, device=embeds.device)
+            out, caches = self._first_step(embeds, caches)
+        else:
+            out, caches = self.mvpformer(inputs_embeds=embeds, past_key_values=caches)
+        similarity = None
+        if forecast is not None:
+            similarity = torch.cosine_similarity(embeds[:, 0].float(), forecast.float(), dim=-1)
+        prediction = self.head(out[:, -1])
+        return similarity, prediction, (caches, prediction)
+
+    @torch.no_grad()
     def classify(self, batch: torch.Tensor):
         """Classification scoring of models/mvpformer.py:947-953: head(mean over channels of the
         last segment's hidden state)."""

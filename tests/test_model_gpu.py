@@ -260,3 +260,28 @@ def test_graph_replayed_stream_step_matches_eager_steps():
         got = step(batch[:, t])
         spread = want.float().abs().max().item() + 1e-3
         assert (got.float() - want.float()).abs().max().item() <= 3e-2 * spread, t
+
+
+def test_streamed_next_segment_scores_match_the_window_forward():
+    """predict_step over a stream of max_steps segments gives, call by call, the columns of
+    predict_next_segment on the whole window (bf16 tolerance)."""
+    from models.mvpformer import HMVPFormer, MVPFormerConfig, MVPFormerHead
+    from models.fftencoder import WaveEncoder
+    torch.manual_seed(11)
+    cfg = MVPFormerConfig(n_embd=256, n_head=4, n_head_kv=2, n_layer=2, n_positions=9, n_channels=12, n_inner=512)
+    model = HMVPFormer(cfg, WaveEncoder(size_input=512, size_output=256), MVPFormerHead(256, 256)).to("cuda", torch.bfloat16).eval()
+    B, T, C = 2, cfg.n_positions, 12
+    batch = torch.randn(B, T, C, 512, device="cuda")
+    want = model.predict_next_segment(batch)                     # [B, T-1, C]
+    past, cols = None, []
+    for t in range(T):
+        sim, pred, past = model.predict_step(batch[:, t], past)
+        assert pred.shape == (B, C, 256)
+        assert (sim is None) == (t == 0)
+        if sim is not None:
+            cols.append(sim)
+    got = torch.stack(cols, dim=1)
+    # the full forward of t+1 segments predicts from rows that END at row T of the position table
+    # only when t+1 == T; earlier columns see the same relative rows through position_end, so all
+    # columns agree
+    assert (got - want).abs().max().item() <= 3e-2
