@@ -164,3 +164,22 @@ def test_bench_refuses_more_than_one_gpu():
     res = subprocess.run([sys.executable, os.path.join(root, "bench.py")], capture_output=True,
                          text=True, timeout=120, env=env)
     assert res.returncode == 2 and "ONE GPU" in res.stderr
+
+
+def test_kv_cache_window_logic_on_the_host():
+    """MvpaKVCache is plain tensor bookkeeping: appending past max_steps keeps exactly the last
+    max_steps time steps, in order, through every wrap of the buffer (runs on the CPU)."""
+    from layers import MvpaKVCache
+    for max_steps, slack in ((5, 2), (4, 0), (1, 3), (7, None)):
+        cache = MvpaKVCache(1, 2, 3, 4, max_steps=max_steps, dtype=torch.float32, device="cpu", slack=slack)
+        assert cache.capacity >= max_steps
+        for i in range(4 * cache.capacity + 3):
+            k, v = cache.append(torch.full((1, 2, 3, 4), float(i)), torch.full((1, 2, 3, 4), -float(i)))
+            want = torch.arange(max(0, i - max_steps + 1), i + 1, dtype=torch.float32)
+            assert k.shape == (1, 2, len(want), 3, 4)
+            assert torch.equal(k[0, 1, :, 2, 3], want) and torch.equal(v[0, 0, :, 0, 0], -want)
+            assert cache.start + cache.length <= cache.capacity
+        cache.reset()
+        assert cache.length == 0
+    with pytest.raises(ValueError):
+        MvpaKVCache(1, 1, 1, 8, max_steps=0, device="cpu")
