@@ -702,6 +702,7 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const TI* __restrict_
 // sum = bf16(a + b + c) and norm = RMSNorm(sum) * w in one pass over the three inputs: the
 // residual update of one block fused with the input norm of the next.  The norm is taken over
 // the ROUNDED sum, so the result equals the two separate kernels bit for bit.
+template <int CHUNKS>     // 16-byte chunks per lane kept in registers (cols <= 512 * CHUNKS); 0 = re-read the sum
 __global__ __launch_bounds__(256) void add3_rmsnorm_bf16_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ b, const bf16_t* __restrict__ c,
     const float* __restrict__ w, bf16_t* __restrict__ sum, bf16_t* __restrict__ norm, int64_t rows,
@@ -711,6 +712,38 @@ __global__ __launch_bounds__(256) void add3_rmsnorm_bf16_kernel(
   const int lane = threadIdx.x & 63;
   const int64_t base = row * cols;
   float ss = 0.f;
+  if constexpr (CHUNKS > 0) {
+    float keep[CHUNKS][8];
+#pragma unroll
+    for (int j = 0; j < CHUNKS; ++j) {
+      const int col = lane * 8 + 512 * j;
+      if (col < cols) {
+        float vb[8], vc[8];
+        vec8<bf16_t>::load(a + base + col, keep[j]);
+        vec8<bf16_t>::load(b + base + col, vb);
+        vec8<bf16_t>::load(c + base + col, vc);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          keep[j][i] = bf16_to_f32(f32_to_bf16(keep[j][i] + vb[i] + vc[i]));
+          ss += keep[j][i] * keep[j][i];
+        }
+        vec8<bf16_t>::store(sum + base + col, keep[j]);
+      }
+    }
+    const float inv = rsqrtf(wave_sum(ss) / (float)cols + eps);
+#pragma unroll
+    for (int j = 0; j < CHUNKS; ++j) {
+      const int col = lane * 8 + 512 * j;
+      if (col < cols) {
+        float g[8];
+        vec8<float>::load(w + col, g);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) keep[j][i] = keep[j][i] * inv * g[i];
+        vec8<bf16_t>::store(norm + base + col, keep[j]);
+      }
+    }
+    return;
+  }
   for (int col = lane * 8; col < cols; col += 512) {
     float va[8], vb[8], vc[8];
     vec8<bf16_t>::load(a + base + col, va);
@@ -1007,7 +1040,9 @@ extern "C" int mvpa_add3_rmsnorm_bf16(const void* a, const void* b, const void* 
   if (cols % 8 != 0 || (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)sum |
                          (uintptr_t)norm | (uintptr_t)weight) & 15) != 0)
     return MVPA_ERR_ALIGN;
-  hipLaunchKernelGGL(add3_rmsnorm_bf16_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+  auto kern = cols <= 1024 ? add3_rmsnorm_bf16_kernel<2> : cols <= 2048 ? add3_rmsnorm_bf16_kernel<4>
+                                                                        : add3_rmsnorm_bf16_kernel<0>;
+  hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)c,
                      weight, (bf16_t*)sum, (bf16_t*)norm, rows, cols, eps);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;

@@ -66,7 +66,7 @@ def test_rmsnorm_row_vector_path(dtype, rows, cols):
     assert (y - ref).abs().max().item() <= tol
 
 
-@pytest.mark.parametrize("rows,cols", [(37, 768), (3, 8), (129, 2048), (6, 1000)])
+@pytest.mark.parametrize("rows,cols", [(37, 768), (3, 8), (129, 2048), (6, 1000), (5, 4096), (9, 1032)])
 def test_add3_rmsnorm_equals_separate_kernels(rows, cols):
     """The fused residual-sum + norm is bit-identical to add3 followed by rmsnorm, and both
     agree with the fp32 statement of the two operations."""
