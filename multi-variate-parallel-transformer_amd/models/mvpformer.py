@@ -310,13 +310,19 @@ class HMVPFormer(BrainModel):
             out, past = self.mvpformer(inputs_embeds=embeds, past_key_values=past)
         return self.head(out[:, -1].float().mean(dim=1).to(out.dtype)), past
 
-    def capture_stream(self, past, segment_like: torch.Tensor):
+    def capture_stream(self, past, segment_like: torch.Tensor, predict: bool = False):
         """Turn a stream whose window is full into a replayable HIP graph.  `past` is what
         classify_step returned once max_steps segments were in (MvpaKVCache per block);
         segment_like a tensor shaped like one segment batch [B, ch, len].  Returns a callable
         step(segment) -> logits that copies the segment into a fixed buffer and replays the graph
         of one classify_step on ring caches (the caches are copied; `past` is left alone).  The
-        returned logits tensor is overwritten by the next call."""
+        returned logits tensor is overwritten by the next call.  predict=True captures predict_step
+        instead (`past` as predict_step returned it): step(segment) -> (similarity, prediction),
+        the similarity scoring the forecast of the call before."""
+        forecast = None
+        if predict:
+            past, forecast = past
+            forecast = forecast.clone()
         clock = MvpaRingClock(past[0].max_steps, past[0].max_steps - 1, segment_like.device)
         rings = tuple(MvpaRingCache.from_cache(c, clock) for c in past)     # one clock for all blocks
         inp = segment_like.clone()
@@ -326,12 +332,17 @@ class HMVPFormer(BrainModel):
             bsz, ch, seg = inp.shape
             embeds = self.encoder(inp.reshape(bsz * ch, seg)).view(bsz, 1, ch, -1)
             out, _ = self.mvpformer(inputs_embeds=embeds, past_key_values=rings)
+            if predict:
+                sim = torch.cosine_similarity(embeds[:, 0].float(), forecast.float(), dim=-1)
+                forecast.copy_(self.head(out[:, -1]))
+                return sim, forecast
             return self.head(out[:, -1].float().mean(dim=1).to(out.dtype))
 
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         saved = [(r.k.clone(), r.v.clone()) for r in rings]
         head0 = clock.head32.clone()
+        forecast0 = forecast.clone() if predict else None
         with torch.cuda.stream(side):
             for _ in range(2):                      # warm-up: fills every host-side cache of the path
                 one_step()
@@ -340,6 +351,8 @@ class HMVPFormer(BrainModel):
             r.k.copy_(k0)
             r.v.copy_(v0)
         clock.head32.copy_(head0)
+        if predict:
+            forecast.copy_(forecast0)
         del saved
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):

@@ -285,3 +285,24 @@ def test_streamed_next_segment_scores_match_the_window_forward():
     # only when t+1 == T; earlier columns see the same relative rows through position_end, so all
     # columns agree
     assert (got - want).abs().max().item() <= 3e-2
+
+
+def test_graph_replayed_prediction_stream_matches_eager_steps():
+    """capture_stream(predict=True): replays of predict_step on ring caches give the similarity
+    and the forecast of the eager predict_step, call after call (bf16 tolerance)."""
+    from models.mvpformer import HMVPFormer, MVPFormerConfig, MVPFormerHead
+    from models.fftencoder import WaveEncoder
+    torch.manual_seed(13)
+    cfg = MVPFormerConfig(n_embd=256, n_head=4, n_head_kv=2, n_layer=2, n_positions=9, n_channels=12, n_inner=512)
+    model = HMVPFormer(cfg, WaveEncoder(size_input=512, size_output=256), MVPFormerHead(256, 256)).to("cuda", torch.bfloat16).eval()
+    B, T, C = 2, cfg.n_positions, 12
+    batch = torch.randn(B, 3 * T, C, 512, device="cuda")
+    past = None
+    for t in range(T):
+        _, _, past = model.predict_step(batch[:, t], past)
+    step = model.capture_stream(past, batch[:, 0], predict=True)
+    for t in range(T, 3 * T):
+        sim_e, pred_e, past = model.predict_step(batch[:, t], past)
+        sim_g, pred_g = step(batch[:, t])
+        assert (sim_g - sim_e).abs().max().item() <= 3e-2, t
+        assert (pred_g.float() - pred_e.float()).abs().max().item() <= 3e-2 * (pred_e.float().abs().max().item() + 1e-3), t
