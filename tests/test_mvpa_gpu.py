@@ -462,3 +462,30 @@ def test_last_step_on_a_ring_of_slots(cfg, n, head):
     v_ring.copy_(v5[:, :, step_of_slot].reshape(B, Hkv, T * C, Dh))
     got2 = mvpa_hip.mvpa_forward(q_last, k_ring, v_ring, *tabs, last_step_only=True, key_splits=n, ring_head=head_t)
     assert (got2.float() - ref.float()).abs().max().item() <= 2e-2
+
+
+def test_decoding_step_at_base_model_size_matches_the_full_forward():
+    """The base model's attention shape (B1 H16 Hkv8 C128 T512 Dh128): one decoding step with the
+    binding's own key runs (16 of 32 steps, the 8-wave key-split build) and on a ring of slots,
+    against the last time step of the full forward."""
+    cfg = dict(B=1, C=128, T=512, H=16, Hkv=8, Dh=128)
+    inp = make_mvpa_inputs(seed=41, **cfg).to("cuda", torch.bfloat16)
+    C, T = cfg["C"], cfg["T"]
+    tabs = (inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan)
+    full, lse_full = mvpa_hip.mvpa_forward(inp.q, inp.k, inp.v, *tabs, return_lse=True)
+    ref, lse_ref = full[:, :, -C:].float(), lse_full[:, :, -C:]
+    q_last = inp.q[:, :, -C:]
+    assert mvpa_hip.default_key_splits(1, 16, T) == 16
+    got, lse_got = mvpa_hip.mvpa_forward(q_last, inp.k, inp.v, *tabs, return_lse=True, last_step_only=True)
+    assert (got.float() - ref).abs().max().item() <= 2e-2
+    assert ((got.float() - ref).norm() / ref.norm()).item() <= 5e-3
+    assert (lse_got - lse_ref).abs().max().item() <= 2e-3
+    head = 200
+    slot = torch.arange(T, device="cuda")
+    step_of_slot = T - 1 - (head - slot) % T
+    k_ring = inp.k.view(1, 8, T, C, 128)[:, :, step_of_slot].reshape(1, 8, T * C, 128).contiguous()
+    v_ring = inp.v.view(1, 8, T, C, 128)[:, :, step_of_slot].reshape(1, 8, T * C, 128).contiguous()
+    ring, _ = mvpa_hip.mvpa_forward(q_last, k_ring, v_ring, *tabs, return_lse=True, last_step_only=True,
+                                    ring_head=torch.tensor([head], dtype=torch.int32, device="cuda"))
+    assert (ring.float() - ref).abs().max().item() <= 2e-2
+    assert ((ring.float() - ref).norm() / ref.norm()).item() <= 5e-3
