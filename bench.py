@@ -2,7 +2,7 @@
 """Benchmark of the MVPA forward hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3] [--no-cpu] [--no-model]
-                    [--no-stream] [--no-backward] [--base-model] [--copy-probe] [--no-mfma-probe]
+                    [--no-stream] [--no-backward] [--base-model] [--copy-probe] [--prewarm P]
 
 A step is one fused MVPA forward (one kernel launch) over one batch of synthetic inputs that
 are already resident in HBM.  The default workload is the configuration the headline metric
@@ -11,10 +11,14 @@ line with the metric, the roofline of the attention kernel (achieved = algorithm
 launch / HIP-event time per launch) and a bounded CPU baseline (the oracle's op-by-op
 restatement of the reference PyTorch path on this box's host cores).  Beside them, never part
 of `value`: `backward` (one mvpa_backward call on the same workload), `mvpformer_s` (the
-MVPFormer-S forward in windows per second), `mvpformer_s_stream` (one new segment of a stream
-against cached keys and values, beside the full forward over the same window) and, on request,
-`mvpformer_base` and `mfma_probe` (what a stream of nothing but bf16 MFMAs reaches on this box,
-on smooth and on random operands).
+MVPFormer-S forward in windows per second, with the oracle stack on the host cores beside it),
+`mvpformer_s_stream` (one new segment of a stream against cached keys and values, beside the
+full forward over the same window) and, on request, `mvpformer_base`.
+
+The GPU's clocks take a few dozen milliseconds of work to reach their steady state after a
+process starts.  Before the W warm-up steps the benchmark therefore runs a fixed number of
+launches of the same kernel (`prewarm_launches` in the output, outside the timed region), so
+that the figure does not depend on how small W is.
 """
 from __future__ import annotations
 
@@ -33,8 +37,10 @@ for _p in (PKG, ROOT):
 BF16_DENSE_PEAK_TFLOPS = 2500.0       # MI355X published dense bf16 MFMA peak
 
 # HBM bytes per launch of the attention kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by
-# what the same counters read for a plain 256 MiB copy (profiles/mvpa_mfma_kernel_c2.md).
-MEASURED_TRAFFIC_BYTES = {"c2": 402.4e6}
+# what the same counters read for a plain device copy of known size; the profile summary named
+# beside each figure holds the two counter runs.
+MEASURED_TRAFFIC_BYTES = {"c2": (402.4e6, "profiles/mvpa_mfma_kernel_c2.md")}
+PREWARM_LAUNCHES = 150
 
 WORKLOADS = {
     "c2": dict(B=4, C=64, T=128, H=16, Hkv=16, Dh=64, validity=False),
@@ -56,7 +62,7 @@ def algorithmic_flops(B, H, T, C, Dh, window=10):
     return B * H * 2 * Dh * (p_causal + p_window + n * (T + C))
 
 
-def cpu_baseline(cfg, budget_s=12.0):
+def cpu_baseline(cfg, budget_s=8.0):
     """Oracle restatement of the reference PyTorch MVPA (same op sequence, same N^2 traffic) on
     the host CPU for a bounded sample: whole (b, h) slices of the workload, fp32."""
     import torch
@@ -94,18 +100,61 @@ def cpu_baseline(cfg, budget_s=12.0):
     }
 
 
+def cpu_baseline_model(B=1, C=64, T=64, seg=512):
+    """The oracle stack (encoder, parallel blocks with the op-by-op attention restatement, final
+    norm) on the host cores, fp32, with MVPFormer-S dims: one window at full length with one and
+    with two blocks; a block's cost is the difference, and the 12-block figure is extrapolated
+    from it (stated in the result)."""
+    import torch
+    from mvpa_hip.synthetic import make_ieeg
+    from models.configs import MVPFORMER_S
+    from oracle import mvpa_oracle as O
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    E, H, Hkv, inner = (MVPFORMER_S[k] for k in ("n_embd", "n_head", "n_head_kv", "n_inner"))
+    kv = E // H * Hkv
+    g = torch.Generator().manual_seed(0)
+    rn = lambda *shape: torch.randn(*shape, generator=g) * 0.02      # noqa: E731
+    dwt = sum(O.dwt_sizes(seg))
+    params = {"encoder.ln.weight": torch.ones(dwt), "encoder.proj.weight": rn(E, dwt),
+              "mvpformer.ln_f.weight": torch.ones(E),
+              "mvpformer.positional_embedding.weight": rn(T, E),
+              "mvpformer.channel_embedding.weight": rn(C, E)}
+    for i in range(1):
+        pre = f"mvpformer.h.{i}."
+        params.update({pre + "ln_1.weight": torch.ones(E), pre + "attn.q_attn.weight": rn(E, E),
+                       pre + "attn.c_attn.weight": rn(2 * kv, E), pre + "attn.position_net.weight": rn(kv, E),
+                       pre + "attn.channel_net.weight": rn(kv, E), pre + "attn.c_proj.weight": rn(E, E),
+                       pre + "attn.attn_bias": rn(3 * kv), pre + "mlp.gate_proj.weight": rn(inner, E),
+                       pre + "mlp.up_proj.weight": rn(inner, E), pre + "mlp.down_proj.weight": rn(E, inner)})
+    x = make_ieeg(B, C, T, seg, seed=0)
+    times = {}
+    with torch.no_grad():
+        O.mvpformer_forward(x[:, :8], params, dict(n_layer=1, n_head=H, n_head_kv=Hkv))   # thread pool warm-up
+        for n_layer in (0, 1):
+            t0 = time.perf_counter()
+            O.mvpformer_forward(x, params, dict(n_layer=n_layer, n_head=H, n_head_kv=Hkv))
+            times[n_layer] = time.perf_counter() - t0
+    per_block = max(times[1] - times[0], 1e-9)
+    full = times[0] + MVPFORMER_S["n_layer"] * per_block
+    return {"value": round(B / full, 4), "unit": "windows/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"oracle stack, fp32, B={B} C={C} T={T} segments of {seg} samples: encoder + final "
+                      f"norm {times[0]:.2f} s, one block {per_block:.2f} s (timed once, first call at this "
+                      f"size); extrapolated to 12 blocks: {full:.1f} s per window"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # the first few dozen launches after start-up run ~12 % slower (clocks still ramping): the
-    # default warm-up covers that
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--prewarm", type=int, default=PREWARM_LAUNCHES,
+                    help="launches before the warm-up steps that bring the clocks up (untimed)")
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-model", action="store_true", help="skip the MVPFormer-S forward leg")
-    ap.add_argument("--no-mfma-probe", action="store_true",
-                    help="skip the pure MFMA stream on smooth and on random operands")
     ap.add_argument("--no-stream", action="store_true", help="skip the MVPFormer-S streamed-segment leg")
     ap.add_argument("--no-backward", action="store_true", help="skip the MVPA backward leg")
     ap.add_argument("--base-model", action="store_true",
@@ -141,6 +190,9 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    for _ in range(max(0, args.prewarm)):
+        step()
+    torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -160,7 +212,8 @@ def main():
     line = {
         "metric": "MVPA fwd TFLOP/s (algorithmic flops), bf16, 1 GPU",
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4),
+        "steps": args.steps, "warmup": args.warmup, "prewarm_launches": max(0, args.prewarm),
+        "ms_per_step": round(wall_ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{args.workload}: MVPA forward B={B} C={C} T={T} H={H} Hkv={Hkv} "
@@ -170,8 +223,9 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 2),
                      "peak": BF16_DENSE_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(kern_tflops / BF16_DENSE_PEAK_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "kernel": "mvpa_mfma_kernel",
-                     "kernel_ms": round(kern_ms, 4)},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, (None, None))[0],
+                     "traffic_source": MEASURED_TRAFFIC_BYTES.get(args.workload, (None, None))[1],
+                     "kernel": "mvpa_mfma_kernel", "kernel_ms": round(kern_ms, 4)},
     }
     if not args.no_backward and C <= 128:   # shapes the matrix-core backward serves
         # the backward of the same workload (reported beside the headline, never part of `value`):
@@ -196,11 +250,6 @@ def main():
         line["backward"] = {"ms_per_step": round(ev0.elapsed_time(ev1) / n_bwd, 4), "steps": n_bwd,
                             "kernels": "mvpa_bwd_query_mfma_kernel + mvpa_bwd_key_mfma_kernel",
                             "outputs": "dq (content share), dk, dv, dbias_time, dbias_chan (fp32)"}
-    if not args.no_mfma_probe:
-        line["mfma_probe"] = {
-            "smooth_operands_tflops": round(mvpa_hip.mfma_probe_tflops(False), 1),
-            "random_operands_tflops": round(mvpa_hip.mfma_probe_tflops(True), 1),
-            "what": "a stream of nothing but v_mfma_f32_32x32x16_bf16 on every SIMD, two waves each"}
     if not args.no_model:
         try:
             from models.bench_model import mvpformer_s_windows_per_s
@@ -215,6 +264,8 @@ def main():
         line["mvpformer_base"] = mvpformer_base_forward_ms(stream=not args.no_stream)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(cfg)
+        if line.get("mvpformer_s"):
+            line["mvpformer_s"]["cpu_baseline"] = cpu_baseline_model()
     print(json.dumps(line))
 
 

@@ -269,15 +269,6 @@ int mvpa_ring_append_bf16(const void* k_new, const void* v_new, void* k_ring, vo
                           int32_t steps, int64_t stride_b, int64_t stride_h, int64_t stride_c,
                           void* stream);
 
-/* Measurement aid with no counterpart in the reference: a stream of nothing but
- * v_mfma_f32_32x32x16_bf16 on every SIMD (512 workgroups x 4 waves x iters x 8 instructions,
- * mvpa_probe_mfma_flops(iters) flop in all), on smooth operands (the same small value in every
- * lane) or, with random_operands != 0, on operands with random bit patterns.  The caller times the
- * launch; sink receives 512*256 floats that only keep the work alive.  The benchmark reports the
- * two rates beside the attention kernel's fraction of the published peak. */
-int mvpa_probe_mfma(int32_t random_operands, int32_t iters, float* sink, void* stream);
-int64_t mvpa_probe_mfma_flops(int32_t iters);
-
 #ifdef __cplusplus
 }
 #endif

@@ -288,10 +288,10 @@ static int launch_bwd_t(const mvpa_bwd_args* a, hipStream_t stream, bool query_p
   (void)hipFuncSetAttribute((const void*)kq, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_q);
   const unsigned nb = (unsigned)((N + BWD_THREADS - 1) / BWD_THREADS);
   if (query_pass) {
-    hipLaunchKernelGGL(kq, dim3(nb, a->B * a->H), dim3(BWD_THREADS), lds_q, stream, *a);
+    MVPA_LAUNCH(kq, dim3(nb, a->B * a->H), dim3(BWD_THREADS), lds_q, stream, *a);
     if (hipGetLastError() != hipSuccess) return MVPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL(kk, dim3(nb, a->B * a->Hkv), dim3(BWD_THREADS), lds_k, stream, *a);
+  MVPA_LAUNCH(kk, dim3(nb, a->B * a->Hkv), dim3(BWD_THREADS), lds_k, stream, *a);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 

@@ -675,7 +675,7 @@ static void launch_query(const mvpa_bwd_args* a, hipStream_t stream, int q0, int
   dim3 grid((unsigned)(nt * a->B * a->H));
   auto kern = mvpa_bwd_query_mfma_kernel<NCT>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  hipLaunchKernelGGL(kern, grid, dim3(nw * 64), lds, stream, *a, q0, k0, accum);
+  MVPA_LAUNCH(kern, grid, dim3(nw * 64), lds, stream, *a, q0, k0, accum);
 }
 
 // ==========================================================================================
@@ -1014,7 +1014,7 @@ static void launch_key(const mvpa_bwd_args* a, hipStream_t stream, int k0, int q
   dim3 grid((unsigned)(((a->T + kt - 1) / kt) * a->B * a->Hkv));
   auto kern = mvpa_bwd_key_mfma_kernel<NCT, MASKED>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  hipLaunchKernelGGL(kern, grid, dim3(nw * 64), lds, stream, *a, k0, q0, accum);
+  MVPA_LAUNCH(kern, grid, dim3(nw * 64), lds, stream, *a, k0, q0, accum);
 }
 
 // Both passes.  Up to 32 channels: one launch each with one channel tile per wave; up to 64: one

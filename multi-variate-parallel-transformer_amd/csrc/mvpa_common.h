@@ -69,6 +69,14 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 }  // namespace mvpa
 
+// A launch whose status is this call's own: HIP keeps the last error until it is read, so an
+// error left by unrelated earlier work would otherwise be reported as a failure of this launch.
+#define MVPA_LAUNCH(...)            \
+  do {                              \
+    (void)hipGetLastError();        \
+    hipLaunchKernelGGL(__VA_ARGS__); \
+  } while (0)
+
 // ---- launchers implemented by the kernel translation units ----------------------------------
 int mvpa_launch_generic(const mvpa_fwd_args* a, hipStream_t stream);
 int mvpa_launch_mfma(const mvpa_fwd_args* a, hipStream_t stream);

@@ -601,7 +601,7 @@ static int launch_big(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, in
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
   constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;
   dim3 grid((unsigned)((N + OUT_COLS - 1) / OUT_COLS), (unsigned)((M + 255) / 256));
-  hipLaunchKernelGGL(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy);
+  MVPA_LAUNCH(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 
@@ -869,7 +869,7 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M,
   auto kern = linear_bf16_skinny_kernel<EPI, XT>;
   if (lds > 64 * 1024)
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-  hipLaunchKernelGGL(kern, dim3((unsigned)((N + 31) / 32)), dim3(SK_WAVES * 64), lds, s, x, w, y, M, N, K, ldx, ldw, ldy);
+  MVPA_LAUNCH(kern, dim3((unsigned)((N + 31) / 32)), dim3(SK_WAVES * 64), lds, s, x, w, y, M, N, K, ldx, ldw, ldy);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 
@@ -906,14 +906,14 @@ extern "C" int mvpa_linear_bf16_splitk(const void* x, const void* w, void* y, in
   int per_group, slices;          // slices: partial tiles per output tile = workgroup rows
   splitk_groups(nw, K, &per_group, &slices);
   (void)hipFuncSetAttribute((const void*)linear_splitk_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SPK_LDS_BYTES);
-  hipLaunchKernelGGL(linear_splitk_kernel, dim3((unsigned)((nw + SPK_COLS - 1) / SPK_COLS), (unsigned)slices), dim3(256),
+  MVPA_LAUNCH(linear_splitk_kernel, dim3((unsigned)((nw + SPK_COLS - 1) / SPK_COLS), (unsigned)slices), dim3(256),
                      SPK_LDS_BYTES, s, (const bf16_t*)x, (const bf16_t*)w, (float*)ws, M, nw, K, ldx, ldw, per_group);
   const int64_t items = M * ((N + 3) / 4);
   if (epilogue == 1)
-    hipLaunchKernelGGL(linear_splitk_reduce_kernel<1>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
+    MVPA_LAUNCH(linear_splitk_reduce_kernel<1>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
                        (const float*)ws, (bf16_t*)y, M, N, nw, slices, ldy);
   else
-    hipLaunchKernelGGL(linear_splitk_reduce_kernel<0>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
+    MVPA_LAUNCH(linear_splitk_reduce_kernel<0>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
                        (const float*)ws, (bf16_t*)y, M, N, nw, slices, ldy);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
@@ -954,10 +954,10 @@ extern "C" int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M
   }
   if (epilogue == 1) {
     dim3 grid((unsigned)((N + GBN / 2 - 1) / (GBN / 2)), (unsigned)((M + GBM - 1) / GBM));
-    hipLaunchKernelGGL(linear_bf16_kernel<1>, grid, dim3(256), 0, s, xp, wp, yp, M, N, K, ldx, ldw, ldy);
+    MVPA_LAUNCH(linear_bf16_kernel<1>, grid, dim3(256), 0, s, xp, wp, yp, M, N, K, ldx, ldw, ldy);
   } else {
     dim3 grid((unsigned)((N + GBN - 1) / GBN), (unsigned)((M + GBM - 1) / GBM));
-    hipLaunchKernelGGL(linear_bf16_kernel<0>, grid, dim3(256), 0, s, xp, wp, yp, M, N, K, ldx, ldw, ldy);
+    MVPA_LAUNCH(linear_bf16_kernel<0>, grid, dim3(256), 0, s, xp, wp, yp, M, N, K, ldx, ldw, ldy);
   }
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
@@ -977,23 +977,23 @@ extern "C" int mvpa_rmsnorm(const void* x, const float* weight, void* y, int64_t
   if (vec_ok) {
     dim3 vgrid((unsigned)((rows + 3) / 4));
     if (in_dtype == MVPA_F32 && out_dtype == MVPA_F32)
-      hipLaunchKernelGGL((rmsnorm_rows_kernel<float, float>), vgrid, block, 0, s, (const float*)x, weight, (float*)y, rows, cols, ldx, ldy, eps);
+      MVPA_LAUNCH((rmsnorm_rows_kernel<float, float>), vgrid, block, 0, s, (const float*)x, weight, (float*)y, rows, cols, ldx, ldy, eps);
     else if (in_dtype == MVPA_F32)
-      hipLaunchKernelGGL((rmsnorm_rows_kernel<float, bf16_t>), vgrid, block, 0, s, (const float*)x, weight, (bf16_t*)y, rows, cols, ldx, ldy, eps);
+      MVPA_LAUNCH((rmsnorm_rows_kernel<float, bf16_t>), vgrid, block, 0, s, (const float*)x, weight, (bf16_t*)y, rows, cols, ldx, ldy, eps);
     else if (out_dtype == MVPA_BF16)
-      hipLaunchKernelGGL((rmsnorm_rows_kernel<bf16_t, bf16_t>), vgrid, block, 0, s, (const bf16_t*)x, weight, (bf16_t*)y, rows, cols, ldx, ldy, eps);
+      MVPA_LAUNCH((rmsnorm_rows_kernel<bf16_t, bf16_t>), vgrid, block, 0, s, (const bf16_t*)x, weight, (bf16_t*)y, rows, cols, ldx, ldy, eps);
     else
-      hipLaunchKernelGGL((rmsnorm_rows_kernel<bf16_t, float>), vgrid, block, 0, s, (const bf16_t*)x, weight, (float*)y, rows, cols, ldx, ldy, eps);
+      MVPA_LAUNCH((rmsnorm_rows_kernel<bf16_t, float>), vgrid, block, 0, s, (const bf16_t*)x, weight, (float*)y, rows, cols, ldx, ldy, eps);
     return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
   }
   if (in_dtype == MVPA_F32 && out_dtype == MVPA_F32)
-    hipLaunchKernelGGL((rmsnorm_kernel<float, float>), grid, block, 0, s, (const float*)x, weight, (float*)y, cols, ldx, ldy, eps);
+    MVPA_LAUNCH((rmsnorm_kernel<float, float>), grid, block, 0, s, (const float*)x, weight, (float*)y, cols, ldx, ldy, eps);
   else if (in_dtype == MVPA_F32 && out_dtype == MVPA_BF16)
-    hipLaunchKernelGGL((rmsnorm_kernel<float, bf16_t>), grid, block, 0, s, (const float*)x, weight, (bf16_t*)y, cols, ldx, ldy, eps);
+    MVPA_LAUNCH((rmsnorm_kernel<float, bf16_t>), grid, block, 0, s, (const float*)x, weight, (bf16_t*)y, cols, ldx, ldy, eps);
   else if (in_dtype == MVPA_BF16 && out_dtype == MVPA_BF16)
-    hipLaunchKernelGGL((rmsnorm_kernel<bf16_t, bf16_t>), grid, block, 0, s, (const bf16_t*)x, weight, (bf16_t*)y, cols, ldx, ldy, eps);
+    MVPA_LAUNCH((rmsnorm_kernel<bf16_t, bf16_t>), grid, block, 0, s, (const bf16_t*)x, weight, (bf16_t*)y, cols, ldx, ldy, eps);
   else if (in_dtype == MVPA_BF16 && out_dtype == MVPA_F32)
-    hipLaunchKernelGGL((rmsnorm_kernel<bf16_t, float>), grid, block, 0, s, (const bf16_t*)x, weight, (float*)y, cols, ldx, ldy, eps);
+    MVPA_LAUNCH((rmsnorm_kernel<bf16_t, float>), grid, block, 0, s, (const bf16_t*)x, weight, (float*)y, cols, ldx, ldy, eps);
   else
     return MVPA_ERR_DTYPE;
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
@@ -1005,12 +1005,12 @@ extern "C" int mvpa_add3_bf16(const void* a, const void* b, const void* c, void*
   if (n <= 0) return MVPA_ERR_SHAPE;
   if (n % 8 == 0 && (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)out) & 15) == 0) {
     const int64_t n8 = n / 8;
-    hipLaunchKernelGGL(add3_bf16_vec_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0,
+    MVPA_LAUNCH(add3_bf16_vec_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)c,
                        (bf16_t*)out, n8);
     return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL(add3_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+  MVPA_LAUNCH(add3_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)c,
                      (bf16_t*)out, n);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
@@ -1026,7 +1026,7 @@ extern "C" int mvpa_ring_append_bf16(const void* k_new, const void* v_new, void*
       (((uintptr_t)k_new | (uintptr_t)v_new | (uintptr_t)k_ring | (uintptr_t)v_ring) & 15))
     return MVPA_ERR_ALIGN;
   const int64_t total = (int64_t)B * Hkv * C * (Dh / 8);
-  hipLaunchKernelGGL(ring_append_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+  MVPA_LAUNCH(ring_append_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)k_new, (const bf16_t*)v_new, (bf16_t*)k_ring,
                      (bf16_t*)v_ring, head, Hkv, C, Dh, steps, stride_b, stride_h, stride_c, total);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
@@ -1042,7 +1042,7 @@ extern "C" int mvpa_add3_rmsnorm_bf16(const void* a, const void* b, const void* 
     return MVPA_ERR_ALIGN;
   auto kern = cols <= 1024 ? add3_rmsnorm_bf16_kernel<2> : cols <= 2048 ? add3_rmsnorm_bf16_kernel<4>
                                                                         : add3_rmsnorm_bf16_kernel<0>;
-  hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+  MVPA_LAUNCH(kern, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)c,
                      weight, (bf16_t*)sum, (bf16_t*)norm, rows, cols, eps);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
@@ -1056,7 +1056,11 @@ extern "C" int mvpa_wavedec_db4(const float* x, float* coeffs, int64_t M, int32_
   for (int lv = 0; lv < levels; ++lv) { n = (n + 7) >> 1; total += n; }
   total += n;
   if (total != dwt_size) return MVPA_ERR_SHAPE;
-  hipLaunchKernelGGL(wavedec_db4_kernel, dim3((unsigned)M), dim3(256), 2 * L * sizeof(float),
+  // two ping-pong rows of L floats: past 64 KiB of dynamic LDS the kernel has to be told
+  if (2 * L * sizeof(float) > 64 * 1024)
+    (void)hipFuncSetAttribute((const void*)wavedec_db4_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)(2 * L * sizeof(float)));
+  MVPA_LAUNCH(wavedec_db4_kernel, dim3((unsigned)M), dim3(256), 2 * L * sizeof(float),
                      (hipStream_t)stream, x, coeffs, L, levels, dwt_size, ldc);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }

@@ -197,7 +197,7 @@ static int launch_generic_t(const mvpa_fwd_args* a, hipStream_t stream) {
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   const int n_rows = (a->flags & MVPA_FLAG_LAST_STEP) ? a->C : N;
   dim3 grid((n_rows + GEN_THREADS - 1) / GEN_THREADS, a->B * a->H);
-  hipLaunchKernelGGL(kern, grid, dim3(GEN_THREADS), lds, stream, *a, chan_table);
+  MVPA_LAUNCH(kern, grid, dim3(GEN_THREADS), lds, stream, *a, chan_table);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 
@@ -227,7 +227,7 @@ extern "C" int mvpa_debug_maps(int32_t T, int32_t C, int32_t window, uint32_t fl
   if (T <= 0 || C <= 0) return MVPA_ERR_CTX;
   const int N = T * C;
   dim3 grid((N + 255) / 256, N);
-  hipLaunchKernelGGL(mvpa::mvpa_debug_maps_kernel, grid, dim3(256), 0, (hipStream_t)stream, T, C,
+  MVPA_LAUNCH(mvpa::mvpa_debug_maps_kernel, grid, dim3(256), 0, (hipStream_t)stream, T, C,
                      window, flags, chan_valid, time_idx, chan_idx, mask_bits);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }

@@ -49,6 +49,7 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 #define kOnes2 (bf16x2{(__bf16)1.0f, (__bf16)1.0f})
+constexpr float kMFloor = -1.0e30f;     // "nothing seen yet" value of a running maximum
 
 // order LDS traffic between the lanes of ONE wave (no workgroup barrier needed)
 __device__ inline void wave_lds_sync() {
@@ -465,6 +466,9 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 #pragma unroll
       for (int i = 0; i < 16; ++i) mx = fmaxf(mx, Bc[t][i]);
     mc = xhalf_max(mx);
+    // every key channel of this wave's part absent (a KH = 2 wave whose channels 64.. are all
+    // masked): Ec = 0 and sumEc = 0 with a finite reference, so the part contributes exactly nothing
+    if (mc == -INFINITY) mc = 0.f;
     float se = 0.f;
 #pragma unroll
     for (int t = 0; t < NCT; ++t) {
@@ -487,8 +491,11 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
       for (int i = 0; i < 16; ++i) Bc[t][i] *= inv_d;
   }
 
-  // running soft-max state of this lane's query; l is a per-half-wave partial sum
-  float m_run = -INFINITY, l_run = 0.f;
+  // running soft-max state of this lane's query; l is a per-half-wave partial sum.  The reference
+  // point starts at a finite floor instead of -inf: exp2(floor - m) is 0 all the same, and a step
+  // whose scores are all -inf (every key of the part masked) gives exp2(-inf + (st - floor)) = 0
+  // instead of exp2(-inf + inf) = NaN
+  float m_run = kMFloor, l_run = 0.f;
   f32x16 acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
@@ -559,7 +566,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     cm = xhalf_max(cm);
     if (tk <= far_max) {                       // the slab holds at least one far step
       const float m_new = fmaxf(m_run, cm + mc);
-      const float alpha = fast_exp2(m_run - m_new);     // exp2(-inf) = 0 on the first slab
+      const float alpha = fast_exp2(m_run - m_new);     // exp2(floor - m) = 0 on the first slab
       m_run = m_new;
       l_run *= alpha;
 #pragma unroll
@@ -827,8 +834,10 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     if (mpar == 1) return;
     const float m1 = mb[0], l1 = mb[64];
     const float m = fmaxf(m_run, m1);
-    const float a0 = m_run == -INFINITY ? 0.f : fast_exp2(m_run - m);
-    const float a1 = m1 == -INFINITY ? 0.f : fast_exp2(m1 - m);
+    // a state that never saw a key still holds the floor: its weight is exp2(floor - m) = 0 and
+    // its l and accumulators are 0, unless both are empty (no valid key at all: 0/0 as before)
+    const float a0 = fast_exp2(m_run - m);
+    const float a1 = fast_exp2(m1 - m);
     m_run = m;
     l_run = a0 * l_run + a1 * l1;
 #pragma unroll
@@ -913,10 +922,10 @@ static int launch_one(const mvpa_fwd_args* a, hipStream_t stream) {
                             (int)G::LDS_BYTES);
   const int nt = (G::TQW == 2 && STAGES == 4 && KH == 1) ? 1 + a->T / 2 : (a->T + G::TQW - 1) / G::TQW;   // as in the kernel
   dim3 grid((unsigned)((last ? n_split : nt) * a->B * a->H));
-  hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), G::LDS_BYTES, stream, *a);
+  MVPA_LAUNCH(kern, grid, dim3(G::THREADS), G::LDS_BYTES, stream, *a);
   if (n_split > 1) {
     const int rows = a->B * a->H * a->C;
-    hipLaunchKernelGGL(mvpa_split_merge_kernel<DH>, dim3((unsigned)((rows + 2048 / DH - 1) / (2048 / DH))), dim3(256), 0, stream, *a);
+    MVPA_LAUNCH(mvpa_split_merge_kernel<DH>, dim3((unsigned)((rows + 2048 / DH - 1) / (2048 / DH))), dim3(256), 0, stream, *a);
   }
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }

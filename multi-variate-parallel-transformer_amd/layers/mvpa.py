@@ -296,6 +296,9 @@ class MVPFormerGQAAttention(torch.nn.Module):
             s /= float(self.layer_idx + 1)                 # layers/mvpa.py:253-254
         return s
 
+    def _content(self) -> bool:
+        return bool(self.global_att)                       # layers/mvpa.py:188-222, 230
+
     def _attend(self, hidden_states, positional_embedding, channel_embedding, attention_mask,
                 head_mask, use_cache, window, layer_past=None):
         if self.training and (self.attn_dropout.p > 0 or self.resid_dropout.p > 0):
@@ -328,7 +331,7 @@ class MVPFormerGQAAttention(torch.nn.Module):
             merged = torch.empty((bsz, n, h, dh), dtype=dt, device=hidden_states.device)
             mvpa_hip.mvpa_forward(
                 q, k, v, u, vb, z, k_time, k_chan, sm_scale=self._scale(), window=window,
-                causal=True, content=bool(self.global_att), chan_valid=chan_valid,
+                causal=True, content=self._content(), chan_valid=chan_valid,
                 key_bias=key_bias, out=merged.permute(0, 2, 1, 3),
                 fp8_qk=self.fp8_qk and dt == torch.bfloat16 and key_bias is None)
             if head_mask is not None:                       # layers/mvpa.py:274-275
@@ -397,7 +400,7 @@ class MVPFormerGQAAttention(torch.nn.Module):
             mvpa_hip.mvpa_forward(
                 q, k.reshape(bsz, hkv, t_len * c_len, dh), v.reshape(bsz, hkv, t_len * c_len, dh),
                 u, vb, z, k_time, k_chan, sm_scale=self._scale(), window=window, causal=True,
-                content=bool(self.global_att), chan_valid=chan_valid, key_bias=key_bias,
+                content=self._content(), chan_valid=chan_valid, key_bias=key_bias,
                 out=merged.permute(0, 2, 1, 3), last_step_only=True,
                 ring_head=ring.head32 if ring is not None else None,
                 fp8_qk=self.fp8_qk and dt == torch.bfloat16 and key_bias is None)
@@ -447,6 +450,16 @@ class MVPFormerGQAFlashAttention(MVPFormerGQAAttention):
     (see _attend_step)."""
 
     _honours_masks = False
+
+    # The reference's flash layer calls its kernel with sm_scale = 1/sqrt(Dh) and the content term
+    # always on, whatever scale_attn_weights, scale_attn_by_inverse_layer_idx and global_att say
+    # (layers/mvpa.py:382-397); the same here, so the two classes differ exactly where the
+    # reference's do.
+    def _scale(self) -> float:
+        return 1.0 / self.head_dim ** 0.5
+
+    def _content(self) -> bool:
+        return True
 
     def forward(self, hidden_states, positional_embedding, channel_embedding, layer_past=None,
                 attention_mask=None, head_mask=None, encoder_hidden_states=None,

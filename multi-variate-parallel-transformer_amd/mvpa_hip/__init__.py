@@ -98,10 +98,6 @@ def load_library() -> ctypes.CDLL:
     lib.mvpa_linear_splitk_ws_bytes.argtypes = [i64, i64, i64, i32]
     lib.mvpa_ring_append_bf16.restype = ctypes.c_int
     lib.mvpa_ring_append_bf16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i64, i64, i64, vp]
-    lib.mvpa_probe_mfma.restype = ctypes.c_int
-    lib.mvpa_probe_mfma.argtypes = [i32, i32, vp, vp]
-    lib.mvpa_probe_mfma_flops.restype = ctypes.c_int64
-    lib.mvpa_probe_mfma_flops.argtypes = [i32]
     lib.mvpa_split_ws_bytes.restype = ctypes.c_size_t
     lib.mvpa_split_ws_bytes.argtypes = [ctypes.POINTER(MvpaFwdArgs)]
     lib.mvpa_forward.restype = ctypes.c_int
@@ -364,22 +360,6 @@ def debug_maps(T: int, C: int, window: int = 10, flags: int = 15, chan_valid=Non
     _check(lib.mvpa_debug_maps(T, C, window, flags, cv.data_ptr() if cv is not None else None,
                                ti.data_ptr(), ci.data_ptr(), mb.data_ptr(), _stream()))
     return ti, ci, mb
-
-
-def mfma_probe_tflops(random_operands: bool, iters: int = 20000, reps: int = 3) -> float:
-    """TFLOP/s of a stream of nothing but bf16 32x32x16 MFMAs on every SIMD (mvpa_probe_mfma),
-    best of `reps` launches timed with events on the current stream."""
-    lib = load_library()
-    sink = torch.empty(512 * 256, dtype=torch.float32, device="cuda")
-    best = 0.0
-    for _ in range(reps + 1):                      # the first launch is a warm-up
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        _check(lib.mvpa_probe_mfma(1 if random_operands else 0, iters, sink.data_ptr(), _stream()))
-        e1.record()
-        torch.cuda.synchronize()
-        best = max(best, lib.mvpa_probe_mfma_flops(iters) / (e0.elapsed_time(e1) * 1e-3) / 1e12)
-    return best
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None,

@@ -25,10 +25,16 @@ Pinning status (what independent evidence fixes each function):
   mvpa_direct                : equality with rel_attn on every small configuration.
   attention_layer_forward    : composition of torch.nn.functional.linear and rel_attn;
                                pinned through rel_attn.
-  wavedec_db4_periodic       : PARITY UNPINNED - the reference delegates to ptwt/pywt
-                               (models/fftencoder.py:82-85), which are not installed; only
-                               the textbook properties of the db4 filter bank (orthogonality,
-                               perfect energy preservation, vanishing moments) are checked.
+  wavedec_db4_periodic       : the reference delegates to ptwt.wavedec (ptwt==0.1.9 with
+                               PyWavelets' db4 filters, models/fftencoder.py:62, 70-88), not
+                               installed here.  Its published algorithm - circular pad of
+                               (2*8-3)//2 = 6 samples left and 6 (+ n%2) right, one stride-2
+                               conv1d with the flipped decomposition filters per level,
+                               floor(log2(n/7)) levels, output [cA_L, cD_L .. cD_1] - is stated
+                               a second time with torch's pad and conv1d in tests/test_oracle.py
+                               and must agree for lengths 512, 2560 and odd lengths; the phase
+                               is spelled out on unit impulses; plus the textbook properties
+                               of the filter bank (orthogonality, energy, vanishing moments).
 """
 from __future__ import annotations
 
@@ -360,7 +366,7 @@ def mvpa_bruteforce(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale=None, window=
 
 
 # --------------------------------------------------------------------------------------
-# segment encoder (models/fftencoder.py:49-106) - DWT part is PARITY UNPINNED
+# segment encoder (models/fftencoder.py:49-106)
 # --------------------------------------------------------------------------------------
 
 DB4_DEC_LO = [

@@ -90,7 +90,7 @@ def test_add3():
     assert torch.equal(y, (a.float() + b.float() + c.float()).bfloat16())
 
 
-@pytest.mark.parametrize("L", [512, 2560, 100])
+@pytest.mark.parametrize("L", [512, 2560, 100, 333, 12000])     # 12000: more than 64 KiB of LDS per row pair
 def test_wavedec_db4(L):
     g = torch.Generator().manual_seed(L)
     x = torch.randn(9, L, generator=g)
@@ -98,15 +98,6 @@ def test_wavedec_db4(L):
     ref = O.wavedec_db4_periodic(x)
     assert y.shape == ref.shape
     assert (y - ref).abs().max().item() <= 2e-5
-
-
-def test_mfma_probe_runs_and_reads_plausibly():
-    """The measurement aid behind bench.py --mfma-probe: a pure MFMA stream reaches a large part of
-    the published 2500 TFLOP/s on smooth operands, and no more than that on random ones."""
-    smooth = mvpa_hip.mfma_probe_tflops(False, iters=4000, reps=2)
-    rand = mvpa_hip.mfma_probe_tflops(True, iters=4000, reps=2)
-    assert 800.0 < smooth < 2700.0, smooth
-    assert 500.0 < rand <= smooth * 1.05, (rand, smooth)
 
 
 def test_ring_append_writes_the_slot_the_device_counter_names():

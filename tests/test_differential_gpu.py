@@ -77,3 +77,46 @@ def test_mfma_paths_match_fp32_kernels(case):
             ref_norm = torch.maximum(ref_norm, (g32[4] * live).norm())
         rel = ((a - b).norm() / ref_norm.clamp_min(1e-20)).item()
         assert rel <= 2e-2, (name, rel)
+
+
+def _forward_cases(n=20, seed=777):
+    rng = random.Random(seed)
+    out = []
+    for it in range(n):
+        hkv, grp = rng.choice([1, 2]), rng.choice([1, 2, 3])
+        out.append(dict(
+            B=rng.choice([1, 2]), Dh=rng.choice([32, 128]),
+            C=rng.choice([8, 20, 32, 33, 48, 64, 65, 80, 100, 117, 128]),
+            T=rng.choice([2, 12, 13, 24, 33, 47, 64, 70]),
+            H=hkv * grp, Hkv=hkv, window=rng.choice([0, 2, 10, 10, 10]),
+            absent=rng.random() < 0.4, seed=1000 + it))
+    return out
+
+
+@pytest.mark.parametrize("case", _forward_cases(), ids=lambda c: "D{Dh}B{B}C{C}T{T}H{H}g{Hkv}w{window}{a}".format(
+    a="v" if c["absent"] else "", **c))
+def test_mfma_forward_matches_fp32_kernel_at_other_head_sizes(case):
+    """Head sizes 32 and 128 (every build of the matrix-core forward the dispatcher can pick for
+    them, far steps included) against the fp32 kernel: output max-abs <= 2e-2, log-sum-exp 2e-2."""
+    import mvpa_hip
+    B, C, T, H, Hkv, Dh = (case[k] for k in ("B", "C", "T", "H", "Hkv", "Dh"))
+    inp = make_mvpa_inputs(B=B, C=C, T=T, H=H, Hkv=Hkv, Dh=Dh, seed=case["seed"],
+                           qkv_unit=True, table_std=0.2).round_to(torch.bfloat16)
+    valid = None
+    if case["absent"]:
+        rng = random.Random(case["seed"])
+        valid = torch.ones(B, C, dtype=torch.bool)
+        for b in range(B):
+            valid[b, rng.sample(range(C), k=max(1, C // 5))] = False
+        valid = valid.cuda()
+    d16, d32 = inp.to("cuda", torch.bfloat16), inp.to("cuda", torch.float32)
+    kw = dict(window=case["window"], chan_valid=valid, return_lse=True)
+    o16, l16 = mvpa_hip.mvpa_forward(d16.q, d16.k, d16.v, d16.u, d16.vb, d16.z, d16.k_time, d16.k_chan,
+                                     kernel=mvpa_hip.KERNEL_MFMA, **kw)
+    o32, l32 = mvpa_hip.mvpa_forward(d32.q, d32.k, d32.v, d32.u, d32.vb, d32.z, d32.k_time, d32.k_chan, **kw)
+    live = torch.ones(B, 1, T, C, dtype=torch.bool, device="cuda") if valid is None \
+        else valid[:, None, None, :].expand(B, 1, T, C)
+    live = live.reshape(B, 1, T * C, 1)
+    assert torch.isfinite(o16.float()).all()
+    assert ((o16.float() - o32) * live).abs().max().item() <= 2e-2
+    assert ((l16 - l32) * live[..., 0]).abs().max().item() <= 2e-2

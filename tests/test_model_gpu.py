@@ -115,6 +115,56 @@ def test_mvpformer_forward_matches_oracle():
     assert score.shape == (2, 5, 8) and torch.isfinite(score).all()
 
 
+def test_mvpformer_s_dims_match_oracle_stack():
+    """MVPFormer-S as shipped (configs/mvpformer_s_generative.yaml:49-71: E768 L12 H12 Hkv4 Dh64
+    n_inner 1728, LoRA adapters on and made non-zero), B1 C64 T16 segments of 512 samples: all
+    twelve blocks in bf16 on the GPU against the fp32 oracle stack on the same parameters."""
+    from models.configs import MVPFORMER_S
+    from models.fftencoder import WaveEncoder
+    from models.mvpformer import HMVPFormer, MVPFormerConfig, MVPFormerHead
+    torch.manual_seed(4)
+    cfg = MVPFormerConfig(**MVPFORMER_S)
+    model = HMVPFormer(cfg, WaveEncoder(512, cfg.n_embd), MVPFormerHead(cfg.n_embd, cfg.n_embd)).to(torch.bfloat16).eval()
+    for name, p in model.named_parameters():
+        if "lora_B" in name:
+            p.data.normal_(0, 0.02)
+        elif "attn" in name or "embedding" in name:
+            p.data.mul_(2.0)
+    x = make_ieeg(1, 64, 16, 512, seed=11)
+    params = {k: v.float() for k, v in model.state_dict().items()}
+    for i, blk in enumerate(model.mvpformer.h):                   # the oracle takes merged weights
+        for lin in ("q_attn", "c_attn"):
+            params[f"mvpformer.h.{i}.attn.{lin}.weight"] = getattr(blk.attn, lin).effective_weight().detach().float()
+    ref, ref_emb = O.mvpformer_forward(x, params, dict(n_layer=12, n_head=12, n_head_kv=4))
+    out, emb = model.cuda()._common_forward(x.cuda())
+    rel_e = ((emb.float().cpu() - ref_emb).norm() / ref_emb.norm()).item()
+    rel_o = ((out.float().cpu() - ref).norm() / ref.norm()).item()
+    print(f"MVPFormer-S dims, 12 blocks: rel-L2 embeddings {rel_e:.3e}, output {rel_o:.3e}")
+    assert rel_e <= 1e-2, rel_e
+    assert rel_o <= 3e-2, rel_o
+
+
+def test_mvpformer_s_full_size_properties():
+    """The benchmark's MVPFormer-S window (B4 C64 T64 segments of 512 samples) at full size,
+    through properties that need no oracle: finite scores, and time-causality of the whole stack,
+    bit for bit - changing the last k segments leaves the hidden states of every earlier segment
+    untouched."""
+    from models.bench_model import build_mvpformer_s
+    model = build_mvpformer_s(512)
+    x = make_ieeg(4, 64, 64, 512, seed=0).cuda()
+    out, _ = model._common_forward(x)
+    assert out.shape == (4, 64, 64, 768) and torch.isfinite(out.float()).all()
+    score = model.predict_next_segment(x)
+    assert score.shape == (4, 63, 64) and torch.isfinite(score).all()
+    x2 = x.clone()
+    x2[:, -9:] = x2[:, -9:].flip(-1) * 1.5
+    out2, _ = model._common_forward(x2)
+    # the last time step keeps the content term for every key, earlier steps only inside the
+    # window, but no step ever sees a later one
+    assert torch.equal(out2[:, :-9], out[:, :-9])
+    assert not torch.equal(out2[:, -9:], out[:, -9:])
+
+
 def test_base_classification_bf16_then_fp8():
     """Base-size dims (E2048 H16 Hkv8 Dh128 n_inner5632, C=128) cut to two layers and 12 segments:
     binary-head logits in bf16 and with fp8 QK^T against the fp32 oracle stack.  Tolerances are

@@ -176,6 +176,14 @@ MFMA_SHAPES = [
     dict(B=2, C=16, T=1, H=4, Dh=64),                              # a single time step
     dict(B=4, C=64, T=9, H=4, Dh=64),                              # two (b,h) per XCD: merged tail order
     dict(B=2, C=48, T=11, H=8, Dh=64, Hkv=2),                      # window just vacuous, GQA 4:1
+    # far steps (T > 11) on every build of the kernel the dispatcher can pick
+    dict(B=1, C=128, T=26, H=2, Dh=128, Hkv=1),                    # <128,4,4,2>: the base model's attention shape, GQA 2:1
+    dict(B=1, C=100, T=24, H=4, Dh=128, Hkv=2, validity=True),     # <128,4,4,2>, ragged channels, absent channels
+    dict(B=1, C=64, T=30, H=2, Dh=128, Hkv=1),                     # <128,2,4,3>
+    dict(B=1, C=48, T=26, H=2, Dh=32),                             # <32,2,8,4>
+    dict(B=1, C=100, T=24, H=2, Dh=32, validity=True),             # <32,4,4,4>
+    dict(B=1, C=64, T=64, H=3, Dh=64, Hkv=1),                      # MVPFormer-S's attention shape: GQA 3:1, two slabs
+    dict(B=1, C=128, T=45, H=2, Dh=128, Hkv=1, validity=True),     # <128,4,4,2> across two 32-step slabs
 ]
 
 
@@ -248,6 +256,170 @@ def test_bf16_mfma_masks_exact_under_perturbation():
     out = run(p)
     same = (out == base).flatten(0, 1).all(-1).view(-1, T, C).all(0).all(-1).cpu()
     assert same.tolist() == [not (t <= 10 or t == T - 1) for t in range(T)]
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(B=2, C=117, T=30, H=2, Dh=64),                            # keys in two parts (KH = 2), far steps
+    dict(B=2, C=128, T=14, H=4, Dh=64, Hkv=2),
+    dict(B=2, C=128, T=26, H=2, Dh=128, Hkv=1),                    # one wave on all four key tiles
+])
+def test_bf16_mfma_whole_key_part_absent(cfg):
+    """Every channel from 64 up absent in one sample (a subject with 64 electrodes padded into a
+    wider batch): the waves that own the second half of the keys see no valid key at all and must
+    contribute exactly nothing - finite output, equal to the oracle."""
+    inp = make_mvpa_inputs(seed=33, table_std=0.3, qkv_unit=True, **cfg).round_to(torch.bfloat16)
+    valid = torch.ones(cfg["B"], cfg["C"], dtype=torch.bool)
+    valid[0, 64:] = False
+    valid[1, :64] = False                                          # and the first half, in the other sample
+    valid[1, 70] = True
+    inp.chan_valid = valid
+    out, lse = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA, return_lse=True)
+    live = valid[:, None, None, :].expand(-1, 1, cfg["T"], -1).reshape(cfg["B"], 1, -1, 1)
+    assert torch.isfinite(out.float().cpu()[live.expand_as(out)]).all()
+    ref, ref_lse = _oracle(inp, return_lse=True)
+    _check_bf16(out.float().cpu() * live, ref * live)
+    assert ((lse.cpu().double() - ref_lse) * live[..., 0]).abs().max().item() <= 3e-2
+
+
+@pytest.mark.parametrize("cfg,n,ring", [
+    (dict(B=1, C=117, T=24, H=2, Hkv=2, Dh=64), 3, False),
+    (dict(B=1, C=128, T=40, H=2, Hkv=1, Dh=128), 5, False),        # the 8-wave key-run build at Dh 128
+    (dict(B=1, C=128, T=40, H=2, Hkv=1, Dh=128), 5, True),
+])
+def test_last_step_whole_key_part_absent(cfg, n, ring):
+    """The same for a decoding step cut into key runs (and on a ring of slots): against the oracle's
+    last time step."""
+    inp = make_mvpa_inputs(seed=35, table_std=0.3, qkv_unit=True, **cfg).round_to(torch.bfloat16)
+    B, C, T, Hkv, Dh = cfg["B"], cfg["C"], cfg["T"], cfg["Hkv"], cfg["Dh"]
+    valid = torch.ones(B, C, dtype=torch.bool)
+    valid[0, 64:] = False
+    inp.chan_valid = valid
+    ref = _oracle(inp)[:, :, -C:].float()
+    d = inp.to("cuda", torch.bfloat16)
+    k, v, head_t = d.k, d.v, None
+    if ring:
+        head = 17
+        slot = torch.arange(T, device="cuda")
+        step_of_slot = T - 1 - (head - slot) % T
+        k = d.k.view(B, Hkv, T, C, Dh)[:, :, step_of_slot].reshape(B, Hkv, T * C, Dh).contiguous()
+        v = d.v.view(B, Hkv, T, C, Dh)[:, :, step_of_slot].reshape(B, Hkv, T * C, Dh).contiguous()
+        head_t = torch.tensor([head], dtype=torch.int32, device="cuda")
+    got = mvpa_hip.mvpa_forward(d.q[:, :, -C:], k, v, d.u, d.vb, d.z, d.k_time, d.k_chan,
+                                chan_valid=d.chan_valid, last_step_only=True, key_splits=n,
+                                ring_head=head_t).float().cpu()
+    live = valid[:, None, :, None]
+    assert torch.isfinite(got[live.expand_as(got)]).all()
+    _check_bf16(got * live, ref * live)
+
+
+# ------------------------------------------------------------------------------------------
+# gathers of the matrix-core kernel itself, on index-revealing inputs
+# ------------------------------------------------------------------------------------------
+# q = 0 and u = 0 switch the content term off.  One bias vector is a unit vector and ONE row j* of
+# its table holds a large value in that coordinate, so the soft-max puts all its weight on the
+# keys whose gathered row is j* (every other key is down by e^-64).  V codes the key's channel
+# (or time step) one-hot, so the output names the keys that got the weight: the expected output is
+# written down from the closed forms C-1-|cq-ck| and T-1-(tq-tk) (layers/mvpa.py:127-159) and an
+# index that is off by one anywhere in the kernel moves ones to other columns.  Head g tests row
+# j* = rows[g] (the tables are per kv head).
+
+GATHER_SHAPES = [
+    dict(C=64, T=40, Dh=64),        # <64,2,4,4>: split last step, far steps, two slabs
+    dict(C=117, T=14, Dh=64),       # keys in two parts
+    dict(C=128, T=40, Dh=128),      # one wave on four key tiles
+    dict(C=48, T=40, Dh=32),
+    dict(C=20, T=70, Dh=64),        # 8 time steps per workgroup, three slabs
+    dict(C=100, T=36, Dh=32),
+]
+PEAK = 64.0
+
+
+def _gather_case(C, T, Dh, rows, axis):
+    """Inputs (fp32, exactly representable in bf16) whose output reveals the gathered row."""
+    H = len(rows)
+    N = T * C
+    q = torch.zeros(1, H, N, Dh)
+    k = torch.zeros(1, H, N, Dh)
+    zero = torch.zeros(H, Dh)
+    unit = torch.zeros(H, Dh)
+    unit[:, 0] = 1.0
+    k_time, k_chan = torch.zeros(H, T, Dh), torch.zeros(H, C, Dh)
+    tab = k_chan if axis == "chan" else k_time
+    for g, j in enumerate(rows):
+        tab[g, j, 0] = PEAK
+    n = torch.arange(N)
+    code = (n % C) if axis == "chan" else (n // C)
+    v = torch.zeros(1, H, N, Dh)
+    v[0, :, n, code % Dh] = 1.0
+    return q, k, v, zero, unit, k_time, k_chan
+
+
+@pytest.mark.parametrize("cfg", GATHER_SHAPES, ids=lambda c: "C{C}T{T}D{Dh}".format(**c))
+def test_mfma_channel_gather_is_exact(cfg):
+    C, T, Dh = cfg["C"], cfg["T"], cfg["Dh"]
+    cq, ck = torch.arange(C)[:, None], torch.arange(C)[None, :]
+    onehot = torch.zeros(C, Dh)
+    onehot[torch.arange(C), torch.arange(C) % Dh] = 1.0
+    for r0 in range(0, C, 16):
+        rows = list(range(r0, min(C, r0 + 16)))
+        q, k, v, zero, unit, k_time, k_chan = _gather_case(C, T, Dh, rows, "chan")
+        out = mvpa_hip.mvpa_forward(*(t.cuda().bfloat16() for t in (q, k, v, zero, zero, unit, k_time, k_chan)),
+                                    sm_scale=1.0, kernel=mvpa_hip.KERNEL_MFMA).float().cpu()
+        for g, j in enumerate(rows):
+            hit = (C - 1 - (cq - ck).abs()) == j                  # keys whose gathered row is j*
+            w = torch.where(hit.any(1, keepdim=True), hit, torch.ones_like(hit)).float()
+            want = (w / w.sum(1, keepdim=True)) @ onehot          # [C, Dh], the same for every tq
+            got = out[0, g].view(T, C, Dh)
+            assert (got - want[None]).abs().max().item() <= 1e-2, (j, (got - want[None]).abs().max().item())
+
+
+@pytest.mark.parametrize("cfg", GATHER_SHAPES, ids=lambda c: "C{C}T{T}D{Dh}".format(**c))
+def test_mfma_time_gather_is_exact(cfg):
+    C, T, Dh = cfg["C"], cfg["T"], cfg["Dh"]
+    for r0 in range(0, T, 16):
+        rows = list(range(r0, min(T, r0 + 16)))
+        q, k, v, zero, unit, k_time, k_chan = _gather_case(C, T, Dh, rows, "time")
+        out = mvpa_hip.mvpa_forward(*(t.cuda().bfloat16() for t in (q, k, v, zero, unit, zero, k_time, k_chan)),
+                                    sm_scale=1.0, kernel=mvpa_hip.KERNEL_MFMA).float().cpu()
+        for g, j in enumerate(rows):
+            got = out[0, g].view(T, C, Dh)
+            for tq in range(T):
+                tk = tq - (T - 1 - j)                             # the key step whose gathered row is j*
+                want = torch.zeros(Dh)
+                if tk >= 0:
+                    want[tk % Dh] = 1.0
+                else:                                             # row j* out of reach: uniform over tk <= tq
+                    for t in range(tq + 1):
+                        want[t % Dh] += 1.0 / (tq + 1)
+                err = (got[tq] - want[None]).abs().max().item()
+                assert err <= 1e-2, (j, tq, err)
+
+
+@pytest.mark.parametrize("cfg,n,head", [
+    (dict(C=64, T=40, Dh=64), 4, 13),
+    (dict(C=128, T=70, Dh=128), 5, 33),        # runs longer than a slab, the ring wraps inside a run
+    (dict(C=20, T=45, Dh=32), 1, 44),
+])
+def test_mfma_time_gather_on_a_ring_is_exact(cfg, n, head):
+    """Decoding step on a ring of slots: the table row of slot s is (s - head - 1) mod T, read per
+    slab inside the kernel.  The step that holds row j* must get the weight wherever the ring
+    stands."""
+    C, T, Dh = cfg["C"], cfg["T"], cfg["Dh"]
+    slot = torch.arange(T)
+    step_of_slot = T - 1 - (head - slot) % T
+    head_t = torch.tensor([head], dtype=torch.int32, device="cuda")
+    for r0 in range(0, T, 16):
+        rows = list(range(r0, min(T, r0 + 16)))
+        H = len(rows)
+        q, k, v, zero, unit, k_time, k_chan = _gather_case(C, T, Dh, rows, "time")
+        v_ring = v.view(1, H, T, C, Dh)[:, :, step_of_slot].reshape(1, H, T * C, Dh)
+        args = [t.cuda().bfloat16() for t in (q[:, :, -C:], k, v_ring, zero, unit, zero, k_time, k_chan)]
+        out = mvpa_hip.mvpa_forward(*args, sm_scale=1.0, last_step_only=True, key_splits=n,
+                                    ring_head=head_t).float().cpu()
+        for g, j in enumerate(rows):
+            want = torch.zeros(Dh)
+            want[j % Dh] = 1.0                                    # tq = T-1: row j* belongs to key step j*
+            assert (out[0, g] - want[None]).abs().max().item() <= 1e-2, j
 
 
 def test_bf16_mfma_strided_layout_and_auto_dispatch():
@@ -489,3 +661,37 @@ def test_decoding_step_at_base_model_size_matches_the_full_forward():
                                     ring_head=torch.tensor([head], dtype=torch.int32, device="cuda"))
     assert (ring.float() - ref).abs().max().item() <= 2e-2
     assert ((ring.float() - ref).norm() / ref.norm()).item() <= 5e-3
+
+
+def test_bf16_base_attention_shape_full_size():
+    """The base model's attention at full length (B1 H16 Hkv8 C128 T512 Dh128, the kernel build
+    with one wave on four key tiles): sampled query rows of one head against the oracle - the
+    first steps, a step whose keys are mostly far, the last step - and masks through bit-exact
+    perturbation, as for the irregular-channel configuration."""
+    C, T = 128, 512
+    inp = make_mvpa_inputs(B=1, C=C, T=T, H=16, Hkv=8, Dh=128, seed=0, qkv_unit=True,
+                           validity=True).round_to(torch.bfloat16)
+    d = inp.to("cuda", torch.bfloat16)
+    out = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
+                                chan_valid=d.chan_valid, kernel=mvpa_hip.KERNEL_MFMA)
+    ranges = [(0, 2 * C), (300 * C, 301 * C), (511 * C, 512 * C)]
+    ref = _oracle(inp, dtype=torch.float32, heads=[(0, 11)], q_ranges=ranges, q_block=128)
+    live = inp.chan_valid[0][:, None]
+    for (r0, r1) in ranges:
+        got = out[0, 11, r0:r1].float().cpu().view(-1, C, 128) * live
+        _check_bf16(got, ref[0, 11, r0:r1].view(-1, C, 128) * live)
+    dead = (~d.chan_valid)[:, None, None, :, None]
+    seven = torch.tensor(7.0, dtype=torch.bfloat16, device="cuda")
+    big = torch.tensor(-3.0e4, dtype=torch.bfloat16, device="cuda")
+    k2 = torch.where(dead, seven, d.k.view(1, 8, T, C, 128)).view(1, 8, T * C, 128).clone()
+    v2 = torch.where(dead, big, d.v.view(1, 8, T, C, 128)).view(1, 8, T * C, 128).clone()
+    k2[:, :, -40 * C:] *= -1.5                        # the last 40 steps: hidden from every earlier row
+    v2[:, :, -40 * C:] += 1.0
+    o2 = mvpa_hip.mvpa_forward(d.q, k2, v2, d.u, d.vb, d.z, d.k_time, d.k_chan, chan_valid=d.chan_valid)
+    assert torch.equal(o2[:, :, :-40 * C], out[:, :, :-40 * C])
+    # keys of step 0 changed: only rows with tq <= 10 and the last step keep the content term there
+    k3 = d.k.clone()
+    k3[:, :, :C] += 1.0
+    o3 = mvpa_hip.mvpa_forward(d.q, k3, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, chan_valid=d.chan_valid)
+    same = (o3 == out).flatten(0, 1).all(-1).view(-1, T, C).all(0).all(-1).cpu()
+    assert same.tolist() == [not (t <= 10 or t == T - 1) for t in range(T)]

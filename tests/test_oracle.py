@@ -190,6 +190,74 @@ def test_db4_filter_bank_properties():
     assert torch.allclose(energy, (x ** 2).sum(-1))
 
 
+def _wavedec_pad_conv(x):
+    """Second, independent statement of what the reference's encoder asks its wavelet library for
+    (models/fftencoder.py:80-88: ptwt.wavedec(x, db4, mode="periodic"), outputs concatenated).
+    The library's published algorithm, level by level: pad the signal circularly by
+    (2*8 - 3) // 2 = 6 samples on the left and 6 (+1 if the length is odd) on the right, then one
+    stride-2 conv1d (cross-correlation) with the FLIPPED decomposition filters [dec_lo, dec_hi];
+    the approximation goes on to the next level, floor(log2(n / 7)) levels in all; the result is
+    [cA_L, cD_L, ..., cD_1].  Written with torch's pad and conv1d, not with the index formula the
+    oracle uses."""
+    F = torch.nn.functional
+    lo = torch.tensor(O.DB4_DEC_LO, dtype=x.dtype).flip(0)
+    hi = torch.tensor(O.DB4_DEC_HI, dtype=x.dtype).flip(0)
+    filt = torch.stack([lo, hi])[:, None, :]                  # [2, 1, 8]
+    a = x[:, None, :]
+    details = []
+    levels = int(math.floor(math.log2(x.shape[-1] / 7)))
+    for _ in range(levels):
+        n = a.shape[-1]
+        padded = F.pad(a, (6, 6 + n % 2), mode="circular")
+        res = F.conv1d(padded, filt, stride=2)                # [M, 2, floor((n + 7) / 2)]
+        a, d = res[:, :1], res[:, 1]
+        details.append(d)
+    return torch.cat([a[:, 0]] + details[::-1], dim=-1)
+
+
+@pytest.mark.parametrize("L", [512, 2560, 97, 333, 1001])
+def test_wavedec_matches_pad_and_conv1d_statement(L):
+    """Pins wavedec_db4_periodic: equal to the pad + strided-conv1d statement of the wavelet
+    library's algorithm for the shipped segment lengths (512 in the benchmark configurations, 2560
+    in the YAMLs) and for odd lengths, where the right pad grows by one; sizes as
+    models/fftencoder.py:70-78 computes them."""
+    x = torch.randn(5, L, dtype=torch.float64, generator=torch.Generator().manual_seed(L))
+    want = _wavedec_pad_conv(x)
+    got = O.wavedec_db4_periodic(x.float())
+    assert got.shape == want.shape and got.shape[-1] == sum(O.dwt_sizes(L))
+    assert (got.double() - want).abs().max().item() <= 2e-5
+    # one level, float64 against float64: the same numbers to rounding of the summation order
+    a, d = O.dwt_level_periodic(x)
+    F = torch.nn.functional
+    padded = F.pad(x[:, None], (6, 6 + L % 2), mode="circular")
+    lo = torch.tensor(O.DB4_DEC_LO, dtype=torch.float64).flip(0)[None, None]
+    hi = torch.tensor(O.DB4_DEC_HI, dtype=torch.float64).flip(0)[None, None]
+    assert torch.allclose(a, F.conv1d(padded, lo, stride=2)[:, 0], atol=1e-13)
+    assert torch.allclose(d, F.conv1d(padded, hi, stride=2)[:, 0], atol=1e-13)
+
+
+def test_wavedec_phase_on_unit_impulses():
+    """The phase (alignment) convention, spelled out on unit impulses by hand from the pad + conv1d
+    definition: with 6 samples of left pad and the flipped filter, output k of a level reads the
+    padded samples 2k .. 2k+7, i.e. signal samples 2k-6 .. 2k+1, against dec_lo[7] .. dec_lo[0].
+    An impulse at sample p therefore puts dec_lo[2k+1-p] into approximation coefficient k."""
+    lo, hi = O.DB4_DEC_LO, O.DB4_DEC_HI
+    n = 16                                        # one level at this length (floor(log2(16/7)) = 1)
+    for p, taps in ((0, {0: 1, 1: 3, 2: 5, 3: 7, 8: 1, 9: 3, 10: 5}),       # k: index into dec_lo
+                    (5, {2: 0, 3: 2, 4: 4, 5: 6, 10: 0}),
+                    (15, {0: 2, 1: 4, 2: 6, 7: 0, 8: 2, 9: 4, 10: 6})):
+        x = torch.zeros(1, n)
+        x[0, p] = 1.0
+        out = O.wavedec_db4_periodic(x)[0]
+        m = (n + 7) // 2
+        assert out.shape[0] == 2 * m
+        for k in range(m):
+            want_a = lo[taps[k]] if k in taps else 0.0
+            want_d = hi[taps[k]] if k in taps else 0.0
+            assert abs(out[k].item() - want_a) < 1e-7, (p, k)
+            assert abs(out[m + k].item() - want_d) < 1e-7, (p, k)
+
+
 def test_golden_c1_fixture():
     """Oracle and input generator against the committed vector (tests/golden/c1_seed0.npz)."""
     import os
