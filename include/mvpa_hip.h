@@ -33,8 +33,10 @@ enum {
   MVPA_ERR_UNSUPPORTED = -8,   /* valid request that the selected kernel cannot serve    */
   MVPA_ERR_STRUCT = -9,        /* struct_size does not match this library                */
   MVPA_ERR_LAUNCH = -10,       /* hipLaunchKernel reported an error                      */
-  MVPA_ERR_NONCAUSAL_BIAS = -11 /* relative biases need the time-causal mask
+  MVPA_ERR_NONCAUSAL_BIAS = -11, /* relative biases need the time-causal mask
                                    (attentions/attn.py:1335-1336)                        */
+  MVPA_ERR_WS_SIZE = -12        /* the request needs more workspace than the library's
+                                   built-in array holds (MVPA_STATIC_WS_BYTES)           */
 };
 
 /* ---- element types ----------------------------------------------------------------- */
@@ -143,6 +145,24 @@ size_t mvpa_split_ws_bytes(const mvpa_fwd_args* args);
 /* Fused forward; replaces attentions/attn.py:1064-1123 + 1305-1314 and
  * layers/mvpa.py:173-278.  Validates, then enqueues on `stream`. */
 int mvpa_forward(const mvpa_fwd_args* args, void* stream);
+
+/*
+ * The split decoding step of mvpa_forward (MVPA_FLAG_LAST_STEP, n_split > 1, bf16 matrix-core
+ * kernel) on a workspace inside the library instead of args->split_ws, which is ignored.  No
+ * counterpart in the reference: it is for callers that cannot allocate device memory - code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The entry point
+ * allocates nothing and frees nothing; q, k, v, o (and lse) are still the caller's.  Same kernels,
+ * same results as mvpa_forward with a caller workspace, bit for bit.
+ *
+ * The workspace is a device array of MVPA_STATIC_WS_BYTES that every GPU the library runs on
+ * holds until the process ends.  Requests with mvpa_split_ws_bytes(args) above that return
+ * MVPA_ERR_WS_SIZE (take fewer runs, or use mvpa_forward with a workspace of your own).  All calls
+ * on one GPU share the array: calls that overlap in time on one GPU (different streams, different
+ * threads) race on it and must be ordered by the caller; calls on different GPUs do not interact.
+ */
+#define MVPA_STATIC_WS_BYTES (16u << 20)
+int mvpa_forward_last_step_static(const mvpa_fwd_args* args, void* stream);
+size_t mvpa_static_ws_bytes(void);
 
 /* ---- backward ------------------------------------------------------------------------------
  * Argument block of mvpa_backward: the boundary of FlashMVPA.backward

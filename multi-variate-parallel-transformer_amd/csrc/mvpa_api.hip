@@ -19,6 +19,7 @@ extern "C" const char* mvpa_error_string(int status) {
     case MVPA_ERR_STRUCT: return "argument struct size does not match the library";
     case MVPA_ERR_LAUNCH: return "kernel launch failed";
     case MVPA_ERR_NONCAUSAL_BIAS: return "relative biases require the time-causal mask";
+    case MVPA_ERR_WS_SIZE: return "request needs more workspace than the library's built-in array holds";
   }
   return "unknown status";
 }

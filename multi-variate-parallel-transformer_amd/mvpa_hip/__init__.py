@@ -102,6 +102,10 @@ def load_library() -> ctypes.CDLL:
     lib.mvpa_split_ws_bytes.argtypes = [ctypes.POINTER(MvpaFwdArgs)]
     lib.mvpa_forward.restype = ctypes.c_int
     lib.mvpa_forward.argtypes = [ctypes.POINTER(MvpaFwdArgs), vp]
+    lib.mvpa_forward_last_step_static.restype = ctypes.c_int
+    lib.mvpa_forward_last_step_static.argtypes = [ctypes.POINTER(MvpaFwdArgs), vp]
+    lib.mvpa_static_ws_bytes.restype = ctypes.c_size_t
+    lib.mvpa_static_ws_bytes.argtypes = []
     lib.mvpa_backward.restype = ctypes.c_int
     lib.mvpa_backward.argtypes = [ctypes.POINTER(MvpaBwdArgs), vp]
     lib.mvpa_debug_maps.restype = ctypes.c_int
@@ -216,7 +220,8 @@ def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float]
                  key_bias: Optional[torch.Tensor] = None, return_lse: bool = False,
                  kernel: int = KERNEL_AUTO, out: Optional[torch.Tensor] = None,
                  fp8_qk: bool = False, last_step_only: bool = False,
-                 key_splits: Optional[int] = None, ring_head: Optional[torch.Tensor] = None):
+                 key_splits: Optional[int] = None, ring_head: Optional[torch.Tensor] = None,
+                 static_ws: bool = False):
     """Fused MVPA forward on the GPU.
 
     q [B,H,N,Dh]; k, v [B,Hkv,N,Dh]; u, vb, z [Hkv,Dh]; k_time [Hkv,T,Dh]; k_chan [Hkv,C,Dh];
@@ -232,6 +237,9 @@ def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float]
     k and v are then the slots of a ring, slot ring_head holding the newest step and slot s the one
     (ring_head - s) mod T steps older.  The kernel reads it from device memory, so a captured
     graph of the call follows a cache that moves on.
+    static_ws (with last_step_only and more than one key run): the runs' partial results go through
+    the workspace built into the library (mvpa_forward_last_step_static) instead of one allocated
+    here; with `out` given the call then allocates no device memory at all.
     """
     lib = load_library()
     _need_cuda(q, k, v, u, vb, z, k_time, k_chan, chan_valid, key_bias)
@@ -280,8 +288,13 @@ def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float]
         n = default_key_splits(B, H, T) if key_splits is None else int(key_splits)
         if n > 1:
             a.n_split = n
+            if static_ws:
+                _check(lib.mvpa_forward_last_step_static(ctypes.byref(a), _stream()))
+                return (out, lse) if return_lse else out
             ws = torch.empty(lib.mvpa_split_ws_bytes(ctypes.byref(a)), dtype=torch.uint8, device=q.device)
             a.split_ws = ws.data_ptr()
+    if static_ws:
+        raise ValueError("static_ws needs last_step_only on the bf16 matrix-core kernel with more than one key run")
     _check(lib.mvpa_forward(ctypes.byref(a), _stream()))
     return (out, lse) if return_lse else out
 
