@@ -273,7 +273,7 @@ class HMVPFormer(BrainModel):
     its `base_model` / `head_model` state dicts load key for key."""
 
     def __init__(self, gpt_config: MVPFormerConfig, encoder: BrainEncoder, head: BrainDecider,
-                 flash: bool = True) -> None:
+                 flash: bool = True, base_model: str = "", head_model: str = "") -> None:
         super().__init__()
         self.gpt_config = gpt_config
         self.mvpformer = MVPFormerModel(gpt_config, flash=flash)
@@ -281,6 +281,24 @@ class HMVPFormer(BrainModel):
         self.encoder = encoder
         self.seizure_embeddings = nn.Parameter(
             torch.normal(mean=0, std=1.0 / encoder.size_input, size=(3, encoder.size_input)))
+        self.base_model = base_model
+        if base_model != "" or head_model != "":                   # models/mvpformer.py:470-479
+            self._load_checkpoint(_load_weights(base_model), _load_weights(head_model))
+
+    def _load_checkpoint(self, base_weights, head_weights):
+        """models/mvpformer.py:481-485: the base state dict must match key for key (strict); the
+        encoder's norm weight is reset to ones, as there."""
+        if base_weights is not None:
+            base_weights = dict(base_weights)
+            base_weights["encoder.ln.weight"] = torch.ones_like(self.encoder.ln.weight)
+            self.load_state_dict(base_weights, strict=True)
+
+    def load_reference_state_dicts(self, base_model_sd=None, head_model_sd=None):
+        """Load state dicts saved by the reference's modules (the `base_model` / `head_model` files of
+        models/mvpformer.py:470-479, already read with torch.load(..., weights_only=True)), under
+        this class's checkpoint policy.  Returns self."""
+        self._load_checkpoint(base_model_sd, head_model_sd)
+        return self
 
     @torch.no_grad()
     def _common_forward(self, batch: torch.Tensor, attention_mask=None):
@@ -296,11 +314,19 @@ class HMVPFormer(BrainModel):
         """Classification score of a stream, one segment at a time: segment [B, ch, len] is the
         newest one, `past` what the previous call returned (None at the start of a stream).
         Returns (logits, past).  Each call runs the encoder on the new segment only and one
-        decoding step of every block against the cached keys and values; as long as the stream is
-        no longer than max_steps (default: the number of position embeddings) every step sees what
-        the full forward over the segments so far sees when its position rows end at max_steps
-        (forward(position_end=max_steps)); at step max_steps that is classify() on the whole
-        window.  After that the oldest segment drops out of the attention window at every step."""
+        decoding step of every block against the cached keys and values.
+
+        What a stream computes: in this model the newest time step keeps the content term for
+        EVERY key while older steps only keep it inside the window of 10 (layers/mvpa.py:231-245).
+        A decoding step is always the newest step, so from the second block on the cached keys and
+        values of a step are the ones it produced as the newest step of its own, shorter, window.
+        For streams of at most 12 segments (the window never bites) or a single block this is
+        exactly the full forward over the segments so far with its position rows ending at
+        max_steps (forward(position_end=max_steps)), and at step max_steps classify() on the whole
+        window.  For longer streams with two or more blocks it is a different function of the
+        same segments - every step computed with full content attention at the time it arrived -
+        and the two differ by far more than rounding (tests/test_model_gpu.py measures it).  After
+        max_steps segments the oldest one drops out of the caches at every step."""
         bsz, ch, seg = segment.shape
         embeds = self.encoder(segment.reshape(bsz * ch, seg)).view(bsz, 1, ch, -1)
         if past is None:
@@ -389,8 +415,9 @@ class HMVPFormer(BrainModel):
         (similarity, prediction, past): `prediction` [B, ch, E] is the head's forecast of the NEXT
         segment's encoding, `similarity` [B, ch] the cosine similarity between this segment's
         encoding and the forecast the previous call made for it (None on the first call) - the
-        column of predict_next_segment's result that this segment closes.  `past` carries the
-        caches and the last forecast from call to call."""
+        column of predict_next_segment's result that this segment closes (equal to it for streams
+        of at most 12 segments or one block; see classify_step for longer ones).  `past` carries
+        the caches and the last forecast from call to call."""
         bsz, ch, seg = segment.shape
         embeds = self.encoder(segment.reshape(bsz * ch, seg)).view(bsz, 1, ch, -1)
         caches, forecast = (None, None) if past is None else past
@@ -411,3 +438,50 @@ class HMVPFormer(BrainModel):
         last segment's hidden state)."""
         out, _ = self._common_forward(batch)
         return self.head(out[:, -1].float().mean(dim=1).to(out.dtype))
+
+
+def _load_weights(path: str):
+    """torch.load(path, weights_only=True), None for an empty or missing path
+    (models/mvpformer.py:471-478)."""
+    if path == "":
+        return None
+    try:
+        return torch.load(path, weights_only=True, map_location="cpu")
+    except FileNotFoundError:
+        return None
+
+
+class ClassificationHMVPFormer(HMVPFormer):
+    """The classification harness's checkpoint policy (models/mvpformer.py:845-904) on the inference
+    model: a base state dict whose head has another shape loses that head; with adapters on, only
+    adapter, head and encoder.proj_* keys may be missing from it; the head state dict must bring
+    the head (and the adapters, with adapters on); `class_loss.weight` is the only key that may be
+    unknown."""
+
+    def _load_checkpoint(self, base_weights, head_weights):
+        lora = bool(self.gpt_config.lora)
+        if base_weights is not None:
+            base_weights = dict(base_weights)
+            if ("head.head.weight" in base_weights
+                    and base_weights["head.head.weight"].shape != self.head.head.weight.shape):
+                del base_weights["head.head.weight"]
+            miss_key, un_key = self.load_state_dict(base_weights, strict=False)
+            if lora:
+                miss_key = [k for k in miss_key
+                            if "lora" not in k.lower() and "head" not in k.lower()
+                            and "encoder.proj_" not in k.lower()]
+                if miss_key:
+                    raise AttributeError(
+                        f"Parameters {miss_key} are missing from the base model and are not trainable.")
+            elif miss_key:
+                raise AttributeError(f"Parameters {list(miss_key)} are missing from the base model.")
+            if len(un_key) > 0:
+                raise AttributeError(f"Parameters {list(un_key)} are unknown in the base model.")
+        if head_weights is not None:
+            miss_key, un_key = self.load_state_dict(dict(head_weights), strict=False)
+            needed = [k for k in miss_key
+                      if "head" in k.lower() or (lora and "lora" in k.lower())]
+            if needed:
+                raise AttributeError(f"Parameters {needed} are missing from the head model.")
+            if len(un_key) > 0 and list(un_key) != ["class_loss.weight"]:
+                raise AttributeError(f"Parameters {list(un_key)} are unknown in the model.")

@@ -253,6 +253,36 @@ def test_stream_of_segments_matches_full_forward():
     assert (logits.float() - ref.float()).abs().max().item() <= 3e-2 * (ref.float().abs().max().item() + 1e-3)
 
 
+def test_stream_differs_from_the_window_forward_once_the_window_bites():
+    """Streams longer than 12 segments: with ONE block a streamed step still equals the last step
+    of the full forward (a decoding step and the last row of the window both keep the content term
+    for every key); with two or more blocks it does not - the cached keys and values of older steps
+    were produced while those steps were the newest ones, with full content attention, whereas the
+    window forward zeroes their content term beyond 10 steps.  The deviation is measured here so
+    that the documentation's statement rests on a number."""
+    from models.mvpformer import HMVPFormer, MVPFormerConfig, MVPFormerHead
+    from models.fftencoder import WaveEncoder
+    B, T, C = 2, 24, 12
+    batch = torch.randn(B, T, C, 512, device="cuda", generator=torch.Generator("cuda").manual_seed(3))
+    dev = {}
+    for n_layer in (1, 3):
+        torch.manual_seed(21)
+        cfg = MVPFormerConfig(n_embd=256, n_head=4, n_head_kv=2, n_layer=n_layer, n_positions=T,
+                              n_channels=C, n_inner=512)
+        model = HMVPFormer(cfg, WaveEncoder(512, 256), MVPFormerHead(256, 2)).to("cuda", torch.bfloat16).eval()
+        for name, p in model.named_parameters():
+            if "attn" in name or "embedding" in name:
+                p.data.mul_(3.0)                 # content logits wide enough for the window to matter
+        past = None
+        for t in range(T):
+            logits, past = model.classify_step(batch[:, t], past)
+        ref = model.classify(batch)
+        dev[n_layer] = ((logits.float() - ref.float()).abs().max() / (ref.float().abs().max() + 1e-3)).item()
+    print(f"stream vs window forward at T=24: 1 block {dev[1]:.3e}, 3 blocks {dev[3]:.3e} (relative to the logit spread)")
+    assert dev[1] <= 3e-2
+    assert dev[3] > 3e-2          # not the same function: far outside bf16 rounding
+
+
 def test_stream_slides_past_the_window():
     """Past max_steps segments the oldest step leaves the caches; the buffers wrap without the
     live steps changing, and the result stays finite and close to the full forward over the last
