@@ -32,145 +32,9 @@
 // One workgroup = NW waves = NW query blocks = NW/NCT consecutive time steps; one barrier per
 // key tile.  Where registers allow, two 4-wave workgroups share a CU so that one computes while
 // the other sits at its barrier.
-#include "mvpa_common.h"
+#include "mvpa_mfma_tools.h"
 
 namespace mvpa {
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
-typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
-
-#define LDS_PTR(T) __attribute__((address_space(3))) T*
-#define GLOBAL_PTR(T) __attribute__((address_space(1))) T*
-
-__device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-#define kOnes2 (bf16x2{(__bf16)1.0f, (__bf16)1.0f})
-constexpr float kMFloor = -1.0e30f;     // "nothing seen yet" value of a running maximum
-
-// order LDS traffic between the lanes of ONE wave (no workgroup barrier needed)
-__device__ inline void wave_lds_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() would also drain every
-// outstanding global load (vmcnt 0), which would serialise the tile prefetch ring.
-__device__ inline void lds_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
-// One 64-lane x 16-byte direct-to-LDS load: lane L's 16 bytes land at lds_base + 16*L.  Issued as
-// inline assembly on purpose: the compiler then keeps no record of an LDS write in flight and
-// does not drain the whole prefetch ring (vmcnt 0) in front of every later LDS read; completion
-// is awaited explicitly with wait_vmcnt() before the barrier that publishes the tile.
-__device__ inline void load_to_lds_16(const void* gptr, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-               :: "v"(gptr), "s"(lds_base) : "memory", "m0");
-}
-
-template <int N>
-__device__ inline void wait_vmcnt_imm() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
-// wait until at most n of this wave's vector-memory operations are outstanding
-__device__ inline void wait_vmcnt(int n) {
-  switch (n) {
-    case 0: wait_vmcnt_imm<0>(); break;
-    case 1: wait_vmcnt_imm<1>(); break;
-    case 2: wait_vmcnt_imm<2>(); break;
-    case 3: wait_vmcnt_imm<3>(); break;
-    case 4: wait_vmcnt_imm<4>(); break;
-    case 5: wait_vmcnt_imm<5>(); break;
-    case 6: wait_vmcnt_imm<6>(); break;
-    case 7: wait_vmcnt_imm<7>(); break;
-    default: wait_vmcnt_imm<8>(); break;      // n >= 8: waiting for <= 8 is only stricter
-  }
-}
-
-// max over a lane and its partner in the other half-wave (lane ^ 32): one register swap between
-// the halves instead of a round trip through the LDS crossbar
-__device__ inline float xhalf_max(float x) {
-  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-
-// 8 bf16 (one 16-byte chunk of a q row) + bias, scaled, back to a bf16 MFMA fragment
-__device__ inline bf16x8 make_qfrag(u32x4 raw, const bf16_t* __restrict__ bias, float scale) {
-  const u32x4 braw = *(const u32x4*)bias;
-  bf16x8 out;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const uint32_t w = raw[i], bw = braw[i];
-    const float lo = (__uint_as_float(w << 16) + __uint_as_float(bw << 16)) * scale;
-    const float hi = (__uint_as_float(w & 0xffff0000u) + __uint_as_float(bw & 0xffff0000u)) * scale;
-    out[2 * i] = (__bf16)lo;
-    out[2 * i + 1] = (__bf16)hi;
-  }
-  return out;
-}
-
-// 8 floats -> 8 fp8 (e4m3) packed in 64 bits, the operand of the 32x32x16 fp8 MFMA
-__device__ inline long pack_fp8(const float (&f)[8]) {
-  int lo = 0, hi = 0;
-  lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
-  lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
-  hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], hi, false);
-  hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
-  return (long)(((unsigned long)(unsigned)hi << 32) | (unsigned)lo);
-}
-
-// (q + bias) * scale as an fp8 fragment
-__device__ inline long make_qfrag_fp8(u32x4 raw, const bf16_t* __restrict__ bias, float scale) {
-  const u32x4 braw = *(const u32x4*)bias;
-  float f[8];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const uint32_t w = raw[i], bw = braw[i];
-    f[2 * i] = (__uint_as_float(w << 16) + __uint_as_float(bw << 16)) * scale;
-    f[2 * i + 1] = (__uint_as_float(w & 0xffff0000u) + __uint_as_float(bw & 0xffff0000u)) * scale;
-  }
-  return pack_fp8(f);
-}
-
-// a bf16 K fragment, scaled, as an fp8 fragment
-__device__ inline long kfrag_fp8(u32x4 raw, float scale) {
-  float f[8];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    f[2 * i] = __uint_as_float(raw[i] << 16) * scale;
-    f[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u) * scale;
-  }
-  return pack_fp8(f);
-}
-
-__device__ inline bf16x8 as_bf16x8(u32x4 v) {
-  union { u32x4 u; bf16x8 b; } c;
-  c.u = v;
-  return c.b;
-}
-
-__device__ inline bf16x8 pack8(const f32x16& v, int base) {
-  bf16x8 out;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) out[i] = (__bf16)v[base + i];
-  return out;
-}
-
-// XOR swizzles of the 16-byte chunk index within a K / V row, chosen so that the lanes that
-// read LDS together (16 consecutive rows at one chunk for K; 4 consecutive rows x 4 chunks for
-// the transposing V read) spread over all banks.
-template <int DH> __device__ inline int swz_k(int row) {
-  return DH == 64 ? ((row >> 1) & 7) : DH == 128 ? (row & 15) : ((row >> 2) & 3);
-}
-template <int DH> __device__ inline int swz_v(int row) {
-  return DH == 64 ? (((row >> 1) & 1) << 2) : DH == 128 ? ((row & 3) << 2) : 0;
-}
 
 // NCT = key-channel tiles a WAVE handles per key step; KH = parts the keys of a step are split
 // into (each part has its own waves, which keep a partial soft-max state over their keys and merge
@@ -361,22 +225,50 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   // smaller than one load per wave
   const int n_issue = G::WLOADS >= NW ? G::LPW : (wave < G::WLOADS ? 1 : 0);
 
+  // Phase A (further down) walks the key steps that are far for every query of the workgroup in
+  // groups of STAGES; only V tiles are in flight there, so the K halves of the ring stages lie
+  // idle.  They are used to take the latency of the time-bias slabs off the critical path:
+  //   * the K half of stage 0 receives the 32 + TQW - 1 rows of the time table that the
+  //     workgroup's next slab needs ("row tile": row r = table row base + r, K-tile swizzle),
+  //     requested like a K tile four key steps before the slab is due;
+  //   * the K halves of stages 1 .. hold each wave's (q+v) fragments, written once at set-up.
+  // A slab inside phase A then takes both MFMA operands from LDS instead of waiting for global
+  // memory.  Slabs outside phase A (the window steps at the end) use the global path.
+  const int fast_end = RUNS ? 0 : min(tk_near - (STAGES - 1), tq0 + 1);
+  const int n_groups = fast_end > 0 ? fast_end / STAGES : 0;
+  // (with EARLY the set-up scratch lies over the last stage while the fragments are stored)
+  constexpr bool SLAB_LDS = !RUNS && STAGES >= 3 && G::WLOADS % NW == 0 && CP >= 31 + G::TQW &&
+                            (STAGES - (G::EARLY ? 2 : 1)) * G::TILE_BYTES >= NW * KS * 1024;
+  const bool slab_lds = SLAB_LDS && n_groups > 0 && has_time;
+  auto issue_rows = [&](int tk) {            // row tile of the slab that starts at key step tk
+    const int base = time_row(tq_hi, tk, T_);
+#pragma unroll
+    for (int i = 0; i < G::LPW; ++i) {
+      const int pc = (wave + NW * i) * 64 + lane;
+      const int row = pc / CHUNKS, phys = pc % CHUNKS;
+      const bf16_t* src = ktime + (int64_t)min(base + row, T_ - 1) * DH + ((phys ^ swz_k<DH>(row)) << 3);
+      load_to_lds_16(src, ring_lds + (wave + NW * i) * 1024);
+    }
+  };
+
   // prologue: tiles 0 .. STAGES-2 in flight.  Where the set-up scratch fits into what the
   // prologue leaves alone (the last stage and the time-bias slabs, both first written after the
   // first barrier of the key loop) the tiles are requested right away, so that their round trip
   // overlaps the set-up instead of following it.
   if (G::EARLY) {
+    if (SLAB_LDS && slab_lds) issue_rows(0);
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s)
       if (s <= tq_hi) issue_tile(s, s, s >= tk_near);
   }
 
   // =========================== setup: Qu, Qv, channel bias tile, Ec ===========================
-  // big configurations (Dh 128, or 4 key tiles per wave) are register bound: there the (q+v)
-  // fragments are re-formed at each 32-step slab instead of kept, and the K fragments of a near
-  // step are requested tile by tile instead of all at once
+  // big configurations (Dh 128, or 4 key tiles per wave) are register bound: there the K
+  // fragments of a near step are requested tile by tile instead of all at once.  The (q+v)
+  // fragments are needed once per 32-step slab only and are re-formed there from q (an L2 hit)
+  // instead of kept in registers.
   constexpr bool LEAN = KS * NCT > 8;
-  bf16x8 Qu[KS], Qv[LEAN ? 1 : KS];     // (q+u), (q+v) * scale as QK^T / time-slab B operands
+  bf16x8 Qu[KS];                        // (q+u) * scale as QK^T B operand
   // fp8 content term: q' = (q+u)*scale/sq and k' = k/sk are rounded to e4m3 with the per-head
   // amax scales sq, sk chosen by the caller; the MFMA accumulates in units of 1/(sq*sk), the
   // channel-bias tile is pre-divided accordingly and the product sq*sk returns inside the exp2 fma
@@ -387,6 +279,9 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     fp8_d = sq * sk;
     fp8_inv_sk = 1.f / sk;
   }
+  // this wave's (q+v) fragments for the slabs of phase A, in the K halves of stages 1 ..
+  unsigned char* qv_lds = smem_raw + G::STAGE_BYTES + ((wave * KS * 1024) / G::TILE_BYTES) * G::STAGE_BYTES +
+                          (wave * KS * 1024) % G::TILE_BYTES + lane * 16;
   f32x16 Bc[NCT];            // channel-bias tile, [ck][q] in accumulator layout; -inf = masked key
   {
     u32x4 raw[KS];
@@ -402,7 +297,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
       const int d0 = ks * 16 + hh * 8;
       Qu[ks] = make_qfrag(raw[ks], bu + d0, sc2);
       if (FP8) Qu8[ks] = make_qfrag_fp8(raw[ks], bu + d0, sc2 / a.fp8_q_scale[h]);
-      if (!LEAN) Qv[ks] = make_qfrag(raw[ks], bv + d0, sc2);
+      if (SLAB_LDS && G::EARLY && slab_lds) *(bf16x8*)(qv_lds + ks * 1024) = make_qfrag(raw[ks], bv + d0, sc2);
       const bf16x8 qz = make_qfrag(raw[ks], bz + d0, sc2);
 #pragma unroll
       for (int t = 0; t < G::QT; ++t) {
@@ -504,9 +399,17 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 
   if (!G::EARLY) {
     lds_barrier();           // the set-up scratch aliases the stages the prologue fills
+    if (SLAB_LDS && slab_lds) issue_rows(0);
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s)
       if (s <= tq_hi) issue_tile(s, s, s >= tk_near);
+  }
+  if (SLAB_LDS && slab_lds && !G::EARLY) {        // (with EARLY the set-up stored them already)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d0 = ks * 16 + hh * 8;
+      *(bf16x8*)(qv_lds + ks * 1024) = make_qfrag(*(const u32x4*)(qrow + d0), bv + d0, sc2);
+    }
   }
 
   float* Stb = Stb_all + wave * (32 * 32);
@@ -540,19 +443,29 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 
   // ---- time-bias slab: St[j][q] for key steps [tk, tk+32) -> LDS, plus one soft-max rescale that
   //      covers every far step of the slab
-  auto time_slab = [&](int tk) {
+  auto time_slab = [&](int tk, bool from_lds) {
     const int j0 = time_row(tq, tk, T_);
     f32x16 stc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) stc[i] = 0.f;
-    if (has_time) {
+    if (SLAB_LDS && from_lds) {
+      // row tile in the K half of stage 0: this wave's rows start tq_hi - tq rows into it
+      const int row = tq_hi - tq + ln;
+      const unsigned char* rp = smem_raw + row * ROWB;
+      const int sw = swz_k<DH>(row);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const bf16x8 rr = *(const bf16x8*)(rp + (((2 * ks + hh) ^ sw) << 4));
+        const bf16x8 qv = *(const bf16x8*)(qv_lds + ks * 1024);
+        stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rr, qv, stc, 0, 0, 0);
+      }
+    } else if (has_time) {
       int j = min(j0 + ln, T_ - 1);                // rows past T-1 belong to tk > tq: never used
       if (ring) j = (t_lo + tk + ln + ring_rot) % a.T;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const u32x4 rr = *(const u32x4*)(ktime + (int64_t)j * DH + ks * 16 + hh * 8);
-        const bf16x8 qv = LEAN ? make_qfrag(*(const u32x4*)(qrow + ks * 16 + hh * 8), bv + ks * 16 + hh * 8, sc2)
-                               : Qv[LEAN ? 0 : ks];
+        const bf16x8 qv = make_qfrag(*(const u32x4*)(qrow + ks * 16 + hh * 8), bv + ks * 16 + hh * 8, sc2);
         stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(rr), qv, stc, 0, 0, 0);
       }
     }
@@ -600,10 +513,37 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
       for (int i = 0; i < 16; ++i) acc[mt][i] += et * tmp[mt][i];
   };
 
+  // Soft-max rescale of the running state.  The multiplies are inline assembly on purpose: they
+  // keep the accumulator tiles in their registers on both sides of the (rarely taken) branch
+  // around the rescale; left to the compiler, the branch that skips it copies all the tiles.
+  // The compiler does not see into the assembly, so the wait states that a vector instruction
+  // needs after a matrix instruction wrote its operand (and before one reads its result) are
+  // spelled out: 12 before, 2 after.  The branch is taken a few times per workgroup.
+  auto rescale_acc = [&](float alpha) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      f32x16 x = acc[mt];
+      asm volatile(
+          "s_nop 7\n\ts_nop 3\n\t"
+          "v_mul_f32 %0, %16, %0\n\tv_mul_f32 %1, %16, %1\n\tv_mul_f32 %2, %16, %2\n\tv_mul_f32 %3, %16, %3\n\t"
+          "v_mul_f32 %4, %16, %4\n\tv_mul_f32 %5, %16, %5\n\tv_mul_f32 %6, %16, %6\n\tv_mul_f32 %7, %16, %7\n\t"
+          "v_mul_f32 %8, %16, %8\n\tv_mul_f32 %9, %16, %9\n\tv_mul_f32 %10, %16, %10\n\tv_mul_f32 %11, %16, %11\n\t"
+          "v_mul_f32 %12, %16, %12\n\tv_mul_f32 %13, %16, %13\n\tv_mul_f32 %14, %16, %14\n\tv_mul_f32 %15, %16, %15\n\t"
+          "s_nop 1"
+          : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7]),
+            "+v"(x[8]), "+v"(x[9]), "+v"(x[10]), "+v"(x[11]), "+v"(x[12]), "+v"(x[13]), "+v"(x[14]), "+v"(x[15])
+          : "v"(alpha));
+      acc[mt] = x;
+    }
+  };
+
   // ---- near tile: S^T = K Q^T + Bc, online soft-max, acc += V^T P^T.  The key-channel tiles are
   // taken one after the other (QK^T chains issued tile by tile, then per tile: row max, lazy
   // rescale, exp2, PV), so that the matrix cores work on the next tile's QK^T / the previous
-  // tile's PV while this wave does the vector work of a tile.
+  // tile's PV while this wave does the vector work of a tile.  The V^T fragments of a tile are
+  // requested from LDS BEFORE the vector work of that tile (the first tile's right after the QK^T
+  // chains are issued, the next tile's before the PV products of the current one), so that their
+  // round trip is over when the PV products need them.
   auto near_step = [&](const unsigned char* stage, int tk) {
     const float st = Stb[(tk & 31) * 32 + ln];
     f32x16 S[NCT];
@@ -643,6 +583,17 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
         }
       }
     }
+    // V^T fragments of one key tile, [s][mt]; PREFETCH: requested a tile ahead of their use
+    constexpr bool PREFETCH = !LEAN;
+    bf16x8 vf[2][MT];
+    if (PREFETCH) {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) vf[s][mt] = v_frag(stage, 0, s, mt);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     float ls = 0.f;
 #pragma unroll
     for (int t = 0; t < NCT; ++t) {
@@ -661,10 +612,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
         m_run = m_new;
         l_run *= alpha;
         ls *= alpha;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[mt][i] *= alpha;
+        rescale_acc(alpha);
       }
       const float off = st - m_run;
 #pragma unroll
@@ -682,11 +630,34 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 #pragma unroll
         for (int j = 0; j < 4; ++j) ls = __builtin_amdgcn_fdot2_f32_bf16(u.q[j], kOnes2, ls, false);
       }
+      if (PREFETCH) {
+        bf16x8 vn[2][MT];
+        if (t + 1 < NCT) {
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
+          for (int s = 0; s < 2; ++s)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(stage, t, s, mt), P[s], acc[mt], 0, 0, 0);
+            for (int mt = 0; mt < MT; ++mt) vn[s][mt] = v_frag(stage, t + 1, s, mt);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[s][mt], P[s], acc[mt], 0, 0, 0);
+        if (t + 1 < NCT) {
+#pragma unroll
+          for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) vf[s][mt] = vn[s][mt];
+        }
+      } else {
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(stage, t, s, mt), P[s], acc[mt], 0, 0, 0);
+      }
     }
     l_run += ls;
   };
@@ -709,7 +680,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
           if (t0 + 2 <= T_ - 1) issue_tile(t0 + 2, 2 - 2 * u, t0 + 2 >= tk_near);
           if (t0 + 3 <= T_ - 1) issue_tile(t0 + 3, 3 - 2 * u, t0 + 3 >= tk_near);
         }
-        if ((t0 & 31) == 0) time_slab(t0);
+        if ((t0 & 31) == 0) time_slab(t0, false);
         const int tkw = t0 + par;
         if (tkw <= T_ - 1) {
           const unsigned char* stage = smem_raw + (2 * u) * G::STAGE_BYTES + par * G::STAGE_BYTES;
@@ -730,8 +701,6 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   {
     // uniform over the workgroup (every wave must reach the same barriers): all of these steps
     // are at or before tq0, hence visible to every query of the workgroup
-    const int fast_end = RUNS ? 0 : min(tk_near - (STAGES - 1), tq0 + 1);
-    const int n_groups = fast_end > 0 ? fast_end / STAGES : 0;
     f32x16 ptmp[MT];                       // V^T Ec^T of the previous step, not yet accumulated
     float pet = 0.f;                       // its weight
 #pragma unroll
@@ -750,10 +719,13 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
       for (int s = 0; s < STAGES; ++s, ++tk) {
         wait_vmcnt_imm<(STAGES - 2) * G::LPW>();
         lds_barrier();
+        // the row tile of a slab that phase A will still reach goes out four steps ahead of it
+        // (everybody is past the previous slab's reads of that buffer by now)
+        if (SLAB_LDS && slab_lds && ((tk + 4) & 31) == 0 && tk + 4 < n_groups * STAGES) issue_rows(tk + 4);
         issue_tile(tk + STAGES - 1, (s + STAGES - 1) % STAGES, false);
         if ((tk & 31) == 0 && active) {
           flush();
-          time_slab(tk);
+          time_slab(tk, slab_lds);
         }
         if (active) {
           const unsigned char* stage = smem_raw + s * G::STAGE_BYTES + key_off;
@@ -803,7 +775,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
       lds_barrier();          // tile tk visible to all; everyone is done with tile tk-1's buffer
       if (tk + STAGES - 1 <= tq_hi)
         issue_tile(tk + STAGES - 1, (s + STAGES - 1) % STAGES, tk + STAGES - 1 >= tk_near);
-      if ((tk & 31) == 0 && active) time_slab(tk);
+      if ((tk & 31) == 0 && active) time_slab(tk, false);
       if (active && tk <= tq) {
         const unsigned char* stage = smem_raw + s * G::STAGE_BYTES + key_off;
         if (!RUNS && is_far(tk)) far_step(stage, tk);

@@ -1,0 +1,145 @@
+// Device helpers shared by the tiled bf16 MFMA forward kernels (gfx950, wave64): vector types,
+// LDS-direct tile loads, wait counters, fragment packing, the XOR swizzles of the K / V rows.
+#pragma once
+
+#include "mvpa_common.h"
+
+namespace mvpa {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+#define LDS_PTR(T) __attribute__((address_space(3))) T*
+#define GLOBAL_PTR(T) __attribute__((address_space(1))) T*
+
+__device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+#define kOnes2 (bf16x2{(__bf16)1.0f, (__bf16)1.0f})
+constexpr float kMFloor = -1.0e30f;     // "nothing seen yet" value of a running maximum
+
+// order LDS traffic between the lanes of ONE wave (no workgroup barrier needed)
+__device__ inline void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() would also drain every
+// outstanding global load (vmcnt 0), which would serialise the tile prefetch ring.
+__device__ inline void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// One 64-lane x 16-byte direct-to-LDS load: lane L's 16 bytes land at lds_base + 16*L.  Issued as
+// inline assembly on purpose: the compiler then keeps no record of an LDS write in flight and
+// does not drain the whole prefetch ring (vmcnt 0) in front of every later LDS read; completion
+// is awaited explicitly with wait_vmcnt() before the barrier that publishes the tile.
+__device__ inline void load_to_lds_16(const void* gptr, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :: "v"(gptr), "s"(lds_base) : "memory", "m0");
+}
+
+template <int N>
+__device__ inline void wait_vmcnt_imm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// wait until at most n of this wave's vector-memory operations are outstanding
+__device__ inline void wait_vmcnt(int n) {
+  switch (n) {
+    case 0: wait_vmcnt_imm<0>(); break;
+    case 1: wait_vmcnt_imm<1>(); break;
+    case 2: wait_vmcnt_imm<2>(); break;
+    case 3: wait_vmcnt_imm<3>(); break;
+    case 4: wait_vmcnt_imm<4>(); break;
+    case 5: wait_vmcnt_imm<5>(); break;
+    case 6: wait_vmcnt_imm<6>(); break;
+    case 7: wait_vmcnt_imm<7>(); break;
+    default: wait_vmcnt_imm<8>(); break;      // n >= 8: waiting for <= 8 is only stricter
+  }
+}
+
+// max over a lane and its partner in the other half-wave (lane ^ 32): one register swap between
+// the halves instead of a round trip through the LDS crossbar
+__device__ inline float xhalf_max(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+// 8 bf16 (one 16-byte chunk of a q row) + bias, scaled, back to a bf16 MFMA fragment
+__device__ inline bf16x8 make_qfrag(u32x4 raw, const bf16_t* __restrict__ bias, float scale) {
+  const u32x4 braw = *(const u32x4*)bias;
+  bf16x8 out;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t w = raw[i], bw = braw[i];
+    const float lo = (__uint_as_float(w << 16) + __uint_as_float(bw << 16)) * scale;
+    const float hi = (__uint_as_float(w & 0xffff0000u) + __uint_as_float(bw & 0xffff0000u)) * scale;
+    out[2 * i] = (__bf16)lo;
+    out[2 * i + 1] = (__bf16)hi;
+  }
+  return out;
+}
+
+// 8 floats -> 8 fp8 (e4m3) packed in 64 bits, the operand of the 32x32x16 fp8 MFMA
+__device__ inline long pack_fp8(const float (&f)[8]) {
+  int lo = 0, hi = 0;
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], hi, false);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
+  return (long)(((unsigned long)(unsigned)hi << 32) | (unsigned)lo);
+}
+
+// (q + bias) * scale as an fp8 fragment
+__device__ inline long make_qfrag_fp8(u32x4 raw, const bf16_t* __restrict__ bias, float scale) {
+  const u32x4 braw = *(const u32x4*)bias;
+  float f[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t w = raw[i], bw = braw[i];
+    f[2 * i] = (__uint_as_float(w << 16) + __uint_as_float(bw << 16)) * scale;
+    f[2 * i + 1] = (__uint_as_float(w & 0xffff0000u) + __uint_as_float(bw & 0xffff0000u)) * scale;
+  }
+  return pack_fp8(f);
+}
+
+// a bf16 K fragment, scaled, as an fp8 fragment
+__device__ inline long kfrag_fp8(u32x4 raw, float scale) {
+  float f[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = __uint_as_float(raw[i] << 16) * scale;
+    f[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u) * scale;
+  }
+  return pack_fp8(f);
+}
+
+__device__ inline bf16x8 as_bf16x8(u32x4 v) {
+  union { u32x4 u; bf16x8 b; } c;
+  c.u = v;
+  return c.b;
+}
+
+__device__ inline bf16x8 pack8(const f32x16& v, int base) {
+  bf16x8 out;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) out[i] = (__bf16)v[base + i];
+  return out;
+}
+
+// XOR swizzles of the 16-byte chunk index within a K / V row, chosen so that the lanes that
+// read LDS together (16 consecutive rows at one chunk for K; 4 consecutive rows x 4 chunks for
+// the transposing V read) spread over all banks.
+template <int DH> __device__ inline int swz_k(int row) {
+  return DH == 64 ? ((row >> 1) & 7) : DH == 128 ? (row & 15) : ((row >> 2) & 3);
+}
+template <int DH> __device__ inline int swz_v(int row) {
+  return DH == 64 ? (((row >> 1) & 1) << 2) : DH == 128 ? ((row & 3) << 2) : 0;
+}
+
+}  // namespace mvpa
