@@ -49,7 +49,13 @@ enum {
 enum {
   MVPA_KERNEL_AUTO = 0,     /* bf16: tiled MFMA kernel when it supports the shape       */
   MVPA_KERNEL_GENERIC = 1,  /* fp32-math row-per-lane kernel, any shape                 */
-  MVPA_KERNEL_MFMA = 2      /* bf16 MFMA kernel, error if the shape is unsupported      */
+  MVPA_KERNEL_MFMA = 2,     /* bf16 MFMA kernel, error if the shape is unsupported      */
+  MVPA_KERNEL_MFMA_STEP = 3 /* the build of the bf16 MFMA kernel in which a wave owns a whole
+                               time step (two tiles of 32 queries; head size 64, 33..64
+                               channels, plain forward), whatever the length; error if the
+                               shape is unsupported.  AUTO and MFMA pick it by themselves for
+                               128 time steps and more or when the content term is off, where
+                               it is the faster one.                                       */
 };
 
 /* ---- flags ------------------------------------------------------------------------- */

@@ -28,7 +28,7 @@ extern "C" int mvpa_validate(const mvpa_fwd_args* a) {
   if (!a) return MVPA_ERR_NULL;
   if (a->struct_size != sizeof(mvpa_fwd_args)) return MVPA_ERR_STRUCT;
   if (a->dtype != MVPA_F32 && a->dtype != MVPA_BF16) return MVPA_ERR_DTYPE;
-  if (a->kernel < MVPA_KERNEL_AUTO || a->kernel > MVPA_KERNEL_MFMA) return MVPA_ERR_DTYPE;
+  if (a->kernel < MVPA_KERNEL_AUTO || a->kernel > MVPA_KERNEL_MFMA_STEP) return MVPA_ERR_DTYPE;
   if (a->Dh != 16 && a->Dh != 32 && a->Dh != 64 && a->Dh != 128) return MVPA_ERR_HEAD_DIM;
   if (a->B <= 0 || a->H <= 0 || a->Hkv <= 0) return MVPA_ERR_SHAPE;
   if (a->H % a->Hkv != 0) return MVPA_ERR_HEAD_RATIO;
@@ -63,7 +63,9 @@ extern "C" int mvpa_validate(const mvpa_fwd_args* a) {
     const int len = (a->T + a->n_split - 1) / a->n_split;
     if ((int64_t)(a->n_split - 1) * len >= a->T) return MVPA_ERR_SHAPE;   // an empty run
   }
-  if (a->kernel == MVPA_KERNEL_MFMA && !mvpa_mfma_supported(a)) {
+  if (a->kernel == MVPA_KERNEL_MFMA_STEP && mvpa_mfma_supported(a) && !mvpa_mfma64_supported(a))
+    return MVPA_ERR_UNSUPPORTED;
+  if ((a->kernel == MVPA_KERNEL_MFMA || a->kernel == MVPA_KERNEL_MFMA_STEP) && !mvpa_mfma_supported(a)) {
     if (a->dtype == MVPA_BF16) {
       const uintptr_t p = (uintptr_t)a->q | (uintptr_t)a->k | (uintptr_t)a->v | (uintptr_t)a->o;
       const int64_t s = a->q_stride_b | a->q_stride_h | a->q_stride_n | a->k_stride_b |
@@ -85,13 +87,14 @@ extern "C" int mvpa_select_kernel(const mvpa_fwd_args* a) {
   const int st = mvpa_validate(a);
   if (st != MVPA_OK) return st;
   if (a->kernel == MVPA_KERNEL_GENERIC) return MVPA_KERNEL_GENERIC;
-  if (a->kernel == MVPA_KERNEL_MFMA) return MVPA_KERNEL_MFMA;
+  if (a->kernel == MVPA_KERNEL_MFMA || a->kernel == MVPA_KERNEL_MFMA_STEP) return MVPA_KERNEL_MFMA;
   return mvpa_mfma_supported(a) ? MVPA_KERNEL_MFMA : MVPA_KERNEL_GENERIC;
 }
 
 extern "C" int mvpa_forward(const mvpa_fwd_args* a, void* stream) {
   const int sel = mvpa_select_kernel(a);
   if (sel < 0) return sel;
+  if (sel == MVPA_KERNEL_MFMA && a->kernel == MVPA_KERNEL_MFMA_STEP) return mvpa_launch_mfma64(a, (hipStream_t)stream);
   if (sel == MVPA_KERNEL_MFMA) return mvpa_launch_mfma(a, (hipStream_t)stream);
   if (a->flags & (MVPA_FLAG_FP8_QK | MVPA_FLAG_RING)) return MVPA_ERR_UNSUPPORTED;
   return mvpa_launch_generic(a, (hipStream_t)stream);

@@ -43,6 +43,14 @@ __device__ inline void load_to_lds_16(const void* gptr, uint32_t lds_base) {
                :: "v"(gptr), "s"(lds_base) : "memory", "m0");
 }
 
+// The same load with the address split into a wave-uniform base (scalar registers) and a 32-bit
+// byte offset per lane: one vector register per load instead of a 64-bit pair, and no 64-bit
+// vector add per tile.
+__device__ inline void load_to_lds_16(const void* sbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(voff), "s"(sbase), "s"(lds_base) : "memory", "m0");
+}
+
 template <int N>
 __device__ inline void wait_vmcnt_imm() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");

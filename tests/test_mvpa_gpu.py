@@ -203,6 +203,90 @@ def test_bf16_mfma_shapes(cfg):
     assert (lse.cpu().double() - ref_lse).abs().max().item() <= 3e-2
 
 
+# the build of the kernel in which a wave owns a whole time step (head size 64, 33..64 channels);
+# the dispatcher picks it from 128 time steps on, the tests force it at every length
+STEP_SHAPES = [
+    dict(B=2, C=64, T=16, H=2, Dh=64),                             # no far steps but the last-step workgroup
+    dict(B=1, C=64, T=40, H=2, Dh=64),                             # far steps, two slabs, T a multiple of 4
+    dict(B=2, C=40, T=33, H=4, Hkv=2, Dh=64, validity=True),       # ragged channels, GQA, T-1 a multiple of 4
+    dict(B=1, C=33, T=70, H=3, Hkv=1, Dh=64),                      # three slabs; B*H not a multiple of 8
+    dict(B=1, C=64, T=134, H=2, Dh=64, validity=True),             # past 128 steps (also the dispatcher's choice)
+    dict(B=4, C=64, T=9, H=4, Dh=64),                              # two (b,h) per XCD: merged tail order
+    dict(B=2, C=48, T=11, H=8, Dh=64, Hkv=2),                      # window just vacuous
+    dict(B=1, C=64, T=64, H=3, Dh=64, Hkv=1),                      # MVPFormer-S's attention shape
+    dict(B=1, C=50, T=1, H=2, Dh=64),                              # a single time step
+    dict(B=1, C=64, T=2, H=1, Dh=64),
+    dict(B=1, C=64, T=5, H=2, Dh=64),
+    dict(B=1, C=36, T=6, H=2, Dh=64),                              # T-1 = 5: a tile of one time step
+]
+
+
+@pytest.mark.parametrize("cfg", STEP_SHAPES)
+def test_bf16_whole_step_build_shapes(cfg):
+    inp = make_mvpa_inputs(seed=27, table_std=0.3, qkv_unit=True, **cfg).round_to(torch.bfloat16)
+    out, lse = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA_STEP, return_lse=True)
+    ref, ref_lse = _oracle(inp, return_lse=True)
+    _check_bf16(out, ref)
+    assert (lse.cpu().double() - ref_lse).abs().max().item() <= 3e-2
+
+
+@pytest.mark.parametrize("kw", [dict(window=3), dict(window=0), dict(content=False), dict(window=1),
+                                dict(time_bias=False), dict(chan_bias=False), dict(sm_scale=0.05),
+                                dict(window=200)])
+def test_bf16_whole_step_build_flags(kw):
+    inp = make_mvpa_inputs(B=1, C=48, T=45, H=2, Dh=64, seed=28, table_std=0.3,
+                           qkv_unit=True).round_to(torch.bfloat16)
+    out = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA_STEP, **kw)
+    okw = dict(kw)
+    if "content" in okw:
+        okw["global_att"] = okw.pop("content")
+    tb, cb = okw.pop("time_bias", True), okw.pop("chan_bias", True)
+    ref_in = inp
+    if not tb or not cb:
+        import copy
+        ref_in = copy.copy(inp)
+        if not tb:
+            ref_in.k_time = torch.zeros_like(inp.k_time)
+        if not cb:
+            ref_in.k_chan = torch.zeros_like(inp.k_chan)
+    _check_bf16(out, _oracle(ref_in, **okw))
+
+
+def test_bf16_whole_step_build_large_logits_and_masks():
+    """Wide score range (running-max bookkeeping across the window passes and the far phase), and
+    masks exact under perturbation, on the whole-time-step build."""
+    inp = make_mvpa_inputs(B=1, C=40, T=48, H=2, Dh=64, seed=23, table_std=1.0).round_to(torch.bfloat16)
+    out = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA_STEP)
+    assert torch.isfinite(out).all()
+    _check_bf16(out, _oracle(inp))
+    cfg = dict(B=1, C=40, T=20, H=2, Dh=64, seed=9, table_std=0.3, qkv_unit=True, validity=True)
+    inp = make_mvpa_inputs(**cfg)
+    inp.chan_valid[0, 2] = False
+    run = lambda i: _gpu(i, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA_STEP)    # noqa: E731
+    base = run(inp)
+    C, T = inp.C, inp.T
+    p = make_mvpa_inputs(**cfg)
+    p.chan_valid = inp.chan_valid
+    dead = (~inp.chan_valid[0]).nonzero().flatten()
+    for t in range(T):
+        p.k[:, :, t * C + dead] += 5.0
+        p.v[:, :, t * C + dead] = 1.0e4
+    p.k[:, :, -C:] *= 2.0
+    p.v[:, :, -C:] *= 2.0
+    assert torch.equal(run(p)[:, :, :-C], base[:, :, :-C])
+    p = make_mvpa_inputs(**cfg)
+    p.chan_valid = inp.chan_valid
+    p.k[:, :, :C] += 1.0
+    same = (run(p) == base).flatten(0, 1).all(-1).view(-1, T, C).all(0).all(-1).cpu()
+    assert same.tolist() == [not (t <= 10 or t == T - 1) for t in range(T)]
+
+
+def test_whole_step_build_refuses_other_shapes():
+    d = make_mvpa_inputs(seed=1, B=1, C=20, T=6, H=1, Dh=64).to("cuda", torch.bfloat16)
+    with pytest.raises(mvpa_hip.MvpaError):
+        mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, kernel=mvpa_hip.KERNEL_MFMA_STEP)
+
+
 @pytest.mark.parametrize("kw", [dict(window=3), dict(window=0), dict(content=False),
                                 dict(time_bias=False), dict(chan_bias=False), dict(sm_scale=0.05)])
 def test_bf16_mfma_flags(kw):
@@ -354,8 +438,13 @@ def _gather_case(C, T, Dh, rows, axis):
     return q, k, v, zero, unit, k_time, k_chan
 
 
-@pytest.mark.parametrize("cfg", GATHER_SHAPES, ids=lambda c: "C{C}T{T}D{Dh}".format(**c))
-def test_mfma_channel_gather_is_exact(cfg):
+GATHER_CASES = [(c, "KERNEL_MFMA") for c in GATHER_SHAPES] + [
+    (dict(C=64, T=40, Dh=64), "KERNEL_MFMA_STEP"), (dict(C=40, T=70, Dh=64), "KERNEL_MFMA_STEP")]
+_gather_id = lambda c: "C{C}T{T}D{Dh}".format(**c) if isinstance(c, dict) else c      # noqa: E731
+
+
+@pytest.mark.parametrize("cfg,kern", GATHER_CASES, ids=_gather_id)
+def test_mfma_channel_gather_is_exact(cfg, kern):
     C, T, Dh = cfg["C"], cfg["T"], cfg["Dh"]
     cq, ck = torch.arange(C)[:, None], torch.arange(C)[None, :]
     onehot = torch.zeros(C, Dh)
@@ -364,7 +453,7 @@ def test_mfma_channel_gather_is_exact(cfg):
         rows = list(range(r0, min(C, r0 + 16)))
         q, k, v, zero, unit, k_time, k_chan = _gather_case(C, T, Dh, rows, "chan")
         out = mvpa_hip.mvpa_forward(*(t.cuda().bfloat16() for t in (q, k, v, zero, zero, unit, k_time, k_chan)),
-                                    sm_scale=1.0, kernel=mvpa_hip.KERNEL_MFMA).float().cpu()
+                                    sm_scale=1.0, kernel=getattr(mvpa_hip, kern)).float().cpu()
         for g, j in enumerate(rows):
             hit = (C - 1 - (cq - ck).abs()) == j                  # keys whose gathered row is j*
             w = torch.where(hit.any(1, keepdim=True), hit, torch.ones_like(hit)).float()
@@ -373,14 +462,14 @@ def test_mfma_channel_gather_is_exact(cfg):
             assert (got - want[None]).abs().max().item() <= 1e-2, (j, (got - want[None]).abs().max().item())
 
 
-@pytest.mark.parametrize("cfg", GATHER_SHAPES, ids=lambda c: "C{C}T{T}D{Dh}".format(**c))
-def test_mfma_time_gather_is_exact(cfg):
+@pytest.mark.parametrize("cfg,kern", GATHER_CASES, ids=_gather_id)
+def test_mfma_time_gather_is_exact(cfg, kern):
     C, T, Dh = cfg["C"], cfg["T"], cfg["Dh"]
     for r0 in range(0, T, 16):
         rows = list(range(r0, min(T, r0 + 16)))
         q, k, v, zero, unit, k_time, k_chan = _gather_case(C, T, Dh, rows, "time")
         out = mvpa_hip.mvpa_forward(*(t.cuda().bfloat16() for t in (q, k, v, zero, unit, zero, k_time, k_chan)),
-                                    sm_scale=1.0, kernel=mvpa_hip.KERNEL_MFMA).float().cpu()
+                                    sm_scale=1.0, kernel=getattr(mvpa_hip, kern)).float().cpu()
         for g, j in enumerate(rows):
             got = out[0, g].view(T, C, Dh)
             for tq in range(T):
