@@ -39,6 +39,16 @@ BF16_DENSE_PEAK_TFLOPS = 2500.0       # MI355X published dense bf16 MFMA peak
 # HBM bytes per launch of the attention kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by
 # what the same counters read for a plain device copy of known size; the profile summary named
 # beside each figure holds the two counter runs.
+def _forward_kernel_name(cfg):
+    """The build of the bf16 forward that the library's own choice (MVPA_KERNEL_AUTO) runs for a
+    workload: the rule of mvpa_forward in csrc/mvpa_api.hip."""
+    if cfg["Dh"] == 128 and 64 < cfg["C"] <= 128:
+        return "mvpa::d128::mvpa_mfma128_kernel"
+    if cfg["Dh"] == 64 and 32 < cfg["C"] <= 64 and cfg["T"] >= 128:
+        return "mvpa::q64::mvpa_mfma64_kernel"
+    return "mvpa::mvpa_mfma_kernel"
+
+
 MEASURED_TRAFFIC_BYTES = {"c2": (402.4e6, "profiles/mvpa_mfma_kernel_c2.md")}
 PREWARM_LAUNCHES = 150
 
@@ -182,7 +192,7 @@ def main():
 
     def step():
         mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
-                              chan_valid=d.chan_valid, out=out, kernel=mvpa_hip.KERNEL_MFMA)
+                              chan_valid=d.chan_valid, out=out)
 
     if args.copy_probe:
         src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device="cuda:0").random_(0, 255)
@@ -225,7 +235,7 @@ def main():
                      "frac": round(kern_tflops / BF16_DENSE_PEAK_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, (None, None))[0],
                      "traffic_source": MEASURED_TRAFFIC_BYTES.get(args.workload, (None, None))[1],
-                     "kernel": "mvpa_mfma_kernel", "kernel_ms": round(kern_ms, 4)},
+                     "kernel": _forward_kernel_name(cfg), "kernel_ms": round(kern_ms, 4)},
     }
     if not args.no_backward and C <= 128:   # shapes the matrix-core backward serves
         # the backward of the same workload (reported beside the headline, never part of `value`):

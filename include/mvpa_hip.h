@@ -47,15 +47,22 @@ enum {
 
 /* ---- kernel selector --------------------------------------------------------------- */
 enum {
-  MVPA_KERNEL_AUTO = 0,     /* bf16: tiled MFMA kernel when it supports the shape       */
+  MVPA_KERNEL_AUTO = 0,     /* bf16: the fastest MFMA build that supports the shape (the general
+                               tiled kernel or one of the two specialised builds below), the
+                               fp32 kernel otherwise                                       */
   MVPA_KERNEL_GENERIC = 1,  /* fp32-math row-per-lane kernel, any shape                 */
-  MVPA_KERNEL_MFMA = 2,     /* bf16 MFMA kernel, error if the shape is unsupported      */
-  MVPA_KERNEL_MFMA_STEP = 3 /* the build of the bf16 MFMA kernel in which a wave owns a whole
-                               time step (two tiles of 32 queries; head size 64, 33..64
-                               channels, plain forward), whatever the length; error if the
-                               shape is unsupported.  AUTO and MFMA pick it by themselves for
-                               128 time steps and more or when the content term is off, where
-                               it is the faster one.                                       */
+  MVPA_KERNEL_MFMA = 2,     /* the general tiled bf16 MFMA kernel (a wave owns one tile of 32
+                               queries and every output column), error if the shape is
+                               unsupported                                                 */
+  MVPA_KERNEL_MFMA_STEP = 3, /* the build in which a wave owns a whole time step (two tiles of
+                               32 queries; head size 64, 33..64 channels, plain forward),
+                               whatever the length; error if the shape is unsupported.  AUTO
+                               picks it for 128 time steps and more or when the content term
+                               is off, where it is the faster one.                         */
+  MVPA_KERNEL_MFMA_SPLIT = 4 /* the build in which the output columns of a query tile are split
+                               over two waves (head size 128, 65..128 channels, plain
+                               forward); error if the shape is unsupported.  AUTO picks it
+                               for every such shape.                                       */
 };
 
 /* ---- flags ------------------------------------------------------------------------- */

@@ -28,7 +28,7 @@ extern "C" int mvpa_validate(const mvpa_fwd_args* a) {
   if (!a) return MVPA_ERR_NULL;
   if (a->struct_size != sizeof(mvpa_fwd_args)) return MVPA_ERR_STRUCT;
   if (a->dtype != MVPA_F32 && a->dtype != MVPA_BF16) return MVPA_ERR_DTYPE;
-  if (a->kernel < MVPA_KERNEL_AUTO || a->kernel > MVPA_KERNEL_MFMA_STEP) return MVPA_ERR_DTYPE;
+  if (a->kernel < MVPA_KERNEL_AUTO || a->kernel > MVPA_KERNEL_MFMA_SPLIT) return MVPA_ERR_DTYPE;
   if (a->Dh != 16 && a->Dh != 32 && a->Dh != 64 && a->Dh != 128) return MVPA_ERR_HEAD_DIM;
   if (a->B <= 0 || a->H <= 0 || a->Hkv <= 0) return MVPA_ERR_SHAPE;
   if (a->H % a->Hkv != 0) return MVPA_ERR_HEAD_RATIO;
@@ -65,7 +65,9 @@ extern "C" int mvpa_validate(const mvpa_fwd_args* a) {
   }
   if (a->kernel == MVPA_KERNEL_MFMA_STEP && mvpa_mfma_supported(a) && !mvpa_mfma64_supported(a))
     return MVPA_ERR_UNSUPPORTED;
-  if ((a->kernel == MVPA_KERNEL_MFMA || a->kernel == MVPA_KERNEL_MFMA_STEP) && !mvpa_mfma_supported(a)) {
+  if (a->kernel == MVPA_KERNEL_MFMA_SPLIT && mvpa_mfma_supported(a) && !mvpa_mfma128_supported(a))
+    return MVPA_ERR_UNSUPPORTED;
+  if (a->kernel >= MVPA_KERNEL_MFMA && !mvpa_mfma_supported(a)) {
     if (a->dtype == MVPA_BF16) {
       const uintptr_t p = (uintptr_t)a->q | (uintptr_t)a->k | (uintptr_t)a->v | (uintptr_t)a->o;
       const int64_t s = a->q_stride_b | a->q_stride_h | a->q_stride_n | a->k_stride_b |
@@ -87,15 +89,29 @@ extern "C" int mvpa_select_kernel(const mvpa_fwd_args* a) {
   const int st = mvpa_validate(a);
   if (st != MVPA_OK) return st;
   if (a->kernel == MVPA_KERNEL_GENERIC) return MVPA_KERNEL_GENERIC;
-  if (a->kernel == MVPA_KERNEL_MFMA || a->kernel == MVPA_KERNEL_MFMA_STEP) return MVPA_KERNEL_MFMA;
+  if (a->kernel >= MVPA_KERNEL_MFMA) return MVPA_KERNEL_MFMA;
   return mvpa_mfma_supported(a) ? MVPA_KERNEL_MFMA : MVPA_KERNEL_GENERIC;
 }
 
 extern "C" int mvpa_forward(const mvpa_fwd_args* a, void* stream) {
   const int sel = mvpa_select_kernel(a);
   if (sel < 0) return sel;
-  if (sel == MVPA_KERNEL_MFMA && a->kernel == MVPA_KERNEL_MFMA_STEP) return mvpa_launch_mfma64(a, (hipStream_t)stream);
-  if (sel == MVPA_KERNEL_MFMA) return mvpa_launch_mfma(a, (hipStream_t)stream);
+  if (sel == MVPA_KERNEL_MFMA) {
+    hipStream_t st = (hipStream_t)stream;
+    if (a->kernel == MVPA_KERNEL_MFMA_STEP) return mvpa_launch_mfma64(a, st);
+    if (a->kernel == MVPA_KERNEL_MFMA_SPLIT) return mvpa_launch_mfma128(a, st);
+    if (a->kernel == MVPA_KERNEL_MFMA) return mvpa_launch_mfma(a, st);
+    // AUTO: the specialised builds where they are the faster ones.
+    // Head size 128, 65..128 channels: the column-split build wins at every length measured
+    // (B1 H16 C128: T 16 .. 1024, 13 .. 20 % less time than the general kernel; C 80 .. 100: 21 .. 40 %).
+    if (mvpa_mfma128_supported(a)) return mvpa_launch_mfma128(a, st);
+    // Head size 64, 33..64 channels: the whole-time-step build pays for its window passes with a
+    // cheaper far phase; against the general kernel it loses at 64 time steps (B4 H12 C64: 0.131
+    // against 0.109 ms), is level at 128 and wins from there on (T 256: 6 %, T 512: 10 %), and
+    // wins by 15 % when there are no window steps at all (content term off).
+    if (mvpa_mfma64_supported(a) && (a->T >= 128 || !(a->flags & MVPA_FLAG_CONTENT))) return mvpa_launch_mfma64(a, st);
+    return mvpa_launch_mfma(a, st);
+  }
   if (a->flags & (MVPA_FLAG_FP8_QK | MVPA_FLAG_RING)) return MVPA_ERR_UNSUPPORTED;
   return mvpa_launch_generic(a, (hipStream_t)stream);
 }

@@ -85,6 +85,8 @@ int mvpa_mfma_supported(const mvpa_fwd_args* a);
 // the build of it in which a wave owns a whole time step (head size 64, 33..64 channels)
 int mvpa_mfma64_supported(const mvpa_fwd_args* a);
 int mvpa_launch_mfma64(const mvpa_fwd_args* a, hipStream_t stream);
+int mvpa_mfma128_supported(const mvpa_fwd_args* a);
+int mvpa_launch_mfma128(const mvpa_fwd_args* a, hipStream_t stream);
 // backward, query pass on MFMA (bf16, Dh = 64, C <= 64)
 int mvpa_bwd_query_mfma_supported(const mvpa_bwd_args* a);
 int mvpa_launch_bwd_mfma(const mvpa_bwd_args* a, hipStream_t stream);

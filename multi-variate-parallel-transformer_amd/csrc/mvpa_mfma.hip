@@ -931,12 +931,6 @@ int mvpa_mfma_supported(const mvpa_fwd_args* a) {
 
 int mvpa_launch_mfma(const mvpa_fwd_args* a, hipStream_t stream) {
   using namespace mvpa;
-  // head size 64, 33..64 channels: the whole-time-step build pays for its window passes with a
-  // cheaper far phase; measured against this kernel it loses at 64 time steps (B4 H12 C64: 0.131
-  // against 0.109 ms), is level at 128 and wins from there on (T 256: 6 %, T 512: 10 %), and
-  // wins by 15 % when there are no window steps at all (content term off)
-  if (mvpa_mfma64_supported(a) && (a->T >= 128 || !(a->flags & MVPA_FLAG_CONTENT)))
-    return mvpa_launch_mfma64(a, stream);
   const int nct = a->C <= 32 ? 1 : a->C <= 64 ? 2 : 4;
   switch (a->Dh) {
     case 32:

@@ -51,6 +51,13 @@ __device__ inline void load_to_lds_16(const void* sbase, uint32_t voff, uint32_t
                :: "v"(voff), "s"(sbase), "s"(lds_base) : "memory", "m0");
 }
 
+// The bare workgroup barrier: LDS reads of this wave may stay in flight across it.  For places
+// where the barrier publishes tiles that arrived by direct-to-LDS loads (awaited with
+// wait_vmcnt) and no wave's outstanding reads touch memory that is rewritten before they return.
+__device__ inline void bare_barrier() {
+  asm volatile("s_barrier" ::: "memory");
+}
+
 template <int N>
 __device__ inline void wait_vmcnt_imm() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");

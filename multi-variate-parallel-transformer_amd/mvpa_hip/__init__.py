@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmvpa_hip.so")
 
 MVPA_F32, MVPA_BF16 = 0, 1
-KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA, KERNEL_MFMA_STEP = 0, 1, 2, 3
+KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA, KERNEL_MFMA_STEP, KERNEL_MFMA_SPLIT = 0, 1, 2, 3, 4
 FLAG_LAST_STEP = 32
 FLAG_RING = 64
 FLAG_CAUSAL, FLAG_CONTENT, FLAG_TIME_BIAS, FLAG_CHAN_BIAS, FLAG_FP8_QK = 1, 2, 4, 8, 16

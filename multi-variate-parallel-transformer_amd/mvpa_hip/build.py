@@ -12,7 +12,7 @@ CSRC = os.path.join(PKG, "csrc")
 INCLUDE = os.path.join(os.path.dirname(PKG), "include")
 LIB = os.path.join(HERE, "libmvpa_hip.so")
 
-SOURCES = ["mvpa_api.hip", "mvpa_generic.hip", "mvpa_mfma.hip", "mvpa_mfma64.hip", "mvpa_dense.hip", "mvpa_backward.hip",
+SOURCES = ["mvpa_api.hip", "mvpa_generic.hip", "mvpa_mfma.hip", "mvpa_mfma64.hip", "mvpa_mfma128.hip", "mvpa_dense.hip", "mvpa_backward.hip",
            "mvpa_backward_mfma.hip", "mvpa_static_ws.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming packed fp32 VALU instructions.

@@ -287,6 +287,91 @@ def test_whole_step_build_refuses_other_shapes():
         mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, kernel=mvpa_hip.KERNEL_MFMA_STEP)
 
 
+# the build of the kernel in which the output columns of a query tile are split over two waves
+# (head size 128, 65..128 channels): the dispatcher's choice for such shapes
+SPLIT_SHAPES = [
+    dict(B=1, C=128, T=26, H=2, Dh=128, Hkv=1),                    # the base model's attention shape, GQA 2:1
+    dict(B=1, C=100, T=24, H=4, Dh=128, Hkv=2, validity=True),     # ragged channels, absent channels
+    dict(B=1, C=128, T=45, H=2, Dh=128, Hkv=1, validity=True),     # two 32-step slabs
+    dict(B=1, C=65, T=40, H=2, Dh=128),                            # just past 64: three key tiles, one nearly empty
+    dict(B=2, C=96, T=13, H=2, Dh=128, Hkv=1),                     # three key tiles exactly; two far steps
+    dict(B=1, C=97, T=70, H=3, Dh=128, Hkv=1),                     # four key tiles, one nearly empty; three slabs; B*H odd
+    dict(B=4, C=80, T=9, H=4, Dh=128),                             # no far steps; two (b,h) per XCD
+    dict(B=1, C=128, T=1, H=2, Dh=128),                            # a single time step
+    dict(B=1, C=70, T=2, H=1, Dh=128),
+    dict(B=1, C=128, T=12, H=2, Dh=128, Hkv=2),                    # exactly one far step
+]
+
+
+@pytest.mark.parametrize("cfg", SPLIT_SHAPES)
+def test_bf16_column_split_build_shapes(cfg):
+    inp = make_mvpa_inputs(seed=29, table_std=0.3, qkv_unit=True, **cfg).round_to(torch.bfloat16)
+    out, lse = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA_SPLIT, return_lse=True)
+    ref, ref_lse = _oracle(inp, return_lse=True)
+    _check_bf16(out, ref)
+    assert (lse.cpu().double() - ref_lse).abs().max().item() <= 3e-2
+    auto = _gpu(inp, torch.bfloat16)                       # the dispatcher picks this build
+    assert torch.equal(auto, out)
+
+
+@pytest.mark.parametrize("kw", [dict(window=3), dict(window=0), dict(content=False), dict(window=1),
+                                dict(time_bias=False), dict(chan_bias=False), dict(sm_scale=0.05),
+                                dict(window=200)])
+def test_bf16_column_split_build_flags(kw):
+    inp = make_mvpa_inputs(B=1, C=72, T=45, H=2, Dh=128, seed=30, table_std=0.3,
+                           qkv_unit=True).round_to(torch.bfloat16)
+    out = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA_SPLIT, **kw)
+    okw = dict(kw)
+    if "content" in okw:
+        okw["global_att"] = okw.pop("content")
+    tb, cb = okw.pop("time_bias", True), okw.pop("chan_bias", True)
+    ref_in = inp
+    if not tb or not cb:
+        import copy
+        ref_in = copy.copy(inp)
+        if not tb:
+            ref_in.k_time = torch.zeros_like(inp.k_time)
+        if not cb:
+            ref_in.k_chan = torch.zeros_like(inp.k_chan)
+    _check_bf16(out, _oracle(ref_in, **okw))
+
+
+def test_bf16_column_split_build_large_logits_and_masks():
+    """Wide score range (running-max bookkeeping across the window steps and the far phase), and
+    masks exact under perturbation, on the column-split build."""
+    inp = make_mvpa_inputs(B=1, C=72, T=48, H=2, Dh=128, seed=23, table_std=1.0).round_to(torch.bfloat16)
+    out = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA_SPLIT)
+    assert torch.isfinite(out).all()
+    _check_bf16(out, _oracle(inp))
+    cfg = dict(B=1, C=100, T=20, H=2, Dh=128, seed=9, table_std=0.3, qkv_unit=True, validity=True)
+    inp = make_mvpa_inputs(**cfg)
+    inp.chan_valid[0, 2] = False
+    run = lambda i: _gpu(i, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA_SPLIT)    # noqa: E731
+    base = run(inp)
+    C, T = inp.C, inp.T
+    p = make_mvpa_inputs(**cfg)
+    p.chan_valid = inp.chan_valid
+    dead = (~inp.chan_valid[0]).nonzero().flatten()
+    for t in range(T):
+        p.k[:, :, t * C + dead] += 5.0
+        p.v[:, :, t * C + dead] = 1.0e4
+    p.k[:, :, -C:] *= 2.0
+    p.v[:, :, -C:] *= 2.0
+    assert torch.equal(run(p)[:, :, :-C], base[:, :, :-C])
+    p = make_mvpa_inputs(**cfg)
+    p.chan_valid = inp.chan_valid
+    p.k[:, :, :C] += 1.0
+    same = (run(p) == base).flatten(0, 1).all(-1).view(-1, T, C).all(0).all(-1).cpu()
+    assert same.tolist() == [not (t <= 10 or t == T - 1) for t in range(T)]
+
+
+def test_column_split_build_refuses_other_shapes():
+    for cfg in (dict(C=64, Dh=128), dict(C=100, Dh=64)):
+        d = make_mvpa_inputs(seed=1, B=1, T=6, H=1, **cfg).to("cuda", torch.bfloat16)
+        with pytest.raises(mvpa_hip.MvpaError):
+            mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, kernel=mvpa_hip.KERNEL_MFMA_SPLIT)
+
+
 @pytest.mark.parametrize("kw", [dict(window=3), dict(window=0), dict(content=False),
                                 dict(time_bias=False), dict(chan_bias=False), dict(sm_scale=0.05)])
 def test_bf16_mfma_flags(kw):
@@ -439,7 +524,8 @@ def _gather_case(C, T, Dh, rows, axis):
 
 
 GATHER_CASES = [(c, "KERNEL_MFMA") for c in GATHER_SHAPES] + [
-    (dict(C=64, T=40, Dh=64), "KERNEL_MFMA_STEP"), (dict(C=40, T=70, Dh=64), "KERNEL_MFMA_STEP")]
+    (dict(C=64, T=40, Dh=64), "KERNEL_MFMA_STEP"), (dict(C=40, T=70, Dh=64), "KERNEL_MFMA_STEP"),
+    (dict(C=128, T=40, Dh=128), "KERNEL_MFMA_SPLIT"), (dict(C=70, T=70, Dh=128), "KERNEL_MFMA_SPLIT")]
 _gather_id = lambda c: "C{C}T{T}D{Dh}".format(**c) if isinstance(c, dict) else c      # noqa: E731
 
 
@@ -532,26 +618,29 @@ def test_bf16_mfma_strided_layout_and_auto_dispatch():
     _check_bf16(merged.permute(0, 2, 1, 3), _oracle(inp))
 
 
-def test_bf16_config2_full_size():
-    """Config c2 (B4 C64 T128 H16 Dh64): two heads against the oracle, the rest through
+@pytest.mark.parametrize("kern", ["KERNEL_AUTO", "KERNEL_MFMA"])
+def test_bf16_config2_full_size(kern):
+    """Config c2 (B4 C64 T128 H16 Dh64) on the build the library picks for it (a wave owns a whole
+    time step) and on the general kernel: two heads against the oracle, the rest through
     size-independent properties."""
+    kern = getattr(mvpa_hip, kern)
     inp = make_mvpa_inputs(B=4, C=64, T=128, H=16, Dh=64, seed=0, qkv_unit=True).round_to(torch.bfloat16)
     d = inp.to("cuda", torch.bfloat16)
     out = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
-                                kernel=mvpa_hip.KERNEL_MFMA)
+                                kernel=kern)
     heads = [(0, 0), (3, 15)]
     ref = _oracle(inp, dtype=torch.float32, heads=heads, q_block=1024)
     for (b, h) in heads:
         _check_bf16(out[b, h], ref[b, h])
     # V == 1 -> every output is 1 (rows of P sum to one)
     ones = torch.ones_like(d.v)
-    o1 = mvpa_hip.mvpa_forward(d.q, d.k, ones, d.u, d.vb, d.z, d.k_time, d.k_chan).float()
+    o1 = mvpa_hip.mvpa_forward(d.q, d.k, ones, d.u, d.vb, d.z, d.k_time, d.k_chan, kernel=kern).float()
     assert (o1 - 1).abs().max().item() <= 1e-2
     # causality, bit exact: changing the last 16 time steps leaves earlier rows untouched
     k2, v2 = d.k.clone(), d.v.clone()
     k2[:, :, -16 * 64:] *= -1.5
     v2[:, :, -16 * 64:] += 1.0
-    o2 = mvpa_hip.mvpa_forward(d.q, k2, v2, d.u, d.vb, d.z, d.k_time, d.k_chan)
+    o2 = mvpa_hip.mvpa_forward(d.q, k2, v2, d.u, d.vb, d.z, d.k_time, d.k_chan, kernel=kern)
     assert torch.equal(o2[:, :, :-16 * 64], out[:, :, :-16 * 64])
     # agreement with the fp32-math generic kernel on every head
     og = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
@@ -635,7 +724,8 @@ def test_last_step_only_equals_last_rows_of_full_forward(cfg, dtype):
     inp = make_mvpa_inputs(seed=17, qkv_unit=True, **cfg).to("cuda", dtype)
     C = cfg["C"]
     tabs = (inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan)
-    full, lse_full = mvpa_hip.mvpa_forward(inp.q, inp.k, inp.v, *tabs, return_lse=True)
+    kern = mvpa_hip.KERNEL_MFMA if dtype == torch.bfloat16 else mvpa_hip.KERNEL_GENERIC
+    full, lse_full = mvpa_hip.mvpa_forward(inp.q, inp.k, inp.v, *tabs, return_lse=True, kernel=kern)
     q_last = inp.q[:, :, -C:]
     step, lse_step = mvpa_hip.mvpa_forward(q_last, inp.k, inp.v, *tabs, return_lse=True,
                                            last_step_only=True, key_splits=1)
@@ -752,17 +842,20 @@ def test_decoding_step_at_base_model_size_matches_the_full_forward():
     assert ((ring.float() - ref).norm() / ref.norm()).item() <= 5e-3
 
 
-def test_bf16_base_attention_shape_full_size():
-    """The base model's attention at full length (B1 H16 Hkv8 C128 T512 Dh128, the kernel build
-    with one wave on four key tiles): sampled query rows of one head against the oracle - the
-    first steps, a step whose keys are mostly far, the last step - and masks through bit-exact
+@pytest.mark.parametrize("kern", ["KERNEL_AUTO", "KERNEL_MFMA"])
+def test_bf16_base_attention_shape_full_size(kern):
+    """The base model's attention at full length (B1 H16 Hkv8 C128 T512 Dh128) on the build the
+    library picks for it (output columns split over two waves) and on the general kernel (one
+    wave on four key tiles): sampled query rows of one head against the oracle - the first
+    steps, a step whose keys are mostly far, the last step - and masks through bit-exact
     perturbation, as for the irregular-channel configuration."""
+    kern = getattr(mvpa_hip, kern)
     C, T = 128, 512
     inp = make_mvpa_inputs(B=1, C=C, T=T, H=16, Hkv=8, Dh=128, seed=0, qkv_unit=True,
                            validity=True).round_to(torch.bfloat16)
     d = inp.to("cuda", torch.bfloat16)
     out = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
-                                chan_valid=d.chan_valid, kernel=mvpa_hip.KERNEL_MFMA)
+                                chan_valid=d.chan_valid, kernel=kern)
     ranges = [(0, 2 * C), (300 * C, 301 * C), (511 * C, 512 * C)]
     ref = _oracle(inp, dtype=torch.float32, heads=[(0, 11)], q_ranges=ranges, q_block=128)
     live = inp.chan_valid[0][:, None]
@@ -776,11 +869,11 @@ def test_bf16_base_attention_shape_full_size():
     v2 = torch.where(dead, big, d.v.view(1, 8, T, C, 128)).view(1, 8, T * C, 128).clone()
     k2[:, :, -40 * C:] *= -1.5                        # the last 40 steps: hidden from every earlier row
     v2[:, :, -40 * C:] += 1.0
-    o2 = mvpa_hip.mvpa_forward(d.q, k2, v2, d.u, d.vb, d.z, d.k_time, d.k_chan, chan_valid=d.chan_valid)
+    o2 = mvpa_hip.mvpa_forward(d.q, k2, v2, d.u, d.vb, d.z, d.k_time, d.k_chan, chan_valid=d.chan_valid, kernel=kern)
     assert torch.equal(o2[:, :, :-40 * C], out[:, :, :-40 * C])
     # keys of step 0 changed: only rows with tq <= 10 and the last step keep the content term there
     k3 = d.k.clone()
     k3[:, :, :C] += 1.0
-    o3 = mvpa_hip.mvpa_forward(d.q, k3, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, chan_valid=d.chan_valid)
+    o3 = mvpa_hip.mvpa_forward(d.q, k3, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, chan_valid=d.chan_valid, kernel=kern)
     same = (o3 == out).flatten(0, 1).all(-1).view(-1, T, C).all(0).all(-1).cpu()
     assert same.tolist() == [not (t <= 10 or t == T - 1) for t in range(T)]
