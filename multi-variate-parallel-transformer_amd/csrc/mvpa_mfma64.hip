@@ -161,27 +161,23 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
     v_off[i] = (uint32_t)(rowc * a.v_stride_n) * 2u + ((phys ^ swz_v<DH>(row)) << 4);
   }
   const uint32_t ring_lds = (uint32_t)(uintptr_t)(LDS_PTR(unsigned char))smem_raw;
-  // The tiles are requested in stream order - pass A (key steps NLO .. tq_hi, K and V), pass B
-  // (the same again), far phase (key steps 0 .. FM, V only) - by a little scalar state machine
+  // The window tiles are requested in stream order - pass A (key steps NLO .. tq_hi, K and V),
+  // pass B (the same again) - by a little scalar state machine
   // that moves two pointers along, so that a request costs a handful of scalar instructions.
   const int64_t kstep = (int64_t)C_ * a.k_stride_n, vstep = (int64_t)C_ * a.v_stride_n;
   int iss_pos = 0, iss_stage = 0;
   const bf16_t* iss_k = kbase + (n_pass > 0 ? NLO : 0) * kstep;
   const bf16_t* iss_v = vbase + (n_pass > 0 ? NLO : 0) * vstep;
   auto issue_next = [&]() {
-    if (iss_pos >= n_total) return;
+    if (iss_pos >= n_near) return;
     const uint32_t stage = ring_lds + iss_stage * STAGE_BYTES;
 #pragma unroll
     for (int i = 0; i < LPW; ++i) load_to_lds_16(iss_v, v_off[i], stage + TILE_BYTES + (wave + NW * i) * 1024);
-    if (iss_pos < n_near) {
 #pragma unroll
-      for (int i = 0; i < LPW; ++i) load_to_lds_16(iss_k, k_off[i], stage + (wave + NW * i) * 1024);
-    }
+    for (int i = 0; i < LPW; ++i) load_to_lds_16(iss_k, k_off[i], stage + (wave + NW * i) * 1024);
     ++iss_pos;
     iss_stage = iss_stage + 1 == STAGES ? 0 : iss_stage + 1;
-    if (iss_pos == n_near) {                 // the far phase starts at key step 0
-      iss_v = vbase;
-    } else if (iss_pos == n_pass) {          // pass B walks the window once more
+    if (iss_pos == n_pass) {                 // pass B walks the window once more
       iss_k = kbase + NLO * kstep;
       iss_v = vbase + NLO * vstep;
     } else {
@@ -488,14 +484,36 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
     tl.l += ls;
   };
 
-  // wait until the tile of stream position s has landed: at most the loads of the one younger
-  // tile in flight (STAGES = 3) may still be outstanding
-  // wait until the tile of stream position s has landed: at most the loads of the one younger
-  // tile in flight (STAGES = 3) may still be outstanding
+  // wait until the window tile of stream position s has landed: at most the loads of the one
+  // younger tile in flight (STAGES = 3) may still be outstanding
   auto wait_tile = [&](int s) {
     if (s + 1 < n_near) wait_vmcnt_imm<2 * LPW>();
-    else if (s + 1 < n_total) wait_vmcnt_imm<LPW>();
     else wait_vmcnt_imm<0>();
+  };
+
+  // Tile requests of the far phase.  The ring is cut anew into slots of one V tile; far tile f
+  // lives in slot (f0 + f) mod FSLOTS, and the barrier of step f publishes it.  One tile is
+  // requested per step, without a branch: past the end it is the last tile once more, into a slot
+  // nobody reads any longer, so that the count of loads in flight is fixed.
+  constexpr int FSLOTS = RING_BYTES / TILE_BYTES;
+  const bf16_t* fv = vbase;
+  int f_iss = 0;
+  uint32_t iss_lds = ring_lds, cur_lds = ring_lds;       // (f0 = 0 unless the passes say otherwise)
+  auto issue_far = [&]() {
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) load_to_lds_16(fv, v_off[i], iss_lds + (wave + NW * i) * 1024);
+    ++f_iss;
+    fv = f_iss < n_far ? fv + vstep : fv;
+    iss_lds = iss_lds + TILE_BYTES == ring_lds + RING_BYTES ? ring_lds : iss_lds + TILE_BYTES;
+  };
+  auto v_addr_at = [&](uint32_t base) {
+    StageAddr sa;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      sa.v[mt] = base + (v_lane[mt] - TILE_BYTES);
+      asm volatile("" : "+v"(sa.v[mt]));
+    }
+    return sa;
   };
 
   // =========================== passes: window steps, one query tile each ===========================
@@ -516,6 +534,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
       // the next tile is requested after it, not before, or the slab would wait for that tile too)
       if (active && (p == 0 || (tk & 31) == 0)) time_slab(x, x, tk & ~31, false);
       issue_next();
+      if (s + 1 == n_near && n_far > 0) {
+        // the last window tile: the other two stages are free, the first four far tiles go there
+        iss_lds = cur_lds = ring_lds + (stg + 1 == STAGES ? 0 : stg + 1) * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < FSLOTS - 2; ++i) issue_far();
+      }
       if (active && tk >= nlo && tk <= tq && (!last_wg || (tk & 1) == par))
         near_step(qt[x], Bc, Qu, Stb, stage_addr(stg), tk);
       stg = stg + 1 == STAGES ? 0 : stg + 1;
@@ -555,6 +579,15 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
   // The phase goes slab by slab (32 key steps): the slabs of both tiles are computed between two
   // segments, where the products of the far steps are not live, so their registers are free for
   // the slab's operands.
+  if (n_far > 0) {
+    if (n_near > 0) {
+      lds_barrier();                     // every wave is through with the last window tile
+      issue_far();
+    } else {
+#pragma unroll
+      for (int i = 0; i < FSLOTS - 1; ++i) issue_far();
+    }
+  }
   for (int tk0 = 0; tk0 < n_far; tk0 += 32) {
     if (tk0 <= far_max) time_slab(0, 1, tk0, true);   // (never for inactive waves)
     f32x16 ptmp[2][MT];
@@ -567,14 +600,13 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
         for (int i = 0; i < 16; ++i) ptmp[x][mt][i] = 0.f;
     const int tk1 = min(tk0 + 32, n_far);
     for (int tk = tk0; tk < tk1; ++tk) {
-      // every tile in flight during this phase is a V tile
-      if (tk + 1 < n_far) wait_vmcnt_imm<LPW>(); else wait_vmcnt_imm<0>();
+      wait_vmcnt_imm<(FSLOTS - 2) * LPW>();
       lds_barrier();
-      issue_next();
-      const int stg_now = stg;
-      stg = stg + 1 == STAGES ? 0 : stg + 1;
+      issue_far();
+      const uint32_t now_lds = cur_lds;
+      cur_lds = cur_lds + TILE_BYTES == ring_lds + RING_BYTES ? ring_lds : cur_lds + TILE_BYTES;
       if (tk <= far_max) {
-        const StageAddr stage = stage_addr(stg_now);
+        const StageAddr stage = v_addr_at(now_lds);
         const float st0 = stb_wave[(tk & 31) * 32 + ln];
         const float st1 = stb_wave[32 * 32 + (tk & 31) * 32 + ln];
         // Order of a step, pinned for the scheduler: the fragments of output tile 0 are requested
@@ -643,6 +675,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
 #pragma unroll
         for (int i = 0; i < 16; ++i) qt[x].acc[mt][i] += pet[x] * ptmp[x][mt][i];
   }
+
+  wait_vmcnt_imm<0>();                   // (the far requests past the end)
 
   // =========================== epilogue ===========================
 #pragma unroll
