@@ -39,6 +39,17 @@ BF16_DENSE_PEAK_TFLOPS = 2500.0       # MI355X published dense bf16 MFMA peak
 # HBM bytes per launch of the attention kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by
 # what the same counters read for a plain device copy of known size; the profile summary named
 # beside each figure holds the two counter runs.
+MEASURED_TRAFFIC_BYTES = {"c2": (402.4e6, "profiles/mvpa_mfma_kernel_c2.md")}
+PREWARM_LAUNCHES = 150
+
+WORKLOADS = {
+    "c2": dict(B=4, C=64, T=128, H=16, Hkv=16, Dh=64, validity=False),
+    "c3": dict(B=8, C=117, T=256, H=16, Hkv=16, Dh=64, validity=True),
+    # the attention shape inside configuration c5 (the base model: one sample, 128 channels, 512 segments)
+    "c5attn": dict(B=1, C=128, T=512, H=16, Hkv=8, Dh=128, validity=False),
+}
+
+
 def _forward_kernel_name(cfg):
     """The build of the bf16 forward that the library's own choice (MVPA_KERNEL_AUTO) runs for a
     workload: the rule of mvpa_forward in csrc/mvpa_api.hip."""
@@ -47,15 +58,6 @@ def _forward_kernel_name(cfg):
     if cfg["Dh"] == 64 and 32 < cfg["C"] <= 64 and cfg["T"] >= 128:
         return "mvpa::q64::mvpa_mfma64_kernel"
     return "mvpa::mvpa_mfma_kernel"
-
-
-MEASURED_TRAFFIC_BYTES = {"c2": (402.4e6, "profiles/mvpa_mfma_kernel_c2.md")}
-PREWARM_LAUNCHES = 150
-
-WORKLOADS = {
-    "c2": dict(B=4, C=64, T=128, H=16, Hkv=16, Dh=64, validity=False),
-    "c3": dict(B=8, C=117, T=256, H=16, Hkv=16, Dh=64, validity=True),
-}
 
 
 def algorithmic_flops(B, H, T, C, Dh, window=10):

@@ -425,6 +425,29 @@ __device__ inline void dma_to_lds_16(const void* gptr, uint32_t lds_base) {
                :: "v"(gptr), "s"(lds_base) : "memory", "m0");
 }
 
+// Linear workgroup id L -> tile coordinates.  Ids that are equal mod 8 run on one XCD (each has an
+// L2 of its own).  Where the tile rows divide evenly (a multiple of 8 * GM), an XCD is given an
+// eighth of the tile rows and walks it in groups of GM tile rows, column by column: the 32
+// workgroups that an XCD runs side by side then cover GM rows x 32/GM columns of tiles and read
+// GM + 32/GM operand panels between them instead of one panel per workgroup and more.  Otherwise
+// row-major.
+__device__ inline void tile_of_workgroup(int64_t L, int64_t mt, int64_t nt, int64_t* tm, int64_t* tn) {
+  constexpr int GM = 4;
+  int64_t m, n;
+  if (mt % (8 * GM) == 0) {
+    const int64_t xcd = L & 7, s = L >> 3, per = mt / 8;
+    const int64_t g = s / (GM * nt), r = s % (GM * nt);
+    n = r / GM;
+    m = xcd * per + g * GM + r % GM;
+  } else {
+    m = L / nt;
+    n = L % nt;
+  }
+  // (wave-uniform by construction; said so to the compiler, which keeps them in scalar registers)
+  *tm = __builtin_amdgcn_readfirstlane((int)m);
+  *tn = __builtin_amdgcn_readfirstlane((int)n);
+}
+
 template <int BN, int EPI>
 __global__ __launch_bounds__(512) void linear_bf16_big_kernel(const bf16_t* __restrict__ X,
                                                               const bf16_t* __restrict__ W,
@@ -442,12 +465,13 @@ __global__ __launch_bounds__(512) void linear_bf16_big_kernel(const bf16_t* __re
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 31, hh = lane >> 5;
   const int wm = wave >> 1, wc = wave & 1;
-  const int64_t m0 = (int64_t)blockIdx.y * BM;
   constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;    // output columns per workgroup
-  const int64_t n0 = (int64_t)blockIdx.x * OUT_COLS;
+  const int64_t mt = (M + BM - 1) / BM, nt = (N + OUT_COLS - 1) / OUT_COLS;
 
-  // which w row feeds tile row r
-  auto w_row = [&](int r) -> int64_t {
+  int64_t m0 = 0, n0 = 0;                             // first x row / output column of the tile
+  const bf16_t* asrc[A_LOADS];
+  const bf16_t* bsrc[B_LOADS];
+  auto w_row = [&](int r) -> int64_t {                // which w row feeds tile row r
     if (EPI == 1) {
       const int wcol = r / WN, nb = (r % WN) / 32, i = r & 31;
       const int64_t col = n0 + wcol * (WN / 2) + (nb >> 1) * 32 + i;
@@ -456,12 +480,12 @@ __global__ __launch_bounds__(512) void linear_bf16_big_kernel(const bf16_t* __re
     const int64_t n = n0 + r;
     return n < N ? n : N - 1;
   };
-
   // per-lane source rows of this wave's loads (row clamped into range: such rows are never stored)
-  const bf16_t* asrc[A_LOADS];
-  const bf16_t* bsrc[B_LOADS];
-  int chunk_k;                                        // logical 16-byte chunk (x8 elements) per lane
-  {
+  auto set_tile = [&](int64_t L) {
+    int64_t tile_m, tile_n;
+    tile_of_workgroup(L, mt, nt, &tile_m, &tile_n);
+    m0 = tile_m * BM;
+    n0 = tile_n * OUT_COLS;
     const int rsub = lane >> 3, phys = lane & 7;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
@@ -474,49 +498,36 @@ __global__ __launch_bounds__(512) void linear_bf16_big_kernel(const bf16_t* __re
       const int row = (wave * B_LOADS + i) * 8 + rsub;
       bsrc[i] = W + w_row(row) * ldw + ((phys ^ ((row >> 1) & 7)) << 3);
     }
-    // all rows of one wave load share (row>>1)&7 pattern per lane only through rsub: recompute
-    chunk_k = 0;   // placeholder, the k offset of a lane is folded into the pointers above
-  }
+  };
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)gsm;
   auto issue = [&](int kt, int stage) {
     const int64_t k0 = (int64_t)kt * BK;
     const uint32_t base = lds0 + stage * STAGE;
-    const bool full = k0 + BK <= K;
+    if (k0 + BK <= K) {                               // (uniform) a whole k-block: nothing but the loads
+#pragma unroll
+      for (int i = 0; i < A_LOADS; ++i) dma_to_lds_16(asrc[i] + k0, base + (wave * A_LOADS + i) * 1024);
+#pragma unroll
+      for (int i = 0; i < B_LOADS; ++i) dma_to_lds_16(bsrc[i] + k0, base + A_BYTES + (wave * B_LOADS + i) * 1024);
+      return;
+    }
+    // the tail block of K: chunks past the end are zero-filled
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
       const uint32_t dst = base + (wave * A_LOADS + i) * 1024;
-      const bf16_t* src = asrc[i] + k0;
-      if (full) {
-        dma_to_lds_16(src, dst);
-      } else {
-        const int row = (wave * A_LOADS + i) * 8 + (lane >> 3);
-        const int64_t kk = k0 + (((lane & 7) ^ ((row >> 1) & 7)) << 3);
-        if (kk < K) dma_to_lds_16(src, dst);
-        else *(u32x4*)(gsm + (dst - lds0) + lane * 16) = u32x4{0u, 0u, 0u, 0u};
-      }
+      const int row = (wave * A_LOADS + i) * 8 + (lane >> 3);
+      const int64_t kk = k0 + (((lane & 7) ^ ((row >> 1) & 7)) << 3);
+      if (kk < K) dma_to_lds_16(asrc[i] + k0, dst);
+      else *(u32x4*)(gsm + (dst - lds0) + lane * 16) = u32x4{0u, 0u, 0u, 0u};
     }
 #pragma unroll
     for (int i = 0; i < B_LOADS; ++i) {
       const uint32_t dst = base + A_BYTES + (wave * B_LOADS + i) * 1024;
-      const bf16_t* src = bsrc[i] + k0;
-      if (full) {
-        dma_to_lds_16(src, dst);
-      } else {
-        const int row = (wave * B_LOADS + i) * 8 + (lane >> 3);
-        const int64_t kk = k0 + (((lane & 7) ^ ((row >> 1) & 7)) << 3);
-        if (kk < K) dma_to_lds_16(src, dst);
-        else *(u32x4*)(gsm + (dst - lds0) + lane * 16) = u32x4{0u, 0u, 0u, 0u};
-      }
+      const int row = (wave * B_LOADS + i) * 8 + (lane >> 3);
+      const int64_t kk = k0 + (((lane & 7) ^ ((row >> 1) & 7)) << 3);
+      if (kk < K) dma_to_lds_16(bsrc[i] + k0, dst);
+      else *(u32x4*)(gsm + (dst - lds0) + lane * 16) = u32x4{0u, 0u, 0u, 0u};
     }
   };
-
-  f32x16 acc[NB][2];
-#pragma unroll
-  for (int i = 0; i < NB; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   // loop-invariant fragment offsets: row ln of a 32-row block, chunk (2ks+hh) ^ swizzle(ln)
   int frag_off[4];
@@ -524,71 +535,97 @@ __global__ __launch_bounds__(512) void linear_bf16_big_kernel(const bf16_t* __re
   for (int ks = 0; ks < 4; ++ks) frag_off[ks] = ln * ROWB + (((2 * ks + hh) ^ ((ln >> 1) & 7)) << 4);
 
   const int nkt = (int)((K + BK - 1) / BK);
-  issue(0, 0);
-  for (int kt = 0; kt < nkt; ++kt) {
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    if (kt + 1 < nkt) issue(kt + 1, (kt + 1) & 1);
-    const unsigned char* sa = gsm + (kt & 1) * STAGE + (wm * 64) * ROWB;
-    const unsigned char* sb = gsm + (kt & 1) * STAGE + A_BYTES + (wc * WN) * ROWB;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      bf16x8 xf[2], wf[NB];
-#pragma unroll
-      for (int j = 0; j < 2; ++j) xf[j] = *(const bf16x8*)(sa + j * 32 * ROWB + frag_off[ks]);
-#pragma unroll
-      for (int i = 0; i < NB; ++i) wf[i] = *(const bf16x8*)(sb + i * 32 * ROWB + frag_off[ks]);
-#pragma unroll
-      for (int i = 0; i < NB; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[i], xf[j], acc[i][j], 0, 0, 0);
-    }
-  }
-
-  // epilogue: lane = x row (ln) of block j; accumulator quad a4 = w rows 8*a4 + 4*hh + 0..3
   typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+  int stage = 0;                                      // ring stage of the k-block to multiply next
+  set_tile(blockIdx.x);
+  issue(0, 0);
+  {
+    const int64_t cm0 = m0, cn0 = n0;
+    f32x16 acc[NB][2];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int64_t m = m0 + wm * 64 + j * 32 + ln;
-    if (m >= M) continue;
-    bf16_t* yrow = Y + m * ldy;
-    if (EPI == 1) {
+    for (int i = 0; i < NB; ++i)
 #pragma unroll
-      for (int p = 0; p < NB / 2; ++p)
+      for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4) {
-          const int64_t n = n0 + wc * (WN / 2) + p * 32 + a4 * 8 + hh * 4;
-          bf16x4 o;
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    for (int kt = 0; kt < nkt; ++kt) {
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      const unsigned char* sa = gsm + stage * STAGE + (wm * 64) * ROWB;
+      const unsigned char* sb = gsm + stage * STAGE + A_BYTES + (wc * WN) * ROWB;
+      // the first fragments are requested before the next block's loads, whose issue covers their
+      // latency; inside the block the fragments of k-step s+1 are requested before the products of s
+      bf16x8 xf[2][2], wf[2][NB];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float gte = acc[2 * p][j][a4 * 4 + r], up = acc[2 * p + 1][j][a4 * 4 + r];
-            o[r] = (__bf16)(gte / (1.f + __expf(-gte)) * up);
-          }
-          if (n + 3 < N) {
-            *(bf16x4*)(yrow + n) = o;
-          } else {
+      for (int j = 0; j < 2; ++j) xf[0][j] = *(const bf16x8*)(sa + j * 32 * ROWB + frag_off[0]);
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (n + r < N) ((__bf16*)yrow)[n + r] = o[r];
-          }
+      for (int i = 0; i < NB; ++i) wf[0][i] = *(const bf16x8*)(sb + i * 32 * ROWB + frag_off[0]);
+      __builtin_amdgcn_sched_barrier(0);
+      if (kt + 1 < nkt) issue(kt + 1, stage ^ 1);
+      stage ^= 1;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int cur = ks & 1, nxt = cur ^ 1;
+        if (ks + 1 < 4) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) xf[nxt][j] = *(const bf16x8*)(sa + j * 32 * ROWB + frag_off[ks + 1]);
+#pragma unroll
+          for (int i = 0; i < NB; ++i) wf[nxt][i] = *(const bf16x8*)(sb + i * 32 * ROWB + frag_off[ks + 1]);
         }
-    } else {
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < NB; ++i)
+        for (int i = 0; i < NB; ++i)
 #pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4) {
-          const int64_t n = n0 + wc * WN + i * 32 + a4 * 8 + hh * 4;
-          bf16x4 o;
+          for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[cur][i], xf[cur][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+
+    // epilogue: lane = x row (ln) of block j; accumulator quad a4 = w rows 8*a4 + 4*hh + 0..3
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][a4 * 4 + r];
-          if (n + 3 < N) {
-            *(bf16x4*)(yrow + n) = o;
-          } else {
+    for (int j = 0; j < 2; ++j) {
+      const int64_t m = cm0 + wm * 64 + j * 32 + ln;
+      if (m >= M) continue;
+      bf16_t* yrow = Y + m * ldy;
+      if (EPI == 1) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (n + r < N) ((__bf16*)yrow)[n + r] = o[r];
+        for (int p = 0; p < NB / 2; ++p)
+#pragma unroll
+          for (int a4 = 0; a4 < 4; ++a4) {
+            const int64_t n = cn0 + wc * (WN / 2) + p * 32 + a4 * 8 + hh * 4;
+            bf16x4 o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float gte = acc[2 * p][j][a4 * 4 + r], up = acc[2 * p + 1][j][a4 * 4 + r];
+              o[r] = (__bf16)(gte / (1.f + __expf(-gte)) * up);
+            }
+            if (n + 3 < N) {
+              *(bf16x4*)(yrow + n) = o;
+            } else {
+#pragma unroll
+              for (int r = 0; r < 4; ++r)
+                if (n + r < N) ((__bf16*)yrow)[n + r] = o[r];
+            }
           }
-        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+#pragma unroll
+          for (int a4 = 0; a4 < 4; ++a4) {
+            const int64_t n = cn0 + wc * WN + i * 32 + a4 * 8 + hh * 4;
+            bf16x4 o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][a4 * 4 + r];
+            if (n + 3 < N) {
+              *(bf16x4*)(yrow + n) = o;
+            } else {
+#pragma unroll
+              for (int r = 0; r < 4; ++r)
+                if (n + r < N) ((__bf16*)yrow)[n + r] = o[r];
+            }
+          }
+      }
     }
   }
 }
@@ -600,7 +637,7 @@ static int launch_big(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, in
   auto kern = linear_bf16_big_kernel<BN, EPI>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
   constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;
-  dim3 grid((unsigned)((N + OUT_COLS - 1) / OUT_COLS), (unsigned)((M + 255) / 256));
+  dim3 grid((unsigned)(((N + OUT_COLS - 1) / OUT_COLS) * ((M + 255) / 256)));
   MVPA_LAUNCH(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
