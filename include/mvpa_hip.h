@@ -61,7 +61,7 @@ enum {
                                is off, where it is the faster one.                         */
   MVPA_KERNEL_MFMA_SPLIT = 4 /* the build in which the output columns of a query tile are split
                                over two waves (head size 128, 65..128 channels, plain
-                               forward); error if the shape is unsupported.  AUTO picks it
+                               forward, bf16 or fp8 content term); error if unsupported.  AUTO picks it
                                for every such shape.                                       */
 };
 

@@ -45,7 +45,7 @@ __device__ inline void wait_units(int n) {            // at most n * U loads of 
   else wait_vmcnt_imm<3 * U>();
 }
 
-template <int NCT>
+template <int NCT, bool FP8>
 __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) {
   using G = Geo<NCT>;
   constexpr int TILE_BYTES = G::TILE_BYTES, LPW = G::LPW, RING_BYTES = G::RING_BYTES;
@@ -253,8 +253,19 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
   // Bc[ck][q] = (q+z).e[C-1-|cq-ck|] * scale in accumulator layout (-inf = masked key) and the
   // (q+u) fragments.  The whole channel table (every distance) goes through the wave's scratch,
   // which is its eighth of the ring: no tile is requested before every wave is through.
+  // fp8 content term (FP8): q' = (q+u)*scale/sq and k' = k/sk are rounded to e4m3 with the
+  // per-head amax scales sq, sk chosen by the caller; the MFMA accumulates in units of 1/(sq*sk),
+  // the channel-bias tile is pre-divided accordingly for the window steps and the product sq*sk
+  // returns inside the exp2 fma.  K is converted on the fly from the bf16 tile.
   f32x16 Bc[NCT];
   bf16x8 Qu[KS];
+  long Qu8[KS];
+  float fp8_d = 1.f, fp8_inv_sk = 1.f;
+  if (FP8) {
+    const float sq = a.fp8_q_scale[h], sk = a.fp8_k_scale[g];
+    fp8_d = sq * sk;
+    fp8_inv_sk = 1.f / sk;
+  }
   {
     f32x16 sct[NCT];
 #pragma unroll
@@ -270,7 +281,8 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
       for (int k4 = 0; k4 < 4; ++k4) {
         const int ks = kh + k4;
         const int d0 = ks * 16 + hh * 8;
-        Qu[ks] = make_qfrag(raw[k4], bu + d0, sc2);
+        if (FP8) Qu8[ks] = make_qfrag_fp8(raw[k4], bu + d0, sc2 / a.fp8_q_scale[h]);
+        else Qu[ks] = make_qfrag(raw[k4], bu + d0, sc2);
         const bf16x8 qz = make_qfrag(raw[k4], bz + d0, sc2);
 #pragma unroll
         for (int t = 0; t < NCT; ++t) {
@@ -313,7 +325,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
         const uint32_t dist = min(max(cq4, ci4) - min(cq4, ci4), (uint32_t)(C_ - 1));
         const float val = *(const float*)(scr_b + (gbase - (int)(dist * 128u)));
         const bool kv = (kbits[t] >> ((i >> 2) * 8 + (i & 3))) & 1u;
-        Bc[t][i] = kv ? val : -INFINITY;
+        Bc[t][i] = kv ? (FP8 ? val * (1.f / fp8_d) : val) : -INFINITY;
       }
   }
   lds_barrier();               // the scratch is ring memory from here on
@@ -380,12 +392,21 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
     float ls = 0.f;
 #pragma unroll
     for (int t = 0; t < NCT; ++t) {
-      bf16x8 ka[KS];
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ka[ks] = k_frag(ka_, t, ks);
       f32x16 S = Bc[t];
+      if (FP8) {
+        u32x4 kr[KS];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], Qu[ks], S, 0, 0, 0);
+        for (int ks = 0; ks < KS; ++ks) kr[ks] = *(LDS_PTR(const u32x4))(uintptr_t)(ka_.k[ks] + t * 32 * ROWB);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          S = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(kfrag_fp8(kr[ks], fp8_inv_sk), Qu8[ks], S, 0, 0, 0);
+      } else {
+        bf16x8 ka[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) ka[ks] = k_frag(ka_, t, ks);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], Qu[ks], S, 0, 0, 0);
+      }
       bf16x8 vf[2][MT];
 #pragma unroll
       for (int s = 0; s < 2; ++s)
@@ -395,6 +416,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
 #pragma unroll
       for (int i = 0; i < 16; ++i) rmax = fmaxf(rmax, S[i]);
       rmax = xhalf_max(rmax);
+      if (FP8) rmax *= fp8_d;
       const float cand = rmax + st;
       if (__ballot(cand > m_run + 8.f) != 0ull) {
         const float m_new = fmaxf(m_run, cand);
@@ -406,7 +428,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
       }
       const float off = st - m_run;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) S[i] = fast_exp2(S[i] + off);
+      for (int i = 0; i < 16; ++i) S[i] = FP8 ? fast_exp2(__builtin_fmaf(S[i], fp8_d, off)) : fast_exp2(S[i] + off);
       bf16x8 P[2];
       P[0] = pack8(S, 0);
       P[1] = pack8(S, 8);
@@ -448,6 +470,12 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
   bf16x8 Ec[NCT][2];
   float sumEc = 0.f;
   {
+    if (FP8) {                                 // back to the units of the scores
+#pragma unroll
+      for (int k = 0; k < NCT; ++k)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) Bc[k][i] *= fp8_d;
+    }
     float mx = -INFINITY;
 #pragma unroll
     for (int k = 0; k < NCT; ++k)
@@ -606,23 +634,25 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
 }  // namespace mvpa
 
 // Shapes the column-split kernel serves: bf16, head size 128, 65..128 channels, a plain forward
-// (no decoding step, no fp8 content term); everything else about the arguments is as for the
-// general kernel (mvpa_mfma_supported).
+// (no decoding step), bf16 or fp8 content term; everything else about the arguments is as for
+// the general kernel (mvpa_mfma_supported).
 int mvpa_mfma128_supported(const mvpa_fwd_args* a) {
   if (a->Dh != 128 || a->C <= 64 || a->C > 128) return 0;
-  if (a->flags & (MVPA_FLAG_LAST_STEP | MVPA_FLAG_RING | MVPA_FLAG_FP8_QK)) return 0;
+  if (a->flags & (MVPA_FLAG_LAST_STEP | MVPA_FLAG_RING)) return 0;
   return 1;
 }
 
-template <int NCT>
+template <int NCT, bool FP8>
 static int launch128(const mvpa_fwd_args* a, hipStream_t stream) {
   using namespace mvpa::d128;
   using G = Geo<NCT>;
-  (void)hipFuncSetAttribute((const void*)mvpa_mfma128_kernel<NCT>, hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
-  MVPA_LAUNCH(mvpa_mfma128_kernel<NCT>, dim3((unsigned)(a->T * a->B * a->H)), dim3(NW * 64), G::LDS_BYTES, stream, *a);
+  auto kern = mvpa_mfma128_kernel<NCT, FP8>;
+  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
+  MVPA_LAUNCH(kern, dim3((unsigned)(a->T * a->B * a->H)), dim3(NW * 64), G::LDS_BYTES, stream, *a);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 
 int mvpa_launch_mfma128(const mvpa_fwd_args* a, hipStream_t stream) {
-  return a->C <= 96 ? launch128<3>(a, stream) : launch128<4>(a, stream);
+  if (a->flags & MVPA_FLAG_FP8_QK) return a->C <= 96 ? launch128<3, true>(a, stream) : launch128<4, true>(a, stream);
+  return a->C <= 96 ? launch128<3, false>(a, stream) : launch128<4, false>(a, stream);
 }

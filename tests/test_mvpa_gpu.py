@@ -699,6 +699,33 @@ def test_fp8_qk_within_stated_tolerance(cfg):
     assert err <= tol["max_abs"] and rel <= tol["rel_l2"], f"max-abs {err:.3e}, rel-L2 {rel:.3e}"
 
 
+@pytest.mark.parametrize("cfg", [
+    dict(B=1, C=128, T=26, H=2, Dh=128, Hkv=1, qkv_unit=False, table_std=0.3),             # far steps too
+    dict(B=1, C=100, T=24, H=4, Dh=128, Hkv=2, qkv_unit=True, table_std=0.3, validity=True),
+    dict(B=2, C=80, T=9, H=2, Dh=128, qkv_unit=False, table_std=0.3),                      # window steps only
+])
+def test_fp8_qk_on_the_column_split_build(cfg):
+    """The fp8 content term on the build with the output columns split over two waves (the
+    library's choice for head size 128 with 65..128 channels): the same stated tolerance against
+    the oracle as on the general kernel, and agreement with the general kernel's fp8 result to
+    bf16 rounding (both round the same q' and k' to e4m3)."""
+    inp = make_mvpa_inputs(seed=33, **cfg).round_to(torch.bfloat16)
+    ref = _oracle(inp).float()
+    o8 = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA_SPLIT, fp8_qk=True).float().cpu()
+    o16 = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA_SPLIT).float().cpu()
+    og8 = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA, fp8_qk=True).float().cpu()
+    auto8 = _gpu(inp, torch.bfloat16, fp8_qk=True).float().cpu()
+    assert not torch.equal(o8, o16)                     # the fp8 path really ran
+    assert torch.equal(auto8, o8)                       # and it is the build the library picks
+    B, T, C = cfg["B"], cfg["T"], cfg["C"]
+    live = torch.ones_like(o8[..., :1]) if inp.chan_valid is None else \
+        inp.chan_valid[:, None, None, :, None].expand(B, 1, T, C, 1).reshape(B, 1, -1, 1).float()
+    err, rel = ((o8 - ref) * live).abs().max().item(), _rel_l2(o8 * live, ref * live)
+    tol = FP8_TOL[cfg["qkv_unit"]]
+    assert err <= tol["max_abs"] and rel <= tol["rel_l2"], f"max-abs {err:.3e}, rel-L2 {rel:.3e}"
+    assert ((o8 - og8) * live).abs().max().item() <= 2e-2
+
+
 def test_fp8_needs_mfma_kernel():
     inp = make_mvpa_inputs(B=1, C=4, T=6, H=1, Dh=32, seed=1)
     d = inp.to("cuda", torch.float32)
