@@ -42,7 +42,9 @@ enum {
 /* ---- element types ----------------------------------------------------------------- */
 enum {
   MVPA_F32 = 0,   /* fp32 in, fp32 math, fp32 out                                   */
-  MVPA_BF16 = 1   /* bf16 in/out, bf16 MFMA with fp32 accumulation                  */
+  MVPA_BF16 = 1,  /* bf16 in/out, bf16 MFMA with fp32 accumulation                  */
+  MVPA_F16 = 2    /* fp16 in/out, fp32 math: forward only, on the row-per-lane kernel
+                     (the reference's kernel takes fp16 or bf16, attentions/attn.py:1064-1066) */
 };
 
 /* ---- kernel selector --------------------------------------------------------------- */
@@ -61,8 +63,8 @@ enum {
                                is off, where it is the faster one.                         */
   MVPA_KERNEL_MFMA_SPLIT = 4 /* the build in which the output columns of a query tile are split
                                over two waves (head size 128, 65..128 channels, plain
-                               forward, bf16 or fp8 content term); error if unsupported.  AUTO picks it
-                               for every such shape.                                       */
+                               forward, bf16 or fp8 content term); error if the shape is
+                               unsupported.  AUTO picks it for every such shape.           */
 };
 
 /* ---- flags ------------------------------------------------------------------------- */
@@ -103,7 +105,7 @@ enum {
  */
 typedef struct mvpa_fwd_args {
   uint32_t struct_size;   /* sizeof(mvpa_fwd_args)                                     */
-  int32_t dtype;          /* MVPA_F32 | MVPA_BF16                                      */
+  int32_t dtype;          /* MVPA_F32 | MVPA_BF16 | MVPA_F16                           */
   int32_t kernel;         /* MVPA_KERNEL_*                                             */
   uint32_t flags;         /* MVPA_FLAG_*                                               */
   int32_t B, H, Hkv, T, C, Dh;

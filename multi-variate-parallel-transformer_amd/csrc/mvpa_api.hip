@@ -27,7 +27,7 @@ extern "C" const char* mvpa_error_string(int status) {
 extern "C" int mvpa_validate(const mvpa_fwd_args* a) {
   if (!a) return MVPA_ERR_NULL;
   if (a->struct_size != sizeof(mvpa_fwd_args)) return MVPA_ERR_STRUCT;
-  if (a->dtype != MVPA_F32 && a->dtype != MVPA_BF16) return MVPA_ERR_DTYPE;
+  if (a->dtype != MVPA_F32 && a->dtype != MVPA_BF16 && a->dtype != MVPA_F16) return MVPA_ERR_DTYPE;
   if (a->kernel < MVPA_KERNEL_AUTO || a->kernel > MVPA_KERNEL_MFMA_SPLIT) return MVPA_ERR_DTYPE;
   if (a->Dh != 16 && a->Dh != 32 && a->Dh != 64 && a->Dh != 128) return MVPA_ERR_HEAD_DIM;
   if (a->B <= 0 || a->H <= 0 || a->Hkv <= 0) return MVPA_ERR_SHAPE;

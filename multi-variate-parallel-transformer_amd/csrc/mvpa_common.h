@@ -64,6 +64,11 @@ template <> struct io<bf16_t> {
   __device__ static inline float load(const bf16_t* p) { return bf16_to_f32(*p); }
   __device__ static inline void store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
 };
+typedef _Float16 f16_t;            // IEEE half as a storage type
+template <> struct io<f16_t> {
+  __device__ static inline float load(const f16_t* p) { return (float)*p; }
+  __device__ static inline void store(f16_t* p, float v) { *p = (f16_t)v; }
+};
 
 constexpr float kLog2e = 1.4426950408889634f;
 

@@ -217,6 +217,7 @@ static int launch_generic_dh(const mvpa_fwd_args* a, hipStream_t stream) {
 int mvpa_launch_generic(const mvpa_fwd_args* a, hipStream_t stream) {
   if (a->dtype == MVPA_F32) return mvpa::launch_generic_dh<float>(a, stream);
   if (a->dtype == MVPA_BF16) return mvpa::launch_generic_dh<mvpa::bf16_t>(a, stream);
+  if (a->dtype == MVPA_F16) return mvpa::launch_generic_dh<mvpa::f16_t>(a, stream);
   return MVPA_ERR_DTYPE;
 }
 

@@ -15,7 +15,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmvpa_hip.so")
 
-MVPA_F32, MVPA_BF16 = 0, 1
+MVPA_F32, MVPA_BF16, MVPA_F16 = 0, 1, 2
 KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA, KERNEL_MFMA_STEP, KERNEL_MFMA_SPLIT = 0, 1, 2, 3, 4
 FLAG_LAST_STEP = 32
 FLAG_RING = 64
@@ -157,7 +157,9 @@ def _dtype_code(dt: torch.dtype) -> int:
         return MVPA_F32
     if dt == torch.bfloat16:
         return MVPA_BF16
-    raise TypeError(f"libmvpa_hip supports float32 and bfloat16, got {dt}")
+    if dt == torch.float16:
+        return MVPA_F16
+    raise TypeError(f"libmvpa_hip supports float32, bfloat16 and float16, got {dt}")
 
 
 def _need_cuda(*tensors) -> None:

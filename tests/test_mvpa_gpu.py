@@ -159,6 +159,23 @@ def test_masks_are_exact_under_perturbation():
 # tiled bf16 MFMA kernel
 # ------------------------------------------------------------------------------------------
 
+@pytest.mark.parametrize("cfg", [dict(B=2, C=8, T=32, H=4, Dh=32), dict(B=1, C=20, T=14, H=2, Hkv=1, Dh=64, validity=True),
+                                 dict(B=1, C=5, T=13, H=2, Dh=128)])
+def test_fp16_io_on_the_fp32_math_kernel(cfg):
+    """fp16 tensors (the reference's kernel takes fp16 or bf16, attentions/attn.py:1064-1066) run
+    on the fp32-math kernel: inputs rounded to fp16, fp32 arithmetic, one rounding of the output.
+    Tolerance: max-abs 2e-3 against the oracle on the same rounded inputs; the log-sum-exp 1e-4."""
+    inp = make_mvpa_inputs(seed=5, table_std=0.3, qkv_unit=True, **cfg).round_to(torch.float16)
+    out, lse = _gpu(inp, torch.float16, return_lse=True)
+    assert out.dtype == torch.float16
+    ref, ref_lse = _oracle(inp, return_lse=True)
+    assert (out.float().cpu().double() - ref).abs().max().item() <= 2e-3
+    assert (lse.cpu().double() - ref_lse).abs().max().item() <= 1e-4
+    d = inp.to("cuda", torch.float16)
+    with pytest.raises(mvpa_hip.MvpaError):            # no matrix-core build for fp16
+        mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, kernel=mvpa_hip.KERNEL_MFMA)
+
+
 MFMA_SHAPES = [
     dict(B=1, C=8, T=32, H=2, Dh=32),                              # c1's grid, padded 8 -> 32
     dict(B=2, C=64, T=16, H=2, Dh=64),                             # one wave per time step
