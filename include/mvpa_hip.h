@@ -61,10 +61,11 @@ enum {
                                whatever the length; error if the shape is unsupported.  AUTO
                                picks it for 128 time steps and more or when the content term
                                is off, where it is the faster one.                         */
-  MVPA_KERNEL_MFMA_SPLIT = 4 /* the build in which the output columns of a query tile are split
-                               over two waves (head size 128, 65..128 channels, plain
-                               forward, bf16 or fp8 content term); error if the shape is
-                               unsupported.  AUTO picks it for every such shape.           */
+  MVPA_KERNEL_MFMA_SPLIT = 4 /* the build for 65..128 channels (plain forward, bf16 or fp8
+                               content term): at head size 128 the output columns of a query
+                               tile are split over two waves, at head size 64 a workgroup
+                               takes two time steps; error if the shape is unsupported.  AUTO
+                               picks it for every such shape.                              */
 };
 
 /* ---- flags ------------------------------------------------------------------------- */

@@ -102,8 +102,11 @@ extern "C" int mvpa_forward(const mvpa_fwd_args* a, void* stream) {
     if (a->kernel == MVPA_KERNEL_MFMA_SPLIT) return mvpa_launch_mfma128(a, st);
     if (a->kernel == MVPA_KERNEL_MFMA) return mvpa_launch_mfma(a, st);
     // AUTO: the specialised builds where they are the faster ones.
-    // Head size 128, 65..128 channels: the column-split build wins at every length measured
-    // (B1 H16 C128: T 16 .. 1024, 13 .. 20 % less time than the general kernel; C 80 .. 100: 21 .. 40 %).
+    // 65..128 channels at head size 64 or 128: the build of csrc/mvpa_mfma128.hip wins at every
+    // length and channel count measured (Dh 128, B1 H16: C128 T 16 .. 1024 13 .. 20 % less time than
+    // the general kernel, C 80 .. 100 21 .. 40 %; Dh 64, H16: B8 C117 T256 11.14 -> 8.58 ms,
+    // B4 C128 T128 1.86 -> 1.34, B4 C80 T128 1.78 -> 1.21, B8 C128 T32 0.53 -> 0.38, B2 C128 T512
+    // 9.99 -> 7.66 ms).
     if (mvpa_mfma128_supported(a)) return mvpa_launch_mfma128(a, st);
     // Head size 64, 33..64 channels: the whole-time-step build pays for its window passes with a
     // cheaper far phase; against the general kernel it loses at 64 time steps (B4 H12 C64: 0.131

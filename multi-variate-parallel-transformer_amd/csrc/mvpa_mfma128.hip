@@ -1,14 +1,19 @@
-// bf16 MFMA forward for head size 128 and 65..128 channels (gfx950, wave64): the output columns of
-// a query tile are split over two waves.
+// bf16 MFMA forward for 65..128 channels at head size 128 or 64 (gfx950, wave64): a wave owns one
+// tile of 32 queries and 64 output columns.
 //
-// The general tiled kernel (mvpa_mfma.hip) gives a wave one tile of 32 queries and all 128 output
-// columns: 64 accumulator registers, 64 more for the product of a far step, the channel-bias tile
-// and the (q+u) fragments - it only fits at one wave per SIMD, and there every wait (an LDS read,
-// the barrier, a dependent matrix instruction) idles the matrix pipe.  Here a wave owns 32 queries
-// x 64 output columns.  A workgroup is one time step: 8 waves = (up to) 4 query tiles x 2 column
-// halves, two waves per SIMD.  The two waves of a query tile compute the same scores and the same
-// soft-max state (nothing is exchanged between them) and differ only in the V^T fragments they
-// read and the columns they write.
+// Head size 128: the general tiled kernel (mvpa_mfma.hip) gives a wave one tile of 32 queries and
+// all 128 output columns: 64 accumulator registers, 64 more for the product of a far step, the
+// channel-bias tile and the (q+u) fragments - it only fits at one wave per SIMD, and there every
+// wait (an LDS read, the barrier, a dependent matrix instruction) idles the matrix pipe.  Here the
+// output columns of a query tile are split over two waves: a workgroup is one time step, 8 waves
+// = (up to) 4 query tiles x 2 column halves, two waves per SIMD.  The two waves of a query tile
+// compute the same scores and the same soft-max state (nothing is exchanged between them) and
+// differ only in the V^T fragments they read and the columns they write.
+//
+// Head size 64: a wave owns every output column of its tile, and the 8 waves of a workgroup are
+// the 4 query tiles of TWO consecutive time steps on one K/V ring (the general kernel instead
+// splits the keys of a step over two waves, each with half the products per key step and a merge
+// at the end).  The keys are padded to 128 channels.
 //
 // The key steps are taken window steps first, far steps after (the online soft-max does not care
 // about the order): the channel-bias tile Bc and the (q+u) fragments are live only in the window
@@ -22,19 +27,24 @@
 namespace mvpa {
 namespace d128 {
 
-constexpr int DH = 128, KS = 8, MT = 2, NW = 8, SLOTS = 4;
-constexpr int ROWB = DH * 2, CHUNKS = DH / 8;
+constexpr int MT = 2, NW = 8, SLOTS = 4;                // a wave owns 64 output columns
 constexpr int STB_WAVE = 32 * 32 * 4;                  // time-bias slab of a wave's query tile
 
-template <int NCT>
+template <int DH, int NCT>
 struct Geo {
+  static constexpr int KS = DH / 16, ROWB = DH * 2, CHUNKS = DH / 8;
+  static constexpr int HALVES = DH / 64;               // waves per query tile (column halves)
+  static constexpr int TQW = 2 / HALVES;               // time steps per workgroup
   static constexpr int CP = 32 * NCT;                  // channels, padded
   static constexpr int TILE_BYTES = CP * ROWB;         // one K or V tile
   static constexpr int LPW = TILE_BYTES / 1024 / NW;   // 64-lane x 16-byte loads per tile and wave
   static constexpr int RING_BYTES = SLOTS * TILE_BYTES;
-  static constexpr int LDS_BYTES = RING_BYTES + NW * STB_WAVE;
+  static constexpr int SCRATCH_WAVE = CP * 32 * 4;     // set-up scratch [CP][32] of a wave
+  // the scratch lies over the ring and the slabs (both are idle during the set-up)
+  static constexpr int LDS_BYTES = RING_BYTES + NW * STB_WAVE > NW * SCRATCH_WAVE ? RING_BYTES + NW * STB_WAVE
+                                                                                   : NW * SCRATCH_WAVE;
+  static_assert(DH == 64 || DH == 128, "head size 64 or 128");
   static_assert(LPW * 1024 * NW == TILE_BYTES, "a tile is a whole number of loads per wave");
-  static_assert(RING_BYTES / NW == CP * 32 * 4, "the set-up scratch [CP][32] of a wave is its eighth of the ring");
 };
 
 template <int U>
@@ -45,15 +55,18 @@ __device__ inline void wait_units(int n) {            // at most n * U loads of 
   else wait_vmcnt_imm<3 * U>();
 }
 
-template <int NCT, bool FP8>
+template <int DH, int NCT, bool FP8>
 __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) {
-  using G = Geo<NCT>;
+  using G = Geo<DH, NCT>;
   constexpr int TILE_BYTES = G::TILE_BYTES, LPW = G::LPW, RING_BYTES = G::RING_BYTES;
+  constexpr int KS = G::KS, ROWB = G::ROWB, CHUNKS = G::CHUNKS, HALVES = G::HALVES, TQW = G::TQW;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 31, hh = lane >> 5;
-  const int qi = wave >> 1, half = wave & 1;        // query tile and column half of this wave
+  // query tile, column half and time step (within the workgroup) of this wave
+  const int qi = HALVES == 2 ? wave >> 1 : wave & 3, half = HALVES == 2 ? wave & 1 : 0;
+  const int ts = HALVES == 2 ? 0 : wave >> 2;
   const int C_ = a.C, W = a.window, T_ = a.T;
   const bool has_content = a.flags & MVPA_FLAG_CONTENT;
   const bool has_time = a.flags & MVPA_FLAG_TIME_BIAS;
@@ -64,16 +77,16 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
   // first (with the content term on it keeps that term for every key step, layers/mvpa.py:244,
   // and takes longest), then one (b, h) after the other, late (= long) steps first; the last two
   // (b, h) of an XCD are interleaved so that the grid does not end on the long steps of one.
-  const int nt = T_;
+  const int nt = (T_ + TQW - 1) / TQW;
   const int nbh = a.B * a.H;
   constexpr int TAIL_MERGE = 2;
-  int bh, tq;
+  int bh, tile;
   {
     const int L = blockIdx.x;
     if ((nbh & 7) == 0 && nt > 1) {
       if (L < nbh) {
         bh = L;
-        tq = nt - 1;
+        tile = nt - 1;
       } else {
         const int L2 = L - nbh;
         const int xcd = L2 & 7, per_xcd = nbh >> 3, s = L2 >> 3;
@@ -81,37 +94,47 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
         const int plain = (per_xcd - merged) * (nt - 1);
         if (s < plain) {
           bh = xcd + 8 * (s / (nt - 1));
-          tq = nt - 2 - s % (nt - 1);
+          tile = nt - 2 - s % (nt - 1);
         } else {
           const int r = s - plain;
           bh = xcd + 8 * (per_xcd - merged + r % merged);
-          tq = nt - 2 - r / merged;
+          tile = nt - 2 - r / merged;
         }
       }
     } else if (nt > 1) {
       if (L < nbh) {
         bh = L;
-        tq = nt - 1;
+        tile = nt - 1;
       } else {
         bh = (L - nbh) / (nt - 1);
-        tq = nt - 2 - (L - nbh) % (nt - 1);
+        tile = nt - 2 - (L - nbh) % (nt - 1);
       }
     } else {
       bh = L;
-      tq = 0;
+      tile = 0;
     }
   }
   const int b = bh / a.H, h = bh % a.H;
   const int g = h / (a.H / a.Hkv);
+  const int tq0 = tile * TQW, tq_hi = min(T_ - 1, tq0 + TQW - 1);
+  const int tq = min(tq0 + ts, T_ - 1);              // (a wave past the end repeats the last step and stores nothing)
   const int cb = 32 * qi;                            // first channel of this wave's queries
-  const bool live = cb < C_;                         // (a wave without queries still moves tiles)
+  const bool live = cb < C_ && tq0 + ts < T_;        // (a wave without queries still moves tiles)
 
-  // ---- key steps 0 .. far_max are far (content term absent or zeroed), far_max+1 .. tq window
+  // ---- for this wave's queries key steps 0 .. far_max are far (content term absent or zeroed),
+  // far_max+1 .. tq window steps.  The workgroup walks window tiles NLO .. tq_hi (a wave skips
+  // what lies outside its own window) and far tiles 0 .. FM (a wave stops at its own far_max).
   const int far_max = !has_content ? tq : (W > 0 && tq != T_ - 1) ? max(-1, tq - W - 1) : -1;
-  const int NLO = far_max + 1;
-  const int n_near = has_content ? tq - far_max : 0;
-  const int n_far = far_max + 1;
-  const int n_total = n_near + n_far;
+  int FM = -1;
+  if (!has_content) {
+    FM = tq_hi;
+  } else if (W > 0) {
+    const int tql = tq_hi == T_ - 1 ? tq_hi - 1 : tq_hi;       // the last step has no far steps
+    if (tql >= tq0) FM = max(-1, tql - W - 1);
+  }
+  const int NLO = (W <= 0 || tq_hi == T_ - 1) ? 0 : max(0, tq0 - W);
+  const int n_near = has_content ? tq_hi - NLO + 1 : 0;
+  const int n_far = FM + 1;
 
   // Loads below are unconditional: rows of padded channels are redirected to an existing row and
   // their results are never used.
@@ -180,7 +203,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
     const int row0 = 4 * hh + e;
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-      const int mt = 2 * half + m;                 // output tile (32 columns) within the row
+      const int mt = (HALVES == 2 ? 2 * half : 0) + m;     // output tile (32 columns) within the row
       v_lane[m] = row0 * ROWB + (((4 * mt + 2 * grp + (aa >> 1)) ^ swz_v<DH>(row0)) << 4) + ((aa & 1) << 3);
     }
 #pragma unroll
@@ -292,7 +315,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
         }
       }
     }
-    float* scr = (float*)(smem_raw + wave * (RING_BYTES / NW));
+    float* scr = (float*)(smem_raw + wave * G::SCRATCH_WAVE);
 #pragma unroll
     for (int t = 0; t < NCT; ++t)
 #pragma unroll
@@ -462,7 +485,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
     // next tiles are requested after it, not before, or the slab would wait for them too)
     if (live && (p == 0 || (tk & 31) == 0)) time_slab(tk & ~31, false);
     issue_avail();
-    if (live) near_step(k_addr(cur_slot), v_addr(cur_slot + 1), tk);
+    if (live && tk > far_max && tk <= tq) near_step(k_addr(cur_slot), v_addr(cur_slot + 1), tk);
     cur_slot = (cur_slot + 2) & (SLOTS - 1);
   }
 
@@ -542,7 +565,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
         for (int s2 = 0; s2 < 2; ++s2) vf0[t * 2 + s2] = v_frag(va_, t, s2, 0);
     }
     for (int tk0 = 0; tk0 < n_far; tk0 += 32) {
-      if (live) time_slab(tk0, true);
+      if (live && tk0 <= far_max) time_slab(tk0, true);
       f32x16 ptmp[MT];
       float pet1 = 0.f;                  // weight of the product waiting in ptmp[1]
 #pragma unroll
@@ -553,7 +576,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
         bare_barrier();                  // (the fragments read ahead stay in flight across it)
         const uint32_t now_lds = cur_lds;
         cur_lds = cur_lds + TILE_BYTES == ring_lds + RING_BYTES ? ring_lds : cur_lds + TILE_BYTES;
-        if (live) {
+        if (live && tk <= far_max) {
           const VAddr va_ = v_addr_at(now_lds), vn_ = v_addr_at(cur_lds);
           // Order of a step, fenced for the scheduler product by product.  First the products of
           // output tile 0 (fragments in registers since the last step); with each of them a
@@ -620,7 +643,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int a4 = 0; a4 < 4; ++a4) {
-        const int d0 = (2 * half + m) * 32 + a4 * 8 + hh * 4;
+        const int d0 = ((HALVES == 2 ? 2 * half : 0) + m) * 32 + a4 * 8 + hh * 4;
         bf16x4 w;
 #pragma unroll
         for (int r = 0; r < 4; ++r) w[r] = (__bf16)(acc[m][a4 * 4 + r] * inv);
@@ -633,26 +656,30 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
 }  // namespace d128
 }  // namespace mvpa
 
-// Shapes the column-split kernel serves: bf16, head size 128, 65..128 channels, a plain forward
-// (no decoding step), bf16 or fp8 content term; everything else about the arguments is as for
-// the general kernel (mvpa_mfma_supported).
+// Shapes this build serves: bf16, 65..128 channels at head size 128 (output columns split over two
+// waves) or 64 (a wave owns every column; the keys are always padded to 128 there), a plain
+// forward (no decoding step), bf16 or fp8 content term; everything else about the arguments is as
+// for the general kernel (mvpa_mfma_supported).
 int mvpa_mfma128_supported(const mvpa_fwd_args* a) {
-  if (a->Dh != 128 || a->C <= 64 || a->C > 128) return 0;
+  if ((a->Dh != 128 && a->Dh != 64) || a->C <= 64 || a->C > 128) return 0;
   if (a->flags & (MVPA_FLAG_LAST_STEP | MVPA_FLAG_RING)) return 0;
   return 1;
 }
 
-template <int NCT, bool FP8>
+template <int DH, int NCT, bool FP8>
 static int launch128(const mvpa_fwd_args* a, hipStream_t stream) {
   using namespace mvpa::d128;
-  using G = Geo<NCT>;
-  auto kern = mvpa_mfma128_kernel<NCT, FP8>;
+  using G = Geo<DH, NCT>;
+  auto kern = mvpa_mfma128_kernel<DH, NCT, FP8>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
-  MVPA_LAUNCH(kern, dim3((unsigned)(a->T * a->B * a->H)), dim3(NW * 64), G::LDS_BYTES, stream, *a);
+  const int nt = (a->T + G::TQW - 1) / G::TQW;
+  MVPA_LAUNCH(kern, dim3((unsigned)(nt * a->B * a->H)), dim3(NW * 64), G::LDS_BYTES, stream, *a);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 
 int mvpa_launch_mfma128(const mvpa_fwd_args* a, hipStream_t stream) {
-  if (a->flags & MVPA_FLAG_FP8_QK) return a->C <= 96 ? launch128<3, true>(a, stream) : launch128<4, true>(a, stream);
-  return a->C <= 96 ? launch128<3, false>(a, stream) : launch128<4, false>(a, stream);
+  const bool fp8 = a->flags & MVPA_FLAG_FP8_QK;
+  if (a->Dh == 64) return fp8 ? launch128<64, 4, true>(a, stream) : launch128<64, 4, false>(a, stream);
+  if (fp8) return a->C <= 96 ? launch128<128, 3, true>(a, stream) : launch128<128, 4, true>(a, stream);
+  return a->C <= 96 ? launch128<128, 3, false>(a, stream) : launch128<128, 4, false>(a, stream);
 }

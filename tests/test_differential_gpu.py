@@ -61,6 +61,11 @@ def test_mfma_paths_match_fp32_kernels(case):
     live = live.reshape(B, 1, T * C, 1)
     assert ((o16.float() - o32) * live).abs().max().item() <= 2e-2
     assert ((l16 - l32) * live[..., 0]).abs().max().item() <= 2e-2
+    if 64 < C <= 128:         # the build for 65..128 channels (here: a workgroup on two time steps)
+        o16w, l16w = mvpa_hip.mvpa_forward(d16.q, d16.k, d16.v, *tabs16, return_lse=True,
+                                           kernel=mvpa_hip.KERNEL_MFMA_SPLIT, **kw)
+        assert ((o16w.float() - o32) * live).abs().max().item() <= 2e-2
+        assert ((l16w - l32) * live[..., 0]).abs().max().item() <= 2e-2
     if 32 < C <= 64:          # the build in which a wave owns a whole time step, at every length
         o16s, l16s = mvpa_hip.mvpa_forward(d16.q, d16.k, d16.v, *tabs16, return_lse=True,
                                            kernel=mvpa_hip.KERNEL_MFMA_STEP, **kw)

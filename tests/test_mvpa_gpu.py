@@ -304,8 +304,9 @@ def test_whole_step_build_refuses_other_shapes():
         mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, kernel=mvpa_hip.KERNEL_MFMA_STEP)
 
 
-# the build of the kernel in which the output columns of a query tile are split over two waves
-# (head size 128, 65..128 channels): the dispatcher's choice for such shapes
+# the build of the kernel for 65..128 channels (head size 128: the output columns of a query tile
+# split over two waves; head size 64: a workgroup on two time steps): the dispatcher's choice for
+# such shapes
 SPLIT_SHAPES = [
     dict(B=1, C=128, T=26, H=2, Dh=128, Hkv=1),                    # the base model's attention shape, GQA 2:1
     dict(B=1, C=100, T=24, H=4, Dh=128, Hkv=2, validity=True),     # ragged channels, absent channels
@@ -317,6 +318,16 @@ SPLIT_SHAPES = [
     dict(B=1, C=128, T=1, H=2, Dh=128),                            # a single time step
     dict(B=1, C=70, T=2, H=1, Dh=128),
     dict(B=1, C=128, T=12, H=2, Dh=128, Hkv=2),                    # exactly one far step
+    # head size 64: a wave owns every output column, a workgroup two time steps
+    dict(B=1, C=117, T=14, H=2, Dh=64, validity=True),             # c3's channel count
+    dict(B=1, C=65, T=40, H=2, Dh=64),                             # just past 64, two slabs, T even
+    dict(B=2, C=128, T=21, H=4, Dh=64, Hkv=2, validity=True),      # T odd: the last workgroup holds one time step
+    dict(B=1, C=96, T=45, H=3, Dh=64),                             # a query tile and a key tile without channels; B*H odd
+    dict(B=1, C=128, T=70, H=2, Dh=64, Hkv=1),                     # three slabs
+    dict(B=1, C=100, T=1, H=2, Dh=64),
+    dict(B=1, C=100, T=2, H=2, Dh=64),
+    dict(B=4, C=80, T=12, H=4, Dh=64),                             # the last pair (10, 11): one far step for step 10 only
+    dict(B=1, C=117, T=13, H=2, Dh=64),                            # pairs (10, 11) and (12): far steps in a workgroup whose partner is the last step
 ]
 
 
@@ -334,8 +345,9 @@ def test_bf16_column_split_build_shapes(cfg):
 @pytest.mark.parametrize("kw", [dict(window=3), dict(window=0), dict(content=False), dict(window=1),
                                 dict(time_bias=False), dict(chan_bias=False), dict(sm_scale=0.05),
                                 dict(window=200)])
-def test_bf16_column_split_build_flags(kw):
-    inp = make_mvpa_inputs(B=1, C=72, T=45, H=2, Dh=128, seed=30, table_std=0.3,
+@pytest.mark.parametrize("dh", [128, 64])
+def test_bf16_column_split_build_flags(kw, dh):
+    inp = make_mvpa_inputs(B=1, C=72, T=45, H=2, Dh=dh, seed=30, table_std=0.3,
                            qkv_unit=True).round_to(torch.bfloat16)
     out = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA_SPLIT, **kw)
     okw = dict(kw)
@@ -353,14 +365,15 @@ def test_bf16_column_split_build_flags(kw):
     _check_bf16(out, _oracle(ref_in, **okw))
 
 
-def test_bf16_column_split_build_large_logits_and_masks():
+@pytest.mark.parametrize("dh", [128, 64])
+def test_bf16_column_split_build_large_logits_and_masks(dh):
     """Wide score range (running-max bookkeeping across the window steps and the far phase), and
-    masks exact under perturbation, on the column-split build."""
-    inp = make_mvpa_inputs(B=1, C=72, T=48, H=2, Dh=128, seed=23, table_std=1.0).round_to(torch.bfloat16)
+    masks exact under perturbation, on the build for 65..128 channels."""
+    inp = make_mvpa_inputs(B=1, C=72, T=48, H=2, Dh=dh, seed=23, table_std=1.0).round_to(torch.bfloat16)
     out = _gpu(inp, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA_SPLIT)
     assert torch.isfinite(out).all()
     _check_bf16(out, _oracle(inp))
-    cfg = dict(B=1, C=100, T=20, H=2, Dh=128, seed=9, table_std=0.3, qkv_unit=True, validity=True)
+    cfg = dict(B=1, C=100, T=20, H=2, Dh=dh, seed=9, table_std=0.3, qkv_unit=True, validity=True)
     inp = make_mvpa_inputs(**cfg)
     inp.chan_valid[0, 2] = False
     run = lambda i: _gpu(i, torch.bfloat16, kernel=mvpa_hip.KERNEL_MFMA_SPLIT)    # noqa: E731
@@ -383,7 +396,7 @@ def test_bf16_column_split_build_large_logits_and_masks():
 
 
 def test_column_split_build_refuses_other_shapes():
-    for cfg in (dict(C=64, Dh=128), dict(C=100, Dh=64)):
+    for cfg in (dict(C=64, Dh=128), dict(C=100, Dh=32), dict(C=64, Dh=64)):
         d = make_mvpa_inputs(seed=1, B=1, T=6, H=1, **cfg).to("cuda", torch.bfloat16)
         with pytest.raises(mvpa_hip.MvpaError):
             mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, kernel=mvpa_hip.KERNEL_MFMA_SPLIT)
@@ -542,7 +555,8 @@ def _gather_case(C, T, Dh, rows, axis):
 
 GATHER_CASES = [(c, "KERNEL_MFMA") for c in GATHER_SHAPES] + [
     (dict(C=64, T=40, Dh=64), "KERNEL_MFMA_STEP"), (dict(C=40, T=70, Dh=64), "KERNEL_MFMA_STEP"),
-    (dict(C=128, T=40, Dh=128), "KERNEL_MFMA_SPLIT"), (dict(C=70, T=70, Dh=128), "KERNEL_MFMA_SPLIT")]
+    (dict(C=128, T=40, Dh=128), "KERNEL_MFMA_SPLIT"), (dict(C=70, T=70, Dh=128), "KERNEL_MFMA_SPLIT"),
+    (dict(C=117, T=41, Dh=64), "KERNEL_MFMA_SPLIT")]
 _gather_id = lambda c: "C{C}T{T}D{Dh}".format(**c) if isinstance(c, dict) else c      # noqa: E731
 
 
@@ -665,14 +679,17 @@ def test_bf16_config2_full_size(kern):
     _check_bf16(out, og.float().cpu())
 
 
-def test_bf16_config3_irregular_channels():
-    """Config c3 (B8 C117 T256 H16 Dh64, per-sample channel validity): sampled query rows of
-    one head against the oracle, masks through bit-exact perturbation."""
+@pytest.mark.parametrize("kern", ["KERNEL_AUTO", "KERNEL_MFMA"])
+def test_bf16_config3_irregular_channels(kern):
+    """Config c3 (B8 C117 T256 H16 Dh64, per-sample channel validity) on the build the library
+    picks for it (65..128 channels: a workgroup on two time steps) and on the general kernel:
+    sampled query rows of one head against the oracle, masks through bit-exact perturbation."""
+    kern = getattr(mvpa_hip, kern)
     inp = make_mvpa_inputs(B=8, C=117, T=256, H=16, Dh=64, seed=0, qkv_unit=True,
                            validity=True).round_to(torch.bfloat16)
     d = inp.to("cuda", torch.bfloat16)
     out = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
-                                chan_valid=d.chan_valid, kernel=mvpa_hip.KERNEL_MFMA)
+                                chan_valid=d.chan_valid, kernel=kern)
     C = 117
     ranges = [(0, 2 * C), (100 * C, 101 * C), (255 * C, 256 * C)]
     ref = _oracle(inp, dtype=torch.float32, heads=[(5, 7)], q_ranges=ranges, q_block=256)
@@ -685,7 +702,7 @@ def test_bf16_config3_irregular_channels():
     k2 = torch.where(dead, seven, d.k.view(8, 16, 256, C, 64)).view(8, 16, 256 * C, 64)
     v2 = torch.where(dead, big, d.v.view(8, 16, 256, C, 64)).view(8, 16, 256 * C, 64)
     o2 = mvpa_hip.mvpa_forward(d.q, k2, v2, d.u, d.vb, d.z, d.k_time, d.k_chan,
-                               chan_valid=d.chan_valid)
+                               chan_valid=d.chan_valid, kernel=kern)
     assert torch.equal(o2, out)
 
 
