@@ -55,7 +55,7 @@ WORKLOADS = {
 def _forward_kernel_name(cfg):
     """The build of the bf16 forward that the library's own choice (MVPA_KERNEL_AUTO) runs for a
     workload: the rule of mvpa_forward in csrc/mvpa_api.hip."""
-    if cfg["Dh"] in (64, 128) and 64 < cfg["C"] <= 128:
+    if (cfg["Dh"] in (64, 128) and 64 < cfg["C"] <= 128) or (cfg["Dh"] == 128 and 32 < cfg["C"] <= 64):
         return "mvpa::d128::mvpa_mfma128_kernel"
     if cfg["Dh"] == 64 and 32 < cfg["C"] <= 64 and cfg["T"] >= 128:
         return "mvpa::q64::mvpa_mfma64_kernel"

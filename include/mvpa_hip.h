@@ -61,11 +61,13 @@ enum {
                                whatever the length; error if the shape is unsupported.  AUTO
                                picks it for 128 time steps and more or when the content term
                                is off, where it is the faster one.                         */
-  MVPA_KERNEL_MFMA_SPLIT = 4 /* the build for 65..128 channels (plain forward, bf16 or fp8
-                               content term): at head size 128 the output columns of a query
-                               tile are split over two waves, at head size 64 a workgroup
-                               takes two time steps; error if the shape is unsupported.  AUTO
-                               picks it for every such shape.                              */
+  MVPA_KERNEL_MFMA_SPLIT = 4 /* the build in which a wave owns 32 queries x 64 output columns
+                               (33..128 channels, head size 64 or 128, plain forward, bf16 or
+                               fp8 content term): at head size 128 the output columns of a
+                               query tile are split over two waves, at head size 64 a
+                               workgroup takes several time steps; error if the shape is
+                               unsupported.  AUTO picks it for 65..128 channels, and for
+                               33..64 channels at head size 128.                           */
 };
 
 /* ---- flags ------------------------------------------------------------------------- */

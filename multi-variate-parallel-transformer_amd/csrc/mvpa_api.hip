@@ -107,7 +107,12 @@ extern "C" int mvpa_forward(const mvpa_fwd_args* a, void* stream) {
     // the general kernel, C 80 .. 100 21 .. 40 %; Dh 64, H16: B8 C117 T256 11.14 -> 8.58 ms,
     // B4 C128 T128 1.86 -> 1.34, B4 C80 T128 1.78 -> 1.21, B8 C128 T32 0.53 -> 0.38, B2 C128 T512
     // 9.99 -> 7.66 ms).
-    if (mvpa_mfma128_supported(a)) return mvpa_launch_mfma128(a, st);
+    if (mvpa_mfma128_supported(a) && a->C > 64) return mvpa_launch_mfma128(a, st);
+    // The same build with two key tiles serves 33..64 channels: at head size 128 it wins too
+    // (B1 H16 C64 T512 3.71 -> 2.87 ms, B4 C64 T64 0.42 -> 0.39); at head size 64 it loses to both
+    // other builds (c2 0.49 against 0.40 and 0.38 ms: 8 products per wave and far step, one
+    // workgroup per CU).
+    if (mvpa_mfma128_supported(a) && a->Dh == 128) return mvpa_launch_mfma128(a, st);
     // Head size 64, 33..64 channels: the whole-time-step build pays for its window passes with a
     // cheaper far phase; against the general kernel it loses at 64 time steps (B4 H12 C64: 0.131
     // against 0.109 ms), is level at 128 and wins from there on (T 256: 6 %, T 512: 10 %), and

@@ -1,4 +1,4 @@
-// bf16 MFMA forward for 65..128 channels at head size 128 or 64 (gfx950, wave64): a wave owns one
+// bf16 MFMA forward for 33..128 channels at head size 128 or 64 (gfx950, wave64): a wave owns one
 // tile of 32 queries and 64 output columns.
 //
 // Head size 128: the general tiled kernel (mvpa_mfma.hip) gives a wave one tile of 32 queries and
@@ -13,7 +13,8 @@
 // Head size 64: a wave owns every output column of its tile, and the 8 waves of a workgroup are
 // the 4 query tiles of TWO consecutive time steps on one K/V ring (the general kernel instead
 // splits the keys of a step over two waves, each with half the products per key step and a merge
-// at the end).  The keys are padded to 128 channels.
+// at the end).  The keys are padded to 64 or 128 channels (two or four key tiles; with two, a time
+// step has two query tiles and a workgroup takes twice as many time steps).
 //
 // The key steps are taken window steps first, far steps after (the online soft-max does not care
 // about the order): the channel-bias tile Bc and the (q+u) fragments are live only in the window
@@ -34,7 +35,8 @@ template <int DH, int NCT>
 struct Geo {
   static constexpr int KS = DH / 16, ROWB = DH * 2, CHUNKS = DH / 8;
   static constexpr int HALVES = DH / 64;               // waves per query tile (column halves)
-  static constexpr int TQW = 2 / HALVES;               // time steps per workgroup
+  static constexpr int QT = NCT <= 2 ? 2 : 4;          // query-tile slots per time step
+  static constexpr int TQW = NW / (HALVES * QT);       // time steps per workgroup
   static constexpr int CP = 32 * NCT;                  // channels, padded
   static constexpr int TILE_BYTES = CP * ROWB;         // one K or V tile
   static constexpr int LPW = TILE_BYTES / 1024 / NW;   // 64-lane x 16-byte loads per tile and wave
@@ -59,14 +61,13 @@ template <int DH, int NCT, bool FP8>
 __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) {
   using G = Geo<DH, NCT>;
   constexpr int TILE_BYTES = G::TILE_BYTES, LPW = G::LPW, RING_BYTES = G::RING_BYTES;
-  constexpr int KS = G::KS, ROWB = G::ROWB, CHUNKS = G::CHUNKS, HALVES = G::HALVES, TQW = G::TQW;
+  constexpr int KS = G::KS, ROWB = G::ROWB, CHUNKS = G::CHUNKS, HALVES = G::HALVES, TQW = G::TQW, QT = G::QT;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 31, hh = lane >> 5;
   // query tile, column half and time step (within the workgroup) of this wave
-  const int qi = HALVES == 2 ? wave >> 1 : wave & 3, half = HALVES == 2 ? wave & 1 : 0;
-  const int ts = HALVES == 2 ? 0 : wave >> 2;
+  const int half = wave % HALVES, qi = (wave / HALVES) % QT, ts = wave / (HALVES * QT);
   const int C_ = a.C, W = a.window, T_ = a.T;
   const bool has_content = a.flags & MVPA_FLAG_CONTENT;
   const bool has_time = a.flags & MVPA_FLAG_TIME_BIAS;
@@ -656,12 +657,12 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
 }  // namespace d128
 }  // namespace mvpa
 
-// Shapes this build serves: bf16, 65..128 channels at head size 128 (output columns split over two
-// waves) or 64 (a wave owns every column; the keys are always padded to 128 there), a plain
+// Shapes this build serves: bf16, 33..128 channels at head size 128 (output columns split over two
+// waves) or 64 (a wave owns every column; the keys are padded to 64 or 128 there), a plain
 // forward (no decoding step), bf16 or fp8 content term; everything else about the arguments is as
 // for the general kernel (mvpa_mfma_supported).
 int mvpa_mfma128_supported(const mvpa_fwd_args* a) {
-  if ((a->Dh != 128 && a->Dh != 64) || a->C <= 64 || a->C > 128) return 0;
+  if ((a->Dh != 128 && a->Dh != 64) || a->C <= 32 || a->C > 128) return 0;
   if (a->flags & (MVPA_FLAG_LAST_STEP | MVPA_FLAG_RING)) return 0;
   return 1;
 }
@@ -679,6 +680,10 @@ static int launch128(const mvpa_fwd_args* a, hipStream_t stream) {
 
 int mvpa_launch_mfma128(const mvpa_fwd_args* a, hipStream_t stream) {
   const bool fp8 = a->flags & MVPA_FLAG_FP8_QK;
+  if (a->C <= 64) {
+    if (a->Dh == 64) return fp8 ? launch128<64, 2, true>(a, stream) : launch128<64, 2, false>(a, stream);
+    return fp8 ? launch128<128, 2, true>(a, stream) : launch128<128, 2, false>(a, stream);
+  }
   if (a->Dh == 64) return fp8 ? launch128<64, 4, true>(a, stream) : launch128<64, 4, false>(a, stream);
   if (fp8) return a->C <= 96 ? launch128<128, 3, true>(a, stream) : launch128<128, 4, true>(a, stream);
   return a->C <= 96 ? launch128<128, 3, false>(a, stream) : launch128<128, 4, false>(a, stream);

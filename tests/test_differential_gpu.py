@@ -61,7 +61,7 @@ def test_mfma_paths_match_fp32_kernels(case):
     live = live.reshape(B, 1, T * C, 1)
     assert ((o16.float() - o32) * live).abs().max().item() <= 2e-2
     assert ((l16 - l32) * live[..., 0]).abs().max().item() <= 2e-2
-    if 64 < C <= 128:         # the build for 65..128 channels (here: a workgroup on two time steps)
+    if 32 < C <= 128:         # the build in which a wave owns 32 queries x 64 columns (here: a workgroup on 2 or 4 time steps)
         o16w, l16w = mvpa_hip.mvpa_forward(d16.q, d16.k, d16.v, *tabs16, return_lse=True,
                                            kernel=mvpa_hip.KERNEL_MFMA_SPLIT, **kw)
         assert ((o16w.float() - o32) * live).abs().max().item() <= 2e-2
@@ -130,7 +130,7 @@ def test_mfma_forward_matches_fp32_kernel_at_other_head_sizes(case):
     assert torch.isfinite(o16.float()).all()
     assert ((o16.float() - o32) * live).abs().max().item() <= 2e-2
     assert ((l16 - l32) * live[..., 0]).abs().max().item() <= 2e-2
-    if Dh == 128 and 64 < C <= 128:      # the build with the output columns split over two waves
+    if Dh == 128 and 32 < C <= 128:      # the build with the output columns split over two waves
         o16s, l16s = mvpa_hip.mvpa_forward(d16.q, d16.k, d16.v, d16.u, d16.vb, d16.z, d16.k_time, d16.k_chan,
                                            kernel=mvpa_hip.KERNEL_MFMA_SPLIT, **kw)
         assert torch.isfinite(o16s.float()).all()
