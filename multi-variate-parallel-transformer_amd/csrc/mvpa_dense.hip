@@ -643,6 +643,255 @@ static int launch_big(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, in
 }
 
 // -----------------------------------------------------------------------------------------
+// The large-tile kernel on a ring of four k-blocks of 32 (K a multiple of 32).
+// With one workgroup per CU and two k-blocks of 64 in LDS, the loads of block k+1 are requested
+// when block k is published and must have landed when it is consumed: every k-block waits out
+// whatever of the L2 / HBM latency its own 2048 matrix cycles do not cover (1.3-1.6 us per
+// k-block measured against 0.85 us of matrix time).  Here a k-block is 32 wide and four are in
+// LDS: the barrier of block k publishes block k+1 (block k was published by the one before),
+// blocks k+2 is in flight and k+3 is requested right after the barrier, so a load has two to
+// three blocks' time to arrive; the first fragments of block k+1 are read before its barrier
+// (the bare s_barrier leaves them in flight), so that a wave leaves the barrier with products to
+// issue.  One block is requested per step without a branch (past the end the last block once
+// more, into a stage nobody reads) so that the waits are fixed vmcnt immediates.
+// Same tile order, roles, row mapping and epilogues as linear_bf16_big_kernel.
+// -----------------------------------------------------------------------------------------
+template <int BN, int EPI>
+__global__ __launch_bounds__(512) void linear_bf16_ring_kernel(const bf16_t* __restrict__ X,
+                                                               const bf16_t* __restrict__ W,
+                                                               bf16_t* __restrict__ Y, int64_t M,
+                                                               int64_t N, int64_t K, int64_t ldx,
+                                                               int64_t ldw, int64_t ldy) {
+  constexpr int BM = 256, BK = 32, ROWB = BK * 2, STAGES = 4;
+  constexpr int WN = BN / 2, NB = WN / 32;            // per-wave extent over w rows
+  constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_LOADS = A_BYTES / 1024 / 8;         // 1 KiB wave loads per wave and block (x rows)
+  constexpr int B_TOT = B_BYTES / 1024, B_LOADS = (B_TOT + 7) / 8;   // w rows: B_TOT loads over 8 waves
+  constexpr bool RAGGED = B_TOT % 8 != 0;             // (BN = 192: waves 0..3 have one load more)
+  static_assert(EPI == 0 || NB % 2 == 0, "gate/up pairs need an even number of sub-blocks");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char gsm[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 31, hh = lane >> 5;
+  const int wm = wave >> 1, wc = wave & 1;
+  constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;    // output columns per workgroup
+  int64_t tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, (M + BM - 1) / BM, (N + OUT_COLS - 1) / OUT_COLS, &tile_m, &tile_n);
+  const int64_t m0 = tile_m * BM, n0 = tile_n * OUT_COLS;
+  const int nkb = (int)(K / BK);
+
+  auto w_row = [&](int r) -> int64_t {                // which w row feeds tile row r
+    if (EPI == 1) {
+      const int wcol = r / WN, nb = (r % WN) / 32, i = r & 31;
+      const int64_t col = n0 + wcol * (WN / 2) + (nb >> 1) * 32 + i;
+      return ((nb & 1) ? N : 0) + (col < N ? col : N - 1);
+    }
+    const int64_t n = n0 + r;
+    return n < N ? n : N - 1;
+  };
+
+  // ---- the request side: the stream of k-blocks, three blocks ahead of the products.  A wave
+  // load covers 16 tile rows x 64 bytes: lane L is row L/4, physical chunk L%4; per-lane byte
+  // offsets from wave-uniform bases (rows clamped into range: such rows are never stored).
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)gsm;
+  int iss_kb = 0;
+  uint32_t iss_lds = lds0;
+  const int64_t wrow0 = w_row(0);
+  const bf16_t* xs = X + m0 * ldx;
+  const bf16_t* ws = W + wrow0 * ldw;
+  uint32_t aoff[A_LOADS], boff[B_LOADS];
+  {
+    const int rsub = lane >> 2, phys = lane & 3;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int row = (wave + 8 * i) * 16 + rsub;
+      const int64_t m = m0 + row;
+      aoff[i] = (uint32_t)((((m < M ? m : M - 1) - m0) * ldx + ((phys ^ ((row >> 2) & 3)) << 3)) * 2);
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+      const int row = min((wave + 8 * i) * 16 + rsub, BN - 1);
+      boff[i] = (uint32_t)(((w_row(row) - wrow0) * ldw + ((phys ^ ((row >> 2) & 3)) << 3)) * 2);
+    }
+  }
+  auto issue_block = [&]() {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(aoff[i]), "s"(xs), "s"(iss_lds + (wave + 8 * i) * 1024) : "memory", "m0");
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+      if (RAGGED && i == B_LOADS - 1 && wave + 8 * i >= B_TOT) continue;   // (uniform per wave)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(boff[i]), "s"(ws), "s"(iss_lds + A_BYTES + (wave + 8 * i) * 1024) : "memory", "m0");
+    }
+    iss_lds = iss_lds + STAGE == lds0 + STAGES * STAGE ? lds0 : iss_lds + STAGE;
+    // on to the next block of the stream; past its end the last block is requested again, into
+    // a stage nobody reads, so that the count of loads in flight stays what the waits assume
+    if (iss_kb + 1 < nkb) {
+      ++iss_kb;
+      xs += BK;
+      ws += BK;
+    }
+  };
+  // at most 1 / 2 blocks' worth of this wave's loads outstanding
+  const bool short_wave = RAGGED && wave + 8 * (B_LOADS - 1) >= B_TOT;
+  auto wait_blocks1 = [&]() {
+    if (short_wave) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(A_LOADS + B_LOADS - 1) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(A_LOADS + B_LOADS) : "memory");
+  };
+  auto wait_blocks2 = [&]() {
+    if (short_wave) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (A_LOADS + B_LOADS - 1)) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (A_LOADS + B_LOADS)) : "memory");
+  };
+
+  // fragment offsets: row ln of a 32-row block, chunk (2ks+hh) ^ swizzle(ln)
+  int frag_off[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) frag_off[ks] = ln * ROWB + (((2 * ks + hh) ^ ((ln >> 2) & 3)) << 4);
+  const int a_lane = (wm * 64) * ROWB, b_lane = A_BYTES + (wc * WN) * ROWB;
+
+  issue_block();
+  issue_block();
+  issue_block();
+  wait_blocks2();
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  bf16x8 xf0[2], wf0[NB];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) xf0[j] = *(const bf16x8*)(gsm + a_lane + j * 32 * ROWB + frag_off[0]);
+#pragma unroll
+  for (int i = 0; i < NB; ++i) wf0[i] = *(const bf16x8*)(gsm + b_lane + i * 32 * ROWB + frag_off[0]);
+  int cur = 0;                                        // stage of the block being multiplied
+  typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+
+  {
+    f32x16 acc[NB][2];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    for (int kb = 0; kb < nkb; ++kb) {
+      wait_blocks1();
+      asm volatile("s_barrier" ::: "memory");         // (fragments read ahead stay in flight across it)
+      const unsigned char* st = gsm + cur * STAGE;
+      cur = (cur + 1) & (STAGES - 1);
+      const unsigned char* sn = gsm + cur * STAGE;
+      bf16x8 xf1[2], wf1[NB];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) xf1[j] = *(const bf16x8*)(st + a_lane + j * 32 * ROWB + frag_off[1]);
+#pragma unroll
+      for (int i = 0; i < NB; ++i) wf1[i] = *(const bf16x8*)(st + b_lane + i * 32 * ROWB + frag_off[1]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf0[i], xf0[j], acc[i][j], 0, 0, 0);
+          if (i == 0 && j == 0) {
+            __builtin_amdgcn_sched_barrier(0);
+            issue_block();
+          }
+        }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) xf0[j] = *(const bf16x8*)(sn + a_lane + j * 32 * ROWB + frag_off[0]);
+#pragma unroll
+      for (int i = 0; i < NB; ++i) wf0[i] = *(const bf16x8*)(sn + b_lane + i * 32 * ROWB + frag_off[0]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf1[i], xf1[j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // ---- epilogue through LDS.  In the accumulators a lane holds 4 consecutive output columns
+    // of one x row (quad a4 = w rows 8*a4 + 4*hh + 0..3 of sub-block i, x row ln of block j): stored
+    // from there, an instruction writes 16 bytes to each of 32 rows.  Staged through the (now idle)
+    // ring, a wave's 32 x WC outputs of a block j leave as whole rows: 16 bytes per lane, a row's
+    // lanes side by side.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // requests past the end; last reads
+    constexpr int WC = EPI == 1 ? WN / 2 : WN;          // output columns of a wave
+    constexpr int PITCH = WC * 2 + 16;                  // bytes per staged row (+16: rows spread over the banks)
+    constexpr int CPR = WC * 2 / 16;                    // 16-byte chunks per row
+    constexpr int RPI = 64 / CPR;                       // rows per store instruction
+    static_assert(8 * 32 * PITCH <= STAGES * STAGE, "the staging area fits the ring");
+    unsigned char* stg = gsm + wave * (32 * PITCH);
+    const bool vec16 = (ldy & 7) == 0 && ((uintptr_t)Y & 15) == 0;
+    const int64_t ncol0 = n0 + wc * WC;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if (EPI == 1) {
+#pragma unroll
+        for (int p2 = 0; p2 < NB / 2; ++p2)
+#pragma unroll
+          for (int a4 = 0; a4 < 4; ++a4) {
+            bf16x4 o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float gte = acc[2 * p2][j][a4 * 4 + r], up = acc[2 * p2 + 1][j][a4 * 4 + r];
+              o[r] = (__bf16)(gte / (1.f + __expf(-gte)) * up);
+            }
+            *(bf16x4*)(stg + ln * PITCH + (p2 * 32 + a4 * 8 + hh * 4) * 2) = o;
+          }
+      } else {
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+#pragma unroll
+          for (int a4 = 0; a4 < 4; ++a4) {
+            bf16x4 o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][a4 * 4 + r];
+            *(bf16x4*)(stg + ln * PITCH + (i * 32 + a4 * 8 + hh * 4) * 2) = o;
+          }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const int rr = lane / CPR, cc = lane % CPR;
+#pragma unroll
+      for (int it = 0; it < (32 + RPI - 1) / RPI; ++it) {
+        const int row = it * RPI + rr;
+        if (rr >= RPI || row >= 32) continue;         // (CPR = 12: 60 lanes carry 5 rows)
+        const u32x4 v = *(const u32x4*)(stg + row * PITCH + cc * 16);
+        const int64_t m = m0 + wm * 64 + j * 32 + row;
+        const int64_t n = ncol0 + cc * 8;
+        if (m < M) {
+          bf16_t* dst = Y + m * ldy + n;
+          if (n + 7 < N && vec16) {
+            *(u32x4*)dst = v;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (n + e < N) dst[e] = (bf16_t)((v[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
+          }
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+  }
+}
+
+template <int BN, int EPI>
+static int launch_ring(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, int64_t N, int64_t K,
+                       int64_t ldx, int64_t ldw, int64_t ldy, hipStream_t s) {
+  constexpr int LDS = 4 * (256 + BN) * 64;
+  auto kern = linear_bf16_ring_kernel<BN, EPI>;
+  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+  constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;
+  dim3 grid((unsigned)(((N + OUT_COLS - 1) / OUT_COLS) * ((M + 255) / 256)));
+  MVPA_LAUNCH(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy);
+  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+}
+
+// -----------------------------------------------------------------------------------------
 // RMSNorm: one workgroup per row, fp32 statistics.
 // -----------------------------------------------------------------------------------------
 template <typename TI, typename TO>
@@ -973,14 +1222,26 @@ extern "C" int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M
       const int64_t wgs = mt * ((N + out_cols - 1) / out_cols);
       return ((wgs + 255) / 256) * bn;
     };
+    // the four-stage ring needs whole k-blocks of 32 and 32-bit byte offsets from a tile's first rows
+    const bool ring = (K & 31) == 0 && K >= 96 && 256 * ldx < ((int64_t)1 << 30) &&
+                      (epilogue == 1 ? 2 * N : (int64_t)256) * ldw < ((int64_t)1 << 30);
     if (epilogue == 1) {
-      if (cost(256, 128) <= cost(128, 64)) return launch_big<256, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
-      return launch_big<128, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
+      // (the wider tile unless it costs a fifth more: [16384 x 768] x [768 x 3456] 114 -> 103 us)
+      if (cost(256, 128) * 5 <= cost(128, 64) * 6)
+        return ring ? launch_ring<256, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+                    : launch_big<256, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
+      return ring ? launch_ring<128, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+                  : launch_big<128, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
     }
     const int64_t c256 = cost(256, 256), c192 = cost(192, 192), c128 = cost(128, 128);
-    if (c256 <= c192 && c256 <= c128) return launch_big<256, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
-    if (c192 <= c128) return launch_big<192, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
-    return launch_big<128, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
+    if (c256 <= c192 && c256 <= c128)
+      return ring ? launch_ring<256, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+                  : launch_big<256, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
+    if (c192 <= c128)
+      return ring ? launch_ring<192, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+                  : launch_big<192, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
+    return ring ? launch_ring<128, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+                : launch_big<128, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
   }
   if (M <= 128) {
     // one decoding step's worth of rows: weight-read bound, spread over N/32 workgroups
