@@ -351,19 +351,23 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
 
   // ---- time-bias slabs: St[j][q] for key steps [tk, tk+32) -> LDS, for the query tiles x0 .. x1.
   // Every operand (the 32 table rows, the time bias vector, the q rows) is requested from global
-  // memory before the first one is used (the q rows of a second tile follow in a trip of their own).
+  // memory before the first one is used.
   // In the far phase (for_far) the soft-max rescale that covers every far step of the slab is
   // done here, once.
   auto time_slab = [&](int x0, int x1, int tk, bool for_far) {
     const int j0 = time_row(tq, tk, T_);
     const int j = min(max(j0 + ln, 0), T_ - 1);       // rows outside the table belong to tk > tq
-    u32x4 rr[KS], br[KS], qr[KS];
+    u32x4 rr[KS], br[KS], qr[2][KS];
     if (has_time) {
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         rr[ks] = *(const u32x4*)((const unsigned char*)ktime + ((uint32_t)j * (DH * 2) + hh * 16) + ks * 32);
         br[ks] = *(const u32x4*)((const unsigned char*)bv + (uint32_t)(hh * 16) + ks * 32);
-        qr[ks] = q_chunk(x0, ks);
+        qr[0][ks] = q_chunk(x0, ks);
+      }
+      if (x1 > x0) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qr[1][ks] = q_chunk(x1, ks);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -376,17 +380,12 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
 #pragma unroll
       for (int i = 0; i < 16; ++i) stc[i] = 0.f;
       if (has_time) {
-        if (x > x0) {                      // the second tile's q rows (the rest is shared)
-#pragma unroll
-          for (int ks = 0; ks < KS; ++ks) qr[ks] = q_chunk(x, ks);
-          __builtin_amdgcn_sched_barrier(0);
-        }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           bf16x8 qv;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const uint32_t w = qr[ks][i], bw = br[ks][i];
+            const uint32_t w = qr[x > x0 ? 1 : 0][ks][i], bw = br[ks][i];
             qv[2 * i] = (__bf16)((__uint_as_float(w << 16) + __uint_as_float(bw << 16)) * sc2);
             qv[2 * i + 1] = (__bf16)((__uint_as_float(w & 0xffff0000u) + __uint_as_float(bw & 0xffff0000u)) * sc2);
           }
@@ -401,7 +400,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
         cm = fmaxf(cm, tk + jj <= far_max ? stc[i] : -INFINITY);
       }
       cm = xhalf_max(cm);
-      if (for_far && tk <= far_max) {            // the slab holds at least one far step
+      if (for_far && tk <= far_max && __ballot(cm + t.mc > t.m) != 0ull) {   // a far step of the slab outgrows the reference
         const float m_new = fmaxf(t.m, cm + t.mc);
         const float alpha = fast_exp2(t.m - m_new);
         t.m = m_new;
@@ -417,9 +416,9 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
   // after it - exponentials, packing, row sums, PV products of the two key tiles - is one
   // straight-line block in which the matrix products of one tile run beside the vector work of
   // the other.  V^T fragments are requested ahead of their use.
-  auto near_step = [&](Tile& tl, const f32x16 (&Bc)[NCT], const bf16x8 (&Qu)[KS], const float* Stb,
-                       const StageAddr& stage, int tk) {
-    const float st = Stb[(tk & 31) * 32 + ln];
+  auto near_step = [&](Tile& tl, const f32x16 (&Bc)[NCT], const bf16x8 (&Qu)[KS], const float* st_at,
+                       const StageAddr& stage) {
+    const float st = *st_at;
     f32x16 S[NCT];
 #pragma unroll
     for (int t = 0; t < NCT; ++t) {
@@ -526,13 +525,20 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
     setup_tile(x, Bc, Qu);
     const float* Stb = stb_wave + x * (32 * 32);
     const int nlo = far_max + 1;                     // this wave's first window step
+    // the time-bias slab of the pass starts at the wave's own first window step: a window of up
+    // to 32 steps never needs a second one
+    int sb = max(nlo, NLO);
+    if (n_pass > 0 && active) time_slab(x, x, sb, false);
     for (int p = 0; p < n_pass; ++p, ++s) {
       const int tk = NLO + p;
       wait_tile(s);
       lds_barrier();
       // (a slab waits for its own operands from global memory, and the load counter is in order:
       // the next tile is requested after it, not before, or the slab would wait for that tile too)
-      if (active && (p == 0 || (tk & 31) == 0)) time_slab(x, x, tk & ~31, false);
+      if (active && tk == sb + 32 && tk <= tq) {
+        sb += 32;
+        time_slab(x, x, sb, false);
+      }
       issue_next();
       if (s + 1 == n_near && n_far > 0) {
         // the last window tile: the other two stages are free, the first four far tiles go there
@@ -541,7 +547,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
         for (int i = 0; i < FSLOTS - 2; ++i) issue_far();
       }
       if (active && tk >= nlo && tk <= tq && (!last_wg || (tk & 1) == par))
-        near_step(qt[x], Bc, Qu, Stb, stage_addr(stg), tk);
+        near_step(qt[x], Bc, Qu, Stb + (tk - sb) * 32 + ln, stage_addr(stg));
       stg = stg + 1 == STAGES ? 0 : stg + 1;
     }
     finish_tile(qt[x], Bc);
