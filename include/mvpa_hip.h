@@ -261,6 +261,16 @@ int mvpa_debug_maps(int32_t T, int32_t C, int32_t window, uint32_t flags,
 int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M, int64_t N, int64_t K,
                      int64_t ldx, int64_t ldw, int64_t ldy, int32_t epilogue, void* stream);
 
+/* y[M,N] = x[M,K] @ w[N,K]^T + r[M,N]: the product with the residual rows added in its epilogue
+ * (the sum is rounded to bf16 once more after the add).  With x = [attention output | MLP
+ * activations] side by side and w = [c_proj | down_proj] it is the whole tail of the parallel
+ * block, hidden + attn + mlp (layers/mvpa.py:400, models/mvpformer.py:146-147), in one kernel.
+ * Large shapes only: M >= 512, K a multiple of 32 and >= 96; MVPA_ERR_UNSUPPORTED otherwise.
+ * y may be r (in place).  ldr is r's row pitch in elements. */
+int mvpa_linear_bf16_residual(const void* x, const void* w, const void* r, void* y, int64_t M,
+                              int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldr,
+                              int64_t ldy, void* stream);
+
 /* The same product for at most 128 rows of x against a large weight (the projections of one
  * decoding step of a wide model), with K split over workgroups: fp32 partial tiles go through the
  * caller's workspace ws (mvpa_linear_splitk_ws_bytes(M, N, K, epilogue) bytes, 16-byte aligned)

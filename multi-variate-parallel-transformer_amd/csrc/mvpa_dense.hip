@@ -458,7 +458,7 @@ __global__ __launch_bounds__(512) void linear_bf16_big_kernel(const bf16_t* __re
   constexpr int WN = BN / 2, NB = WN / 32;            // per-wave extent over w rows
   constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
   constexpr int A_LOADS = A_BYTES / 1024 / 8, B_LOADS = B_BYTES / 1024 / 8;   // per wave
-  static_assert(EPI == 0 || NB % 2 == 0, "gate/up pairs need an even number of sub-blocks");
+  static_assert(EPI != 1 || NB % 2 == 0, "gate/up pairs need an even number of sub-blocks");
   extern __shared__ __attribute__((aligned(1024))) unsigned char gsm[];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -656,19 +656,22 @@ static int launch_big(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, in
 // more, into a stage nobody reads) so that the waits are fixed vmcnt immediates.
 // Same tile order, roles, row mapping and epilogues as linear_bf16_big_kernel.
 // -----------------------------------------------------------------------------------------
+// EPI 2: Y = X W^T + R, the residual rows R (bf16, row pitch ldr) added where the staged rows
+// are read back, 16 bytes per lane like the stores.
 template <int BN, int EPI>
 __global__ __launch_bounds__(512) void linear_bf16_ring_kernel(const bf16_t* __restrict__ X,
                                                                const bf16_t* __restrict__ W,
                                                                bf16_t* __restrict__ Y, int64_t M,
                                                                int64_t N, int64_t K, int64_t ldx,
-                                                               int64_t ldw, int64_t ldy) {
+                                                               int64_t ldw, int64_t ldy,
+                                                               const bf16_t* __restrict__ R, int64_t ldr) {
   constexpr int BM = 256, BK = 32, ROWB = BK * 2, STAGES = 4;
   constexpr int WN = BN / 2, NB = WN / 32;            // per-wave extent over w rows
   constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
   constexpr int A_LOADS = A_BYTES / 1024 / 8;         // 1 KiB wave loads per wave and block (x rows)
   constexpr int B_TOT = B_BYTES / 1024, B_LOADS = (B_TOT + 7) / 8;   // w rows: B_TOT loads over 8 waves
   constexpr bool RAGGED = B_TOT % 8 != 0;             // (BN = 192: waves 0..3 have one load more)
-  static_assert(EPI == 0 || NB % 2 == 0, "gate/up pairs need an even number of sub-blocks");
+  static_assert(EPI != 1 || NB % 2 == 0, "gate/up pairs need an even number of sub-blocks");
   extern __shared__ __attribute__((aligned(1024))) unsigned char gsm[];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -822,7 +825,8 @@ __global__ __launch_bounds__(512) void linear_bf16_ring_kernel(const bf16_t* __r
     constexpr int RPI = 64 / CPR;                       // rows per store instruction
     static_assert(8 * 32 * PITCH <= STAGES * STAGE, "the staging area fits the ring");
     unsigned char* stg = gsm + wave * (32 * PITCH);
-    const bool vec16 = (ldy & 7) == 0 && ((uintptr_t)Y & 15) == 0;
+    const bool vec16 = (ldy & 7) == 0 && ((uintptr_t)Y & 15) == 0 &&
+                       (EPI != 2 || ((ldr & 7) == 0 && ((uintptr_t)R & 15) == 0));
     const int64_t ncol0 = n0 + wc * WC;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -858,17 +862,30 @@ __global__ __launch_bounds__(512) void linear_bf16_ring_kernel(const bf16_t* __r
       for (int it = 0; it < (32 + RPI - 1) / RPI; ++it) {
         const int row = it * RPI + rr;
         if (rr >= RPI || row >= 32) continue;         // (CPR = 12: 60 lanes carry 5 rows)
-        const u32x4 v = *(const u32x4*)(stg + row * PITCH + cc * 16);
+        u32x4 v = *(const u32x4*)(stg + row * PITCH + cc * 16);
         const int64_t m = m0 + wm * 64 + j * 32 + row;
         const int64_t n = ncol0 + cc * 8;
         if (m < M) {
           bf16_t* dst = Y + m * ldy + n;
           if (n + 7 < N && vec16) {
+            if (EPI == 2) {
+              const u32x4 r = *(const u32x4*)(R + m * ldr + n);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const float lo = __uint_as_float(v[e] << 16) + __uint_as_float(r[e] << 16);
+                const float hi = __uint_as_float(v[e] & 0xffff0000u) + __uint_as_float(r[e] & 0xffff0000u);
+                v[e] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+              }
+            }
             *(u32x4*)dst = v;
           } else {
 #pragma unroll
             for (int e = 0; e < 8; ++e)
-              if (n + e < N) dst[e] = (bf16_t)((v[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
+              if (n + e < N) {
+                bf16_t o = (bf16_t)((v[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
+                if (EPI == 2) o = f32_to_bf16(bf16_to_f32(o) + bf16_to_f32(R[m * ldr + n + e]));
+                dst[e] = o;
+              }
           }
         }
       }
@@ -881,13 +898,14 @@ __global__ __launch_bounds__(512) void linear_bf16_ring_kernel(const bf16_t* __r
 
 template <int BN, int EPI>
 static int launch_ring(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, int64_t N, int64_t K,
-                       int64_t ldx, int64_t ldw, int64_t ldy, hipStream_t s) {
+                       int64_t ldx, int64_t ldw, int64_t ldy, hipStream_t s,
+                       const bf16_t* r = nullptr, int64_t ldr = 0) {
   constexpr int LDS = 4 * (256 + BN) * 64;
   auto kern = linear_bf16_ring_kernel<BN, EPI>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
   constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;
   dim3 grid((unsigned)(((N + OUT_COLS - 1) / OUT_COLS) * ((M + 255) / 256)));
-  MVPA_LAUNCH(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy);
+  MVPA_LAUNCH(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy, r, ldr);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 
@@ -1258,6 +1276,29 @@ extern "C" int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M
     MVPA_LAUNCH(linear_bf16_kernel<0>, grid, dim3(256), 0, s, xp, wp, yp, M, N, K, ldx, ldw, ldy);
   }
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+}
+
+// Y = X W^T + R in one kernel (the large-tile ring kernel only): at least 512 rows, K a multiple
+// of 32 and at least 96.  Other shapes: MVPA_ERR_UNSUPPORTED (the caller adds R itself).
+extern "C" int mvpa_linear_bf16_residual(const void* x, const void* w, const void* r, void* y,
+                                         int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw,
+                                         int64_t ldr, int64_t ldy, void* stream) {
+  if (!x || !w || !y || !r) return MVPA_ERR_NULL;
+  if (M <= 0 || N <= 0 || K <= 0 || ldx < K || ldw < K || ldy < N || ldr < N) return MVPA_ERR_SHAPE;
+  if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || (ldx & 7) || (ldw & 7)) return MVPA_ERR_ALIGN;
+  if (((uintptr_t)y & 1) || ((uintptr_t)r & 1)) return MVPA_ERR_ALIGN;
+  const bool ring = M >= 512 && (K & 31) == 0 && K >= 96 && 256 * ldx < ((int64_t)1 << 30) &&
+                    256 * ldw < ((int64_t)1 << 30);
+  if (!ring) return MVPA_ERR_UNSUPPORTED;
+  hipStream_t s = (hipStream_t)stream;
+  const bf16_t *xp = (const bf16_t*)x, *wp = (const bf16_t*)w, *rp = (const bf16_t*)r;
+  bf16_t* yp = (bf16_t*)y;
+  const int64_t mt = (M + 255) / 256;
+  auto cost = [&](int bn) -> int64_t { return ((mt * ((N + bn - 1) / bn) + 255) / 256) * bn; };
+  const int64_t c256 = cost(256), c192 = cost(192), c128 = cost(128);
+  if (c256 <= c192 && c256 <= c128) return launch_ring<256, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s, rp, ldr);
+  if (c192 <= c128) return launch_ring<192, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s, rp, ldr);
+  return launch_ring<128, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s, rp, ldr);
 }
 
 extern "C" int mvpa_rmsnorm(const void* x, const float* weight, void* y, int64_t rows,

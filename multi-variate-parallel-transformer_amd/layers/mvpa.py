@@ -300,7 +300,9 @@ class MVPFormerGQAAttention(torch.nn.Module):
         return bool(self.global_att)                       # layers/mvpa.py:188-222, 230
 
     def _attend(self, hidden_states, positional_embedding, channel_embedding, attention_mask,
-                head_mask, use_cache, window, layer_past=None):
+                head_mask, use_cache, window, layer_past=None, merged_out=None):
+        """merged_out: a [B, T*C, H, Dh] view (unit last stride, any row pitch) that receives the
+        merged heads; c_proj is then left to the caller and merged_out is what comes back."""
         if self.training and (self.attn_dropout.p > 0 or self.resid_dropout.p > 0):
             raise NotImplementedError("MVPA HIP layer: dropout/training is not implemented; call .eval()")
         if self.is_cross_attention:
@@ -312,6 +314,8 @@ class MVPFormerGQAAttention(torch.nn.Module):
         n = t_len * c_len
         dt = hidden_states.dtype
         if layer_past is not None:
+            if merged_out is not None:
+                raise NotImplementedError("merged_out goes with a whole-sequence forward")
             return self._attend_step(hidden_states, positional_embedding, channel_embedding,
                                      attention_mask, head_mask, use_cache, window, layer_past)
         with torch.no_grad():
@@ -328,7 +332,8 @@ class MVPFormerGQAAttention(torch.nn.Module):
                 chan_valid = self._as_channel_validity(attention_mask, bsz, t_len, c_len)
                 if chan_valid is None:
                     key_bias = attention_mask.reshape(bsz, n).to(torch.float32)
-            merged = torch.empty((bsz, n, h, dh), dtype=dt, device=hidden_states.device)
+            merged = merged_out if merged_out is not None else \
+                torch.empty((bsz, n, h, dh), dtype=dt, device=hidden_states.device)
             mvpa_hip.mvpa_forward(
                 q, k, v, u, vb, z, k_time, k_chan, sm_scale=self._scale(), window=window,
                 causal=True, content=self._content(), chan_valid=chan_valid,
@@ -337,8 +342,12 @@ class MVPFormerGQAAttention(torch.nn.Module):
             if head_mask is not None:                       # layers/mvpa.py:274-275
                 if head_mask.numel() != h:
                     raise NotImplementedError("head_mask must hold one factor per head")
-                merged = merged * head_mask.to(dt).reshape(1, 1, h, 1)
-            out = _linear(merged.view(bsz, t_len, c_len, e), self.c_proj.weight)
+                if merged_out is not None:
+                    merged_out.mul_(head_mask.to(dt).reshape(1, 1, h, 1))
+                else:
+                    merged = merged * head_mask.to(dt).reshape(1, 1, h, 1)
+            out = merged if merged_out is not None else \
+                _linear(merged.view(bsz, t_len, c_len, e), self.c_proj.weight)
         present = None
         if use_cache is True:                               # layers/mvpa.py:318-321
             present = (k.reshape(bsz, hkv, t_len, c_len, dh), v.reshape(bsz, hkv, t_len, c_len, dh))
@@ -442,6 +451,17 @@ class MVPFormerGQAAttention(torch.nn.Module):
         if output_attentions:
             outputs += (None,)                            # layers/mvpa.py:407-408
         return outputs
+
+
+    def forward_merged(self, hidden_states, positional_embedding, channel_embedding, merged_out,
+                       attention_mask=None, head_mask=None, use_cache=False):
+        """forward() up to the merged heads: they are written into merged_out ([B, T*C, H, Dh], unit
+        last stride, any row pitch) and c_proj (layers/mvpa.py:400) is left to the caller, who can
+        fold it into a later product.  Returns (merged_out, present)."""
+        if not self._honours_masks:
+            attention_mask, head_mask = None, None
+        return self._attend(hidden_states, positional_embedding, channel_embedding, attention_mask,
+                            head_mask, use_cache, window=10, merged_out=merged_out)
 
 
 class MVPFormerGQAFlashAttention(MVPFormerGQAAttention):

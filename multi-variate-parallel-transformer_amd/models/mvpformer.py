@@ -98,6 +98,12 @@ class GatedMLP(nn.Module):
         mid = mvpa_hip.linear(x, self._gate_up(), gated=True)
         return mvpa_hip.linear(mid, self.down_proj.weight.to(torch.bfloat16))
 
+    @torch.no_grad()
+    def activations_into(self, x, out):
+        """silu(gate(x)) * up(x) written into out, a [rows, intermediate] view of any row pitch:
+        the MLP up to its down projection, for a caller that folds that into a later product."""
+        mvpa_hip.linear(x, self._gate_up(), gated=True, out=out)
+
 
 class MVPFormerBlock(nn.Module):
     """Parallel block: x + MLP(ln_1(x)) + Attn(ln_1(x)); ln_2 exists but is unused
@@ -111,6 +117,18 @@ class MVPFormerBlock(nn.Module):
         self.attn = cls(config, layer_idx=layer_idx)
         self.ln_2 = RMSNorm(hidden_size, eps=config.layer_norm_epsilon)
         self.mlp = GatedMLP(config)
+        self._tail_w = None
+        self._tail_key = None
+
+    def _tail_weight(self) -> torch.Tensor:
+        """[c_proj | down_proj] side by side ([E, E + intermediate]), cached until one changes:
+        attn_out + mlp_out = [merged heads | MLP activations] @ this^T."""
+        wc, wd = self.attn.c_proj.weight, self.mlp.down_proj.weight
+        key = (wc.data_ptr(), wc._version, wd.data_ptr(), wd._version)
+        if self._tail_key != key:
+            self._tail_w = torch.cat([wc, wd], 1).detach().to(torch.bfloat16).contiguous()
+            self._tail_key = key
+        return self._tail_w
 
     def forward(self, hidden_states, positional_embedding, channel_embedding, layer_past=None,
                 attention_mask=None, head_mask=None, encoder_hidden_states=None,
@@ -131,6 +149,27 @@ class MVPFormerBlock(nn.Module):
         residual = hidden_states
         if normed is None:
             normed = self.ln_1(hidden_states)
+        e, inner = self.attn.embed_dim, self.mlp.down_proj.in_features
+        rows = hidden_states.numel() // e
+        if (layer_past is None and not output_attentions and residual.is_cuda
+                and residual.dtype == torch.bfloat16 and normed.dtype == torch.bfloat16
+                and (head_mask is None or not self.attn._honours_masks)
+                and mvpa_hip.linear_residual_supported(rows, e + inner)):
+            # One product for the whole tail of the block: the attention kernel writes the merged
+            # heads and the gate/up product its activations side by side into one buffer, and
+            # hidden + c_proj(merged) + down(activations) = hidden + [merged | act] @ [c_proj | down]^T
+            bsz, t_len, c_len, _ = hidden_states.shape
+            h, dh = self.attn.num_heads, self.attn.head_dim
+            both = torch.empty((rows, e + inner), dtype=torch.bfloat16, device=residual.device)
+            merged = both[:, :e].unflatten(0, (bsz, t_len * c_len)).unflatten(2, (h, dh))
+            _, present = self.attn.forward_merged(normed, positional_embedding, channel_embedding, merged,
+                                                  attention_mask=attention_mask, use_cache=use_cache)
+            self.mlp.activations_into(normed.reshape(rows, e), both[:, e:])
+            hidden_states = mvpa_hip.linear(both, self._tail_weight(),
+                                            residual=residual.reshape(rows, e)).view(residual.shape)
+            next_normed = next_norm(hidden_states) if next_norm is not None else None
+            outputs = (hidden_states, present) if use_cache else (hidden_states,)
+            return outputs, next_normed
         attn_outputs = self.attn(normed, positional_embedding, channel_embedding,
                                  layer_past=layer_past, attention_mask=attention_mask,
                                  head_mask=head_mask, use_cache=use_cache,

@@ -112,6 +112,8 @@ def load_library() -> ctypes.CDLL:
     lib.mvpa_debug_maps.argtypes = [i32, i32, i32, u32, vp, vp, vp, vp, vp]
     lib.mvpa_linear_bf16.restype = ctypes.c_int
     lib.mvpa_linear_bf16.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, i32, vp]
+    lib.mvpa_linear_bf16_residual.restype = ctypes.c_int
+    lib.mvpa_linear_bf16_residual.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp]
     lib.mvpa_rmsnorm.restype = ctypes.c_int
     lib.mvpa_rmsnorm.argtypes = [vp, vp, vp, i64, i32, i64, i64, f32, i32, i32, vp]
     lib.mvpa_add3_bf16.restype = ctypes.c_int
@@ -377,24 +379,48 @@ def debug_maps(T: int, C: int, window: int = 10, flags: int = 15, chan_valid=Non
     return ti, ci, mb
 
 
+def linear_residual_supported(M: int, K: int) -> bool:
+    """Shapes mvpa_linear_bf16_residual takes (the large-tile kernel: see include/mvpa_hip.h)."""
+    return M >= 512 and K % 32 == 0 and K >= 96
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None,
-           gated: bool = False, split_k: Optional[bool] = None) -> torch.Tensor:
+           gated: bool = False, split_k: Optional[bool] = None,
+           residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y = x @ weight.T in bf16 on MFMA.  gated=True: weight stacks [gate; up] rows and the
     result is silu(x@gate.T) * (x@up.T).  split_k: the K-split kernel pair through a workspace
-    (at most 128 rows); None picks it for K >= 1536 and at most 4096 rows of weight."""
+    (at most 128 rows); None picks it for K >= 1536 and at most 4096 rows of weight.
+    x may be a 2-D row-pitched view (unit last stride), out a 2-D view [rows, N] likewise.
+    residual: [rows, N] bf16 added in the product's epilogue (shapes for which
+    linear_residual_supported holds; otherwise MvpaError)."""
     lib = load_library()
     _need_cuda(x, weight)
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
         raise TypeError("linear: bf16 only")
     K = x.shape[-1]
-    x2 = x.reshape(-1, K)
+    x2 = x if x.dim() == 2 and x.stride(-1) == 1 else x.reshape(-1, K)
     if x2.stride(-1) != 1:
         x2 = x2.contiguous()
     assert weight.shape[1] == K and weight.stride(1) == 1
     M = x2.shape[0]
     N = weight.shape[0] // 2 if gated else weight.shape[0]
+    given = out is not None
     if out is None:
         out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    else:
+        if out.dim() != 2 or tuple(out.shape) != (M, N) or out.stride(1) != 1 or out.dtype != torch.bfloat16:
+            raise ValueError("linear: out must be a bf16 [rows, N] tensor or view with unit last stride")
+    if residual is not None:
+        if gated or split_k:
+            raise ValueError("linear: residual goes with the plain product only")
+        r2 = residual.reshape(M, N) if residual.dim() != 2 else residual
+        if tuple(r2.shape) != (M, N) or r2.stride(1) != 1 or r2.dtype != torch.bfloat16:
+            raise ValueError("linear: residual must be bf16 [rows, N] with unit last stride")
+        _need_cuda(r2)
+        _check(lib.mvpa_linear_bf16_residual(x2.data_ptr(), weight.data_ptr(), r2.data_ptr(), out.data_ptr(),
+                                             M, N, K, x2.stride(0), weight.stride(0), r2.stride(0),
+                                             out.stride(0), _stream()))
+        return out if given else out.view(*x.shape[:-1], N)
     if split_k is None:
         # measured on graph replays (GPU time): [128x2048]x[2048x4096] 22.9 -> 18.6 us,
         # [128x5632]x[5632x2048] 58.1 -> 21.0 us, [64x1728]x[1728x768] 13.2 -> 10.0 us; the wide
@@ -406,11 +432,11 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = 
         _check(lib.mvpa_linear_bf16_splitk(x2.data_ptr(), weight.data_ptr(), out.data_ptr(), M, N, K,
                                            x2.stride(0), weight.stride(0), out.stride(0),
                                            1 if gated else 0, ws.data_ptr(), ws.numel(), _stream()))
-        return out.view(*x.shape[:-1], N)
+        return out if given else out.view(*x.shape[:-1], N)
     _check(lib.mvpa_linear_bf16(x2.data_ptr(), weight.data_ptr(), out.data_ptr(), M, N, K,
                                 x2.stride(0), weight.stride(0), out.stride(0),
                                 1 if gated else 0, _stream()))
-    return out.view(*x.shape[:-1], N)
+    return out if given else out.view(*x.shape[:-1], N)
 
 
 def _as_f32_weight(weight: torch.Tensor) -> torch.Tensor:

@@ -45,6 +45,49 @@ def test_linear_gated(M, N, K):
     assert (y.double() - ref).abs().max().item() <= 2 ** -7 * ref.abs().max().item() + 1e-5
 
 
+@pytest.mark.parametrize("M,N,K", [(1024, 768, 2496), (16384, 768, 2496), (600, 130, 96), (4096, 2048, 7680),
+                                   (2000, 200, 160), (8192, 520, 256)])
+def test_linear_with_residual_in_the_epilogue(M, N, K):
+    """y = x w^T + r against float64 (fp32 accumulation, the product rounded to bf16, the sum with r
+    rounded once more: 2^-8 of the product's range + 2^-8 of the sum's), with the operands as
+    column slices of wider buffers (row pitches that are not the row lengths) and r odd-pitched."""
+    g = torch.Generator().manual_seed(M + N + K)
+    xw = torch.randn(M, K + 64, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16()
+    rw = torch.randn(M, N + 3, generator=g).bfloat16()
+    xg, rg = xw.cuda(), rw.cuda()
+    y = mvpa_hip.linear(xg[:, 32:32 + K], w.cuda(), residual=rg[:, :N]).float().cpu()
+    prod = xw[:, 32:32 + K].double() @ w.double().T
+    ref = prod + rw[:, :N].double()
+    tol = 2 ** -8 * prod.abs().max().item() + 2 ** -8 * ref.abs().max().item() + 1e-6
+    assert (y.double() - ref).abs().max().item() <= tol
+    # into a view of a wider output, in place over the residual
+    wide = torch.zeros(M, N + 40, dtype=torch.bfloat16, device="cuda")
+    wide[:, 8:8 + N] = rg[:, :N]
+    mvpa_hip.linear(xg[:, 32:32 + K], w.cuda(), residual=wide[:, 8:8 + N], out=wide[:, 8:8 + N])
+    assert torch.equal(wide[:, 8:8 + N].float().cpu(), y)
+    assert wide[:, :8].abs().max().item() == 0 and wide[:, 8 + N:].abs().max().item() == 0
+
+
+def test_linear_with_residual_refuses_small_shapes():
+    x = torch.zeros(64, 768, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(768, 768, dtype=torch.bfloat16, device="cuda")
+    assert not mvpa_hip.linear_residual_supported(64, 768)
+    with pytest.raises(mvpa_hip.MvpaError):
+        mvpa_hip.linear(x, w, residual=x)
+
+
+def test_linear_into_a_column_slice():
+    """The gated product written into a column slice of a wider buffer (the block's tail operand)."""
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(1024, 768, generator=g).bfloat16().cuda()
+    w = (torch.randn(2 * 1728, 768, generator=g) * 0.05).bfloat16().cuda()
+    ref = mvpa_hip.linear(x, w, gated=True)
+    both = torch.full((1024, 768 + 1728), 7.0, dtype=torch.bfloat16, device="cuda")
+    mvpa_hip.linear(x, w, gated=True, out=both[:, 768:])
+    assert torch.equal(both[:, 768:], ref) and (both[:, :768] == 7.0).all()
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_rmsnorm(dtype):
     g = torch.Generator().manual_seed(1)
