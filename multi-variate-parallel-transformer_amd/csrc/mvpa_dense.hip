@@ -642,6 +642,98 @@ static int launch_big(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, in
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 
+// ---- epilogue of the large-tile kernels, through LDS (LDS_BYTES of it, idle by now).
+// In the accumulators a lane holds 4 consecutive output columns of one x row (quad a4 = w rows
+// 8*a4 + 4*hh + 0..3 of sub-block i, x row ln of block j): stored from there, an instruction writes
+// 16 bytes to each of 32 rows.  Staged through LDS, a wave's 32 x WC outputs of a block j leave as
+// whole rows: 16 bytes per lane, a row's lanes side by side.  EPI 1: SiLU gate; EPI 2: the residual
+// rows R are added where the staged rows are read back.
+template <int BN, int EPI, int LDS_BYTES>
+__device__ inline void staged_epilogue(const f32x16 (&acc)[BN / 64][2], unsigned char* gsm, int wave, int lane,
+                                       int64_t m0, int64_t n0, int64_t M, int64_t N,
+                                       bf16_t* __restrict__ Y, int64_t ldy,
+                                       const bf16_t* __restrict__ R, int64_t ldr) {
+  typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+  constexpr int WN = BN / 2, NB = WN / 32;
+  const int ln = lane & 31, hh = lane >> 5;
+  const int wm = wave >> 1, wc = wave & 1;
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // requests past the end; last reads
+  constexpr int WC = EPI == 1 ? WN / 2 : WN;          // output columns of a wave
+  constexpr int PITCH = WC * 2 + 16;                  // bytes per staged row (+16: rows spread over the banks)
+  constexpr int CPR = WC * 2 / 16;                    // 16-byte chunks per row
+  constexpr int RPI = 64 / CPR;                       // rows per store instruction
+  static_assert(8 * 32 * PITCH <= LDS_BYTES, "the staging area fits the ring");
+  unsigned char* stg = gsm + wave * (32 * PITCH);
+  const bool vec16 = (ldy & 7) == 0 && ((uintptr_t)Y & 15) == 0 &&
+                     (EPI != 2 || ((ldr & 7) == 0 && ((uintptr_t)R & 15) == 0));
+  const int64_t ncol0 = n0 + wc * WC;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    if (EPI == 1) {
+#pragma unroll
+      for (int p2 = 0; p2 < NB / 2; ++p2)
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) {
+          bf16x4 o;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float gte = acc[2 * p2][j][a4 * 4 + r], up = acc[2 * p2 + 1][j][a4 * 4 + r];
+            o[r] = (__bf16)(gte / (1.f + __expf(-gte)) * up);
+          }
+          *(bf16x4*)(stg + ln * PITCH + (p2 * 32 + a4 * 8 + hh * 4) * 2) = o;
+        }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) {
+          bf16x4 o;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][a4 * 4 + r];
+          *(bf16x4*)(stg + ln * PITCH + (i * 32 + a4 * 8 + hh * 4) * 2) = o;
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int rr = lane / CPR, cc = lane % CPR;
+#pragma unroll
+    for (int it = 0; it < (32 + RPI - 1) / RPI; ++it) {
+      const int row = it * RPI + rr;
+      if (rr >= RPI || row >= 32) continue;         // (CPR = 12: 60 lanes carry 5 rows)
+      u32x4 v = *(const u32x4*)(stg + row * PITCH + cc * 16);
+      const int64_t m = m0 + wm * 64 + j * 32 + row;
+      const int64_t n = ncol0 + cc * 8;
+      if (m < M) {
+        bf16_t* dst = Y + m * ldy + n;
+        if (n + 7 < N && vec16) {
+          if (EPI == 2) {
+            const u32x4 r = *(const u32x4*)(R + m * ldr + n);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float lo = __uint_as_float(v[e] << 16) + __uint_as_float(r[e] << 16);
+              const float hi = __uint_as_float(v[e] & 0xffff0000u) + __uint_as_float(r[e] & 0xffff0000u);
+              v[e] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+            }
+          }
+          *(u32x4*)dst = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (n + e < N) {
+              bf16_t o = (bf16_t)((v[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
+              if (EPI == 2) o = f32_to_bf16(bf16_to_f32(o) + bf16_to_f32(R[m * ldr + n + e]));
+              dst[e] = o;
+            }
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+}
+
 // -----------------------------------------------------------------------------------------
 // The large-tile kernel on a ring of four k-blocks of 32 (K a multiple of 32).
 // With one workgroup per CU and two k-blocks of 64 in LDS, the loads of block k+1 are requested
@@ -813,86 +905,7 @@ __global__ __launch_bounds__(512) void linear_bf16_ring_kernel(const bf16_t* __r
       __builtin_amdgcn_sched_barrier(0);
     }
 
-    // ---- epilogue through LDS.  In the accumulators a lane holds 4 consecutive output columns
-    // of one x row (quad a4 = w rows 8*a4 + 4*hh + 0..3 of sub-block i, x row ln of block j): stored
-    // from there, an instruction writes 16 bytes to each of 32 rows.  Staged through the (now idle)
-    // ring, a wave's 32 x WC outputs of a block j leave as whole rows: 16 bytes per lane, a row's
-    // lanes side by side.
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // requests past the end; last reads
-    constexpr int WC = EPI == 1 ? WN / 2 : WN;          // output columns of a wave
-    constexpr int PITCH = WC * 2 + 16;                  // bytes per staged row (+16: rows spread over the banks)
-    constexpr int CPR = WC * 2 / 16;                    // 16-byte chunks per row
-    constexpr int RPI = 64 / CPR;                       // rows per store instruction
-    static_assert(8 * 32 * PITCH <= STAGES * STAGE, "the staging area fits the ring");
-    unsigned char* stg = gsm + wave * (32 * PITCH);
-    const bool vec16 = (ldy & 7) == 0 && ((uintptr_t)Y & 15) == 0 &&
-                       (EPI != 2 || ((ldr & 7) == 0 && ((uintptr_t)R & 15) == 0));
-    const int64_t ncol0 = n0 + wc * WC;
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      if (EPI == 1) {
-#pragma unroll
-        for (int p2 = 0; p2 < NB / 2; ++p2)
-#pragma unroll
-          for (int a4 = 0; a4 < 4; ++a4) {
-            bf16x4 o;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const float gte = acc[2 * p2][j][a4 * 4 + r], up = acc[2 * p2 + 1][j][a4 * 4 + r];
-              o[r] = (__bf16)(gte / (1.f + __expf(-gte)) * up);
-            }
-            *(bf16x4*)(stg + ln * PITCH + (p2 * 32 + a4 * 8 + hh * 4) * 2) = o;
-          }
-      } else {
-#pragma unroll
-        for (int i = 0; i < NB; ++i)
-#pragma unroll
-          for (int a4 = 0; a4 < 4; ++a4) {
-            bf16x4 o;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][a4 * 4 + r];
-            *(bf16x4*)(stg + ln * PITCH + (i * 32 + a4 * 8 + hh * 4) * 2) = o;
-          }
-      }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      const int rr = lane / CPR, cc = lane % CPR;
-#pragma unroll
-      for (int it = 0; it < (32 + RPI - 1) / RPI; ++it) {
-        const int row = it * RPI + rr;
-        if (rr >= RPI || row >= 32) continue;         // (CPR = 12: 60 lanes carry 5 rows)
-        u32x4 v = *(const u32x4*)(stg + row * PITCH + cc * 16);
-        const int64_t m = m0 + wm * 64 + j * 32 + row;
-        const int64_t n = ncol0 + cc * 8;
-        if (m < M) {
-          bf16_t* dst = Y + m * ldy + n;
-          if (n + 7 < N && vec16) {
-            if (EPI == 2) {
-              const u32x4 r = *(const u32x4*)(R + m * ldr + n);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const float lo = __uint_as_float(v[e] << 16) + __uint_as_float(r[e] << 16);
-                const float hi = __uint_as_float(v[e] & 0xffff0000u) + __uint_as_float(r[e] & 0xffff0000u);
-                v[e] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
-              }
-            }
-            *(u32x4*)dst = v;
-          } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-              if (n + e < N) {
-                bf16_t o = (bf16_t)((v[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
-                if (EPI == 2) o = f32_to_bf16(bf16_to_f32(o) + bf16_to_f32(R[m * ldr + n + e]));
-                dst[e] = o;
-              }
-          }
-        }
-      }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
+    staged_epilogue<BN, EPI, STAGES * STAGE>(acc, gsm, wave, lane, m0, n0, M, N, Y, ldy, R, ldr);
   }
 }
 
@@ -902,6 +915,191 @@ static int launch_ring(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, i
                        const bf16_t* r = nullptr, int64_t ldr = 0) {
   constexpr int LDS = 4 * (256 + BN) * 64;
   auto kern = linear_bf16_ring_kernel<BN, EPI>;
+  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+  constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;
+  dim3 grid((unsigned)(((N + OUT_COLS - 1) / OUT_COLS) * ((M + 255) / 256)));
+  MVPA_LAUNCH(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy, r, ldr);
+  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+}
+
+// -----------------------------------------------------------------------------------------
+// The large-tile kernel on two stages of 64-wide k-blocks (K a multiple of 64).
+// A request of the 32-wide ring covers 64 bytes of a row - half a cache line, whose other half
+// the next k-block asks for again, one k-block's worth of other lines (32 KiB per CU) later.  Here
+// a wave load covers 8 rows x 128 bytes, whole lines, and LDS holds two blocks of 64.  The order of a
+// block keeps what the ring gained: the barrier sits in front of the block's LAST quarter, whose
+// fragments are in registers by then (lgkmcnt 0 before it: nobody still reads the block); it
+// publishes the next block, whose first fragments are read under that last quarter's products, and
+// frees this block's stage, into which the block after next is requested at once - a full block's
+// time ahead of the barrier that will wait for it.  One request per block without a branch (past
+// the end the last block again, into a stage nobody reads), so the wait is a fixed vmcnt(0).
+// Same tile order, roles, row mapping and epilogues as the other large-tile kernels.
+// -----------------------------------------------------------------------------------------
+template <int BN, int EPI>
+__global__ __launch_bounds__(512) void linear_bf16_pair_kernel(const bf16_t* __restrict__ X,
+                                                               const bf16_t* __restrict__ W,
+                                                               bf16_t* __restrict__ Y, int64_t M,
+                                                               int64_t N, int64_t K, int64_t ldx,
+                                                               int64_t ldw, int64_t ldy,
+                                                               const bf16_t* __restrict__ R, int64_t ldr) {
+  constexpr int BM = 256, BK = 64, ROWB = BK * 2, STAGES = 2;
+  constexpr int WN = BN / 2, NB = WN / 32;            // per-wave extent over w rows
+  constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_LOADS = A_BYTES / 1024 / 8, B_LOADS = B_BYTES / 1024 / 8;   // 1 KiB wave loads per wave and block
+  static_assert(B_BYTES % (8 * 1024) == 0, "every wave issues the same number of loads");
+  static_assert(EPI != 1 || NB % 2 == 0, "gate/up pairs need an even number of sub-blocks");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char gsm[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 31, hh = lane >> 5;
+  const int wm = wave >> 1, wc = wave & 1;
+  constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;    // output columns per workgroup
+  int64_t tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, (M + BM - 1) / BM, (N + OUT_COLS - 1) / OUT_COLS, &tile_m, &tile_n);
+  const int64_t m0 = tile_m * BM, n0 = tile_n * OUT_COLS;
+  const int nkb = (int)(K / BK);
+
+  auto w_row = [&](int r) -> int64_t {                // which w row feeds tile row r
+    if (EPI == 1) {
+      const int wcol = r / WN, nb = (r % WN) / 32, i = r & 31;
+      const int64_t col = n0 + wcol * (WN / 2) + (nb >> 1) * 32 + i;
+      return ((nb & 1) ? N : 0) + (col < N ? col : N - 1);
+    }
+    const int64_t n = n0 + r;
+    return n < N ? n : N - 1;
+  };
+
+  // ---- the request side.  A wave load covers 8 tile rows x 128 bytes: lane L is row L/8, physical
+  // chunk L%8; per-lane byte offsets from wave-uniform bases (rows clamped into range: such rows
+  // are never stored).
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)gsm;
+  int iss_kb = 0;
+  uint32_t iss_lds = lds0;
+  const int64_t wrow0 = w_row(0);
+  const bf16_t* xs = X + m0 * ldx;
+  const bf16_t* ws = W + wrow0 * ldw;
+  uint32_t aoff[A_LOADS], boff[B_LOADS];
+  {
+    const int rsub = lane >> 3, phys = lane & 7;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int row = (wave + 8 * i) * 8 + rsub;
+      const int64_t m = m0 + row;
+      aoff[i] = (uint32_t)((((m < M ? m : M - 1) - m0) * ldx + ((phys ^ ((row >> 1) & 7)) << 3)) * 2);
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+      const int row = (wave + 8 * i) * 8 + rsub;
+      boff[i] = (uint32_t)(((w_row(row) - wrow0) * ldw + ((phys ^ ((row >> 1) & 7)) << 3)) * 2);
+    }
+  }
+  auto issue_block = [&]() {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(aoff[i]), "s"(xs), "s"(iss_lds + (wave + 8 * i) * 1024) : "memory", "m0");
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(boff[i]), "s"(ws), "s"(iss_lds + A_BYTES + (wave + 8 * i) * 1024) : "memory", "m0");
+    iss_lds = iss_lds == lds0 ? lds0 + STAGE : lds0;
+    if (iss_kb + 1 < nkb) {
+      ++iss_kb;
+      xs += BK;
+      ws += BK;
+    }
+  };
+
+  // fragment offsets: row ln of a 32-row block, chunk (2s+hh) ^ swizzle(ln) for the four 16-wide slices
+  int frag_off[4];
+#pragma unroll
+  for (int sl = 0; sl < 4; ++sl) frag_off[sl] = ln * ROWB + (((2 * sl + hh) ^ ((ln >> 1) & 7)) << 4);
+  const int a_lane = (wm * 64) * ROWB, b_lane = A_BYTES + (wc * WN) * ROWB;
+
+  issue_block();
+  issue_block();
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(A_LOADS + B_LOADS) : "memory");
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  bf16x8 xf0[2], wf0[NB];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) xf0[j] = *(const bf16x8*)(gsm + a_lane + j * 32 * ROWB + frag_off[0]);
+#pragma unroll
+  for (int i = 0; i < NB; ++i) wf0[i] = *(const bf16x8*)(gsm + b_lane + i * 32 * ROWB + frag_off[0]);
+  int cur = 0;                                        // stage of the block being multiplied
+
+  f32x16 acc[NB][2];
+#pragma unroll
+  for (int i = 0; i < NB; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  for (int kb = 0; kb < nkb; ++kb) {
+    const unsigned char* st = gsm + cur * STAGE;
+    cur ^= 1;
+    const unsigned char* sn = gsm + cur * STAGE;
+    bf16x8 xf1[2], wf1[NB];
+    // slices 0 .. 2: the fragments of slice s+1 are requested before the products of slice s
+#pragma unroll
+    for (int j = 0; j < 2; ++j) xf1[j] = *(const bf16x8*)(st + a_lane + j * 32 * ROWB + frag_off[1]);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) wf1[i] = *(const bf16x8*)(st + b_lane + i * 32 * ROWB + frag_off[1]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf0[i], xf0[j], acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) xf0[j] = *(const bf16x8*)(st + a_lane + j * 32 * ROWB + frag_off[2]);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) wf0[i] = *(const bf16x8*)(st + b_lane + i * 32 * ROWB + frag_off[2]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf1[i], xf1[j], acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) xf1[j] = *(const bf16x8*)(st + a_lane + j * 32 * ROWB + frag_off[3]);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) wf1[i] = *(const bf16x8*)(st + b_lane + i * 32 * ROWB + frag_off[3]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf0[i], xf0[j], acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    // the next block has landed, and every fragment of this one is in registers: publish / free
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+    for (int j = 0; j < 2; ++j) xf0[j] = *(const bf16x8*)(sn + a_lane + j * 32 * ROWB + frag_off[0]);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) wf0[i] = *(const bf16x8*)(sn + b_lane + i * 32 * ROWB + frag_off[0]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf1[i], xf1[j], acc[i][j], 0, 0, 0);
+        if (i == 0 && j == 0) {
+          __builtin_amdgcn_sched_barrier(0);
+          issue_block();                              // the block after next, into the stage just freed
+        }
+      }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  staged_epilogue<BN, EPI, STAGES * STAGE>(acc, gsm, wave, lane, m0, n0, M, N, Y, ldy, R, ldr);
+}
+
+template <int BN, int EPI>
+static int launch_pair(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, int64_t N, int64_t K,
+                       int64_t ldx, int64_t ldw, int64_t ldy, hipStream_t s,
+                       const bf16_t* r = nullptr, int64_t ldr = 0) {
+  constexpr int LDS = 2 * (256 + BN) * 128;
+  auto kern = linear_bf16_pair_kernel<BN, EPI>;
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
   constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;
   dim3 grid((unsigned)(((N + OUT_COLS - 1) / OUT_COLS) * ((M + 255) / 256)));
@@ -1243,22 +1441,29 @@ extern "C" int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M
     // the four-stage ring needs whole k-blocks of 32 and 32-bit byte offsets from a tile's first rows
     const bool ring = (K & 31) == 0 && K >= 96 && 256 * ldx < ((int64_t)1 << 30) &&
                       (epilogue == 1 ? 2 * N : (int64_t)256) * ldw < ((int64_t)1 << 30);
+    // whole cache lines per request where K is a multiple of 64
+    const bool pair = ring && (K & 63) == 0 && K >= 128;
     if (epilogue == 1) {
       // (the wider tile unless it costs a fifth more: [16384 x 768] x [768 x 3456] 114 -> 103 us)
       if (cost(256, 128) * 5 <= cost(128, 64) * 6)
-        return ring ? launch_ring<256, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+        return pair ? launch_pair<256, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+           : ring ? launch_ring<256, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
                     : launch_big<256, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
-      return ring ? launch_ring<128, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+      return pair ? launch_pair<128, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+           : ring ? launch_ring<128, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
                   : launch_big<128, 1>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
     }
     const int64_t c256 = cost(256, 256), c192 = cost(192, 192), c128 = cost(128, 128);
     if (c256 <= c192 && c256 <= c128)
-      return ring ? launch_ring<256, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+      return pair ? launch_pair<256, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+           : ring ? launch_ring<256, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
                   : launch_big<256, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
     if (c192 <= c128)
-      return ring ? launch_ring<192, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+      return pair ? launch_pair<192, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+           : ring ? launch_ring<192, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
                   : launch_big<192, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
-    return ring ? launch_ring<128, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+    return pair ? launch_pair<128, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
+           : ring ? launch_ring<128, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s)
                 : launch_big<128, 0>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s);
   }
   if (M <= 128) {
@@ -1296,9 +1501,15 @@ extern "C" int mvpa_linear_bf16_residual(const void* x, const void* w, const voi
   const int64_t mt = (M + 255) / 256;
   auto cost = [&](int bn) -> int64_t { return ((mt * ((N + bn - 1) / bn) + 255) / 256) * bn; };
   const int64_t c256 = cost(256), c192 = cost(192), c128 = cost(128);
-  if (c256 <= c192 && c256 <= c128) return launch_ring<256, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s, rp, ldr);
-  if (c192 <= c128) return launch_ring<192, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s, rp, ldr);
-  return launch_ring<128, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s, rp, ldr);
+  const bool pair = (K & 63) == 0 && K >= 128;
+  if (c256 <= c192 && c256 <= c128)
+    return pair ? launch_pair<256, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s, rp, ldr)
+                : launch_ring<256, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s, rp, ldr);
+  if (c192 <= c128)
+    return pair ? launch_pair<192, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s, rp, ldr)
+                : launch_ring<192, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s, rp, ldr);
+  return pair ? launch_pair<128, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s, rp, ldr)
+              : launch_ring<128, 2>(xp, wp, yp, M, N, K, ldx, ldw, ldy, s, rp, ldr);
 }
 
 extern "C" int mvpa_rmsnorm(const void* x, const float* weight, void* y, int64_t rows,
