@@ -289,6 +289,16 @@ int mvpa_rmsnorm(const void* x, const float* weight, void* y, int64_t rows, int3
                  int64_t ldx, int64_t ldy, float eps, int32_t in_dtype, int32_t out_dtype,
                  void* stream);
 
+/* Cosine similarity of row pairs in fp32: out[g * rows_per_group + r] = a_gr . b_gr /
+ * (max(|a_gr|, eps) * max(|b_gr|, eps)) with a_gr = a + g * group_stride_a + r * lda (elements;
+ * cols a multiple of 8, 16-byte aligned rows).  The generative score of the reference,
+ * torch.cosine_similarity(next segment's encoding, head's prediction, dim=-1)
+ * (models/mvpformer.py:749-764), in one pass over both tensors: a group is one batch entry, its
+ * rows "all time steps but the first" of one tensor against "all but the last" of the other. */
+int mvpa_cosine_rows_bf16(const void* a, const void* b, float* out, int64_t groups,
+                          int64_t rows_per_group, int32_t cols, int64_t lda, int64_t ldb,
+                          int64_t group_stride_a, int64_t group_stride_b, float eps, void* stream);
+
 /* out = a + b + c elementwise, bf16 (models/mvpformer.py:147 residual + mlp + attn). */
 int mvpa_add3_bf16(const void* a, const void* b, const void* c, void* out, int64_t n,
                    void* stream);

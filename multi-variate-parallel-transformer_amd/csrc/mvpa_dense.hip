@@ -1201,6 +1201,41 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const TI* __restrict_
   }
 }
 
+// Cosine similarity of row pairs: out[r] = a_r . b_r / (max(|a_r|, eps) * max(|b_r|, eps)), fp32
+// arithmetic, one wave per row pair.  Rows come in groups (a batch entry each) of rows_per_group
+// consecutive rows, group g starting at a + g * group_stride_a (elements), so that "all time steps
+// but the first" of one tensor can be paired with "all but the last" of another without copies.
+__global__ __launch_bounds__(256) void cosine_rows_bf16_kernel(const bf16_t* __restrict__ a,
+                                                               const bf16_t* __restrict__ b,
+                                                               float* __restrict__ out, int64_t rows,
+                                                               int64_t rows_per_group, int cols,
+                                                               int64_t lda, int64_t ldb,
+                                                               int64_t group_stride_a,
+                                                               int64_t group_stride_b, float eps) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t g = row / rows_per_group, r = row % rows_per_group;
+  const bf16_t* ar = a + g * group_stride_a + r * lda;
+  const bf16_t* br = b + g * group_stride_b + r * ldb;
+  float dot = 0.f, na = 0.f, nb = 0.f;
+  for (int c = lane * 8; c < cols; c += 512) {
+    float x[8], y[8];
+    vec8<bf16_t>::load(ar + c, x);
+    vec8<bf16_t>::load(br + c, y);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      dot += x[i] * y[i];
+      na += x[i] * x[i];
+      nb += y[i] * y[i];
+    }
+  }
+  dot = wave_sum(dot);
+  na = wave_sum(na);
+  nb = wave_sum(nb);
+  if (lane == 0) out[row] = dot / (fmaxf(sqrtf(na), eps) * fmaxf(sqrtf(nb), eps));
+}
+
 // sum = bf16(a + b + c) and norm = RMSNorm(sum) * w in one pass over the three inputs: the
 // residual update of one block fused with the input norm of the next.  The norm is taken over
 // the ROUNDED sum, so the result equals the two separate kernels bit for bit.
@@ -1546,6 +1581,22 @@ extern "C" int mvpa_rmsnorm(const void* x, const float* weight, void* y, int64_t
     MVPA_LAUNCH((rmsnorm_kernel<bf16_t, float>), grid, block, 0, s, (const bf16_t*)x, weight, (float*)y, cols, ldx, ldy, eps);
   else
     return MVPA_ERR_DTYPE;
+  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+}
+
+extern "C" int mvpa_cosine_rows_bf16(const void* a, const void* b, float* out, int64_t groups,
+                                     int64_t rows_per_group, int32_t cols, int64_t lda, int64_t ldb,
+                                     int64_t group_stride_a, int64_t group_stride_b, float eps,
+                                     void* stream) {
+  if (!a || !b || !out) return MVPA_ERR_NULL;
+  if (groups <= 0 || rows_per_group <= 0 || cols <= 0 || lda < cols || ldb < cols) return MVPA_ERR_SHAPE;
+  if ((cols & 7) || (lda & 7) || (ldb & 7) || (group_stride_a & 7) || (group_stride_b & 7) ||
+      (((uintptr_t)a | (uintptr_t)b) & 15))
+    return MVPA_ERR_ALIGN;
+  const int64_t rows = groups * rows_per_group;
+  MVPA_LAUNCH(cosine_rows_bf16_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+              (const bf16_t*)a, (const bf16_t*)b, out, rows, rows_per_group, cols, lda, ldb,
+              group_stride_a, group_stride_b, eps);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 

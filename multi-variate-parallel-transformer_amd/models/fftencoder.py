@@ -44,13 +44,17 @@ class WaveEncoder(BrainEncoder):
         """[M, L] -> [M, dwt_size] float32 coefficients [cA_L, cD_L, ..., cD_1]."""
         return mvpa_hip.wavedec_db4(x.float())
 
+    def _padded_k(self) -> int:
+        """dwt_size (550 for 512-sample segments) rounded up to whole 64-element k-blocks: the
+        GEMM then fetches whole cache lines and needs no tail block."""
+        return (self.dwt_size + 63) // 64 * 64
+
     def _padded_weight(self) -> Tensor:
-        """bf16 copy of proj.weight with its rows padded to a multiple of 8 elements, so the GEMM
-        can use 16-byte loads although dwt_size (550 for 512-sample segments) is odd-sized."""
+        """bf16 copy of proj.weight with its rows zero-padded to _padded_k() elements."""
         w = self.proj.weight
         key = (w.data_ptr(), w._version)
         if self._proj_key != key:
-            kp = (self.dwt_size + 7) // 8 * 8
+            kp = self._padded_k()
             buf = torch.zeros((w.shape[0], kp), dtype=torch.bfloat16, device=w.device)
             buf[:, : self.dwt_size] = w.detach().to(torch.bfloat16)
             self._proj_padded, self._proj_key = buf, key
@@ -60,9 +64,10 @@ class WaveEncoder(BrainEncoder):
     def forward(self, x: Tensor) -> Tensor:
         """x [M, L] -> [M, size_output]; bf16 output (the model's compute dtype)."""
         m = x.shape[0]
-        kp = (self.dwt_size + 7) // 8 * 8
-        coeffs = mvpa_hip.wavedec_db4(x.float(), pitch=kp)               # [M, dwt] view, pitch kp
-        normed = torch.zeros((m, kp), dtype=torch.bfloat16, device=x.device)
+        kp = self._padded_k()
+        coeffs = mvpa_hip.wavedec_db4(x.float(), pitch=kp, zero_pad=False)   # [M, dwt] view, pitch kp
+        normed = torch.empty((m, kp), dtype=torch.bfloat16, device=x.device)
+        normed[:, self.dwt_size:].zero_()
         mvpa_hip.rmsnorm(coeffs, self.ln.weight, 1e-5, out=normed[:, : self.dwt_size])
         w = self._padded_weight()
         return mvpa_hip.linear(normed, w)          # the zero padding contributes nothing

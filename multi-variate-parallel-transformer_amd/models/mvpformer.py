@@ -446,6 +446,8 @@ class HMVPFormer(BrainModel):
         prediction at segment t and the encoding of segment t+1, per channel."""
         out, enc = self._common_forward(batch)
         out = self.head(out)
+        if enc.is_cuda and enc.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and enc.shape[-1] % 8 == 0:
+            return mvpa_hip.cosine_similarity_steps(enc, out)
         return torch.cosine_similarity(enc[:, 1:].float(), out[:, :-1].float(), dim=-1)
 
     @torch.no_grad()

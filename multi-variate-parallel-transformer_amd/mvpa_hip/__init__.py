@@ -112,6 +112,8 @@ def load_library() -> ctypes.CDLL:
     lib.mvpa_debug_maps.argtypes = [i32, i32, i32, u32, vp, vp, vp, vp, vp]
     lib.mvpa_linear_bf16.restype = ctypes.c_int
     lib.mvpa_linear_bf16.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, i32, vp]
+    lib.mvpa_cosine_rows_bf16.restype = ctypes.c_int
+    lib.mvpa_cosine_rows_bf16.argtypes = [vp, vp, vp, i64, i64, i32, i64, i64, i64, i64, ctypes.c_float, vp]
     lib.mvpa_linear_bf16_residual.restype = ctypes.c_int
     lib.mvpa_linear_bf16_residual.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp]
     lib.mvpa_rmsnorm.restype = ctypes.c_int
@@ -439,6 +441,26 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = 
     return out if given else out.view(*x.shape[:-1], N)
 
 
+def cosine_similarity_steps(nxt: torch.Tensor, pred: torch.Tensor, eps: float = 1e-8) -> torch.Tensor:
+    """torch.cosine_similarity(nxt[:, 1:], pred[:, :-1], dim=-1) for two bf16 tensors [B, T, C, E]
+    (the reference's generative score, models/mvpformer.py:749-764) in one kernel, fp32 result
+    [B, T-1, C]."""
+    lib = load_library()
+    _need_cuda(nxt, pred)
+    if nxt.dtype != torch.bfloat16 or pred.dtype != torch.bfloat16:
+        raise TypeError("cosine_similarity_steps: bf16 only")
+    if nxt.shape != pred.shape or nxt.dim() != 4:
+        raise ValueError("cosine_similarity_steps: two tensors [B, T, C, E] of one shape")
+    nxt, pred = nxt.contiguous(), pred.contiguous()
+    B, T, C, E = nxt.shape
+    out = torch.empty((B, max(T - 1, 0), C), dtype=torch.float32, device=nxt.device)
+    if T > 1 and B > 0 and C > 0:
+        a = nxt[:, 1:]
+        _check(lib.mvpa_cosine_rows_bf16(a.data_ptr(), pred.data_ptr(), out.data_ptr(), B, (T - 1) * C, E,
+                                         E, E, T * C * E, T * C * E, eps, _stream()))
+    return out
+
+
 def _as_f32_weight(weight: torch.Tensor) -> torch.Tensor:
     """fp32 contiguous copy of a (norm) weight, kept on the tensor object and refreshed when the
     tensor is modified in place, so a bf16 module does not convert its weight on every call."""
@@ -542,9 +564,10 @@ def dwt_sizes(size_input: int):
     return levels, sizes
 
 
-def wavedec_db4(x: torch.Tensor, pitch: Optional[int] = None) -> torch.Tensor:
+def wavedec_db4(x: torch.Tensor, pitch: Optional[int] = None, zero_pad: bool = True) -> torch.Tensor:
     """x [M,L] float32 -> coefficients [M,dwt_size] float32, ordered [cA_L, cD_L, .., cD_1].
-    With `pitch` the result is a [M,dwt_size] view of a zero-filled [M,pitch] buffer."""
+    With `pitch` the result is a [M,dwt_size] view of a [M,pitch] buffer, zero-filled unless
+    zero_pad is False (the columns past dwt_size are then undefined)."""
     lib = load_library()
     _need_cuda(x)
     x = x.to(torch.float32).contiguous()
@@ -552,6 +575,6 @@ def wavedec_db4(x: torch.Tensor, pitch: Optional[int] = None) -> torch.Tensor:
     levels, sizes = dwt_sizes(L)
     total = sum(sizes)
     ldc = total if pitch is None else pitch
-    buf = (torch.empty if ldc == total else torch.zeros)((M, ldc), dtype=torch.float32, device=x.device)
+    buf = (torch.empty if ldc == total or not zero_pad else torch.zeros)((M, ldc), dtype=torch.float32, device=x.device)
     _check(lib.mvpa_wavedec_db4(x.data_ptr(), buf.data_ptr(), M, L, levels, total, ldc, _stream()))
     return buf[:, :total]

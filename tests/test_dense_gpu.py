@@ -77,6 +77,21 @@ def test_linear_with_residual_refuses_small_shapes():
         mvpa_hip.linear(x, w, residual=x)
 
 
+@pytest.mark.parametrize("B,T,C,E", [(4, 64, 64, 768), (1, 2, 3, 8), (2, 5, 7, 1032), (3, 1, 4, 64)])
+def test_cosine_similarity_of_consecutive_steps(B, T, C, E):
+    """The generative score in one kernel against torch.cosine_similarity on the fp32 values."""
+    g = torch.Generator().manual_seed(B * T + C)
+    a = torch.randn(B, T, C, E, generator=g).bfloat16()
+    b = (torch.randn(B, T, C, E, generator=g) * 3).bfloat16()
+    b[0, 0, 0] = 0                                   # a zero row: eps keeps it finite
+    out = mvpa_hip.cosine_similarity_steps(a.cuda(), b.cuda()).cpu()
+    assert out.shape == (B, T - 1, C) and out.dtype == torch.float32
+    if T > 1:
+        ref = torch.cosine_similarity(a[:, 1:].double(), b[:, :-1].double(), dim=-1)
+        assert torch.isfinite(out).all()
+        assert (out.double() - ref).abs().max().item() <= 2e-6
+
+
 def test_linear_into_a_column_slice():
     """The gated product written into a column slice of a wider buffer (the block's tail operand)."""
     g = torch.Generator().manual_seed(9)
