@@ -271,6 +271,16 @@ int mvpa_linear_bf16_residual(const void* x, const void* w, const void* r, void*
                               int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldr,
                               int64_t ldy, void* stream);
 
+/* Two products on one x in one launch: y0[M,N0] = x @ w0^T and y1[M,N1] = silu(x @ wg^T) * (x @ wu^T)
+ * with w1 holding the gate rows [0,N1) and the up rows [N1,2*N1) - the fused q/kv projection
+ * (layers/mvpa.py:354-356) and the MLP's gate/up product (models/mvpformer.py:146), which both read
+ * ln_1(x) in the parallel block.  Launched separately each product ends on a partly filled round
+ * of tiles; in one grid only their sum does.  Large shapes only: M >= 512, K a multiple of 64;
+ * MVPA_ERR_UNSUPPORTED otherwise. */
+int mvpa_linear_bf16_dual(const void* x, const void* w0, void* y0, const void* w1, void* y1, int64_t M,
+                          int64_t N0, int64_t N1, int64_t K, int64_t ldx, int64_t ldw0, int64_t ldy0,
+                          int64_t ldw1, int64_t ldy1, void* stream);
+
 /* The same product for at most 128 rows of x against a large weight (the projections of one
  * decoding step of a wide model), with K split over workgroups: fp32 partial tiles go through the
  * caller's workspace ws (mvpa_linear_splitk_ws_bytes(M, N, K, epilogue) bytes, 16-byte aligned)

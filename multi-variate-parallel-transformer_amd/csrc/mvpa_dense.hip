@@ -936,19 +936,17 @@ static int launch_ring(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, i
 // Same tile order, roles, row mapping and epilogues as the other large-tile kernels.
 // -----------------------------------------------------------------------------------------
 template <int BN, int EPI>
-__global__ __launch_bounds__(512) void linear_bf16_pair_kernel(const bf16_t* __restrict__ X,
-                                                               const bf16_t* __restrict__ W,
-                                                               bf16_t* __restrict__ Y, int64_t M,
-                                                               int64_t N, int64_t K, int64_t ldx,
-                                                               int64_t ldw, int64_t ldy,
-                                                               const bf16_t* __restrict__ R, int64_t ldr) {
+__device__ __forceinline__ void linear_pair_tile(int64_t tile, unsigned char* gsm,
+                                                 const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+                                                 bf16_t* __restrict__ Y, int64_t M, int64_t N, int64_t K,
+                                                 int64_t ldx, int64_t ldw, int64_t ldy,
+                                                 const bf16_t* __restrict__ R, int64_t ldr) {
   constexpr int BM = 256, BK = 64, ROWB = BK * 2, STAGES = 2;
   constexpr int WN = BN / 2, NB = WN / 32;            // per-wave extent over w rows
   constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
   constexpr int A_LOADS = A_BYTES / 1024 / 8, B_LOADS = B_BYTES / 1024 / 8;   // 1 KiB wave loads per wave and block
   static_assert(B_BYTES % (8 * 1024) == 0, "every wave issues the same number of loads");
   static_assert(EPI != 1 || NB % 2 == 0, "gate/up pairs need an even number of sub-blocks");
-  extern __shared__ __attribute__((aligned(1024))) unsigned char gsm[];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -956,7 +954,7 @@ __global__ __launch_bounds__(512) void linear_bf16_pair_kernel(const bf16_t* __r
   const int wm = wave >> 1, wc = wave & 1;
   constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;    // output columns per workgroup
   int64_t tile_m, tile_n;
-  tile_of_workgroup(blockIdx.x, (M + BM - 1) / BM, (N + OUT_COLS - 1) / OUT_COLS, &tile_m, &tile_n);
+  tile_of_workgroup(tile, (M + BM - 1) / BM, (N + OUT_COLS - 1) / OUT_COLS, &tile_m, &tile_n);
   const int64_t m0 = tile_m * BM, n0 = tile_n * OUT_COLS;
   const int nkb = (int)(K / BK);
 
@@ -1095,6 +1093,42 @@ __global__ __launch_bounds__(512) void linear_bf16_pair_kernel(const bf16_t* __r
 }
 
 template <int BN, int EPI>
+__global__ __launch_bounds__(512) void linear_bf16_pair_kernel(const bf16_t* __restrict__ X,
+                                                               const bf16_t* __restrict__ W,
+                                                               bf16_t* __restrict__ Y, int64_t M,
+                                                               int64_t N, int64_t K, int64_t ldx,
+                                                               int64_t ldw, int64_t ldy,
+                                                               const bf16_t* __restrict__ R, int64_t ldr) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char gsm[];
+  linear_pair_tile<BN, EPI>(blockIdx.x, gsm, X, W, Y, M, N, K, ldx, ldw, ldy, R, ldr);
+}
+
+// Two products of one launch: y0 = x w0^T (tiles 256 x BN0) and y1 = silu(x wg^T) * (x wu^T)
+// (tiles 256 x 256), both on the same x.  Launched one after the other, each product ends on a
+// round of tiles that fills part of the chip; in one grid - the gated product's tiles first, they
+// are the longer ones - only the sum does.
+struct linear_pair_problem {
+  const bf16_t* w;
+  bf16_t* y;
+  int64_t N, ldw, ldy;
+};
+
+template <int BN0>
+__global__ __launch_bounds__(512) void linear_bf16_pair_dual_kernel(const bf16_t* __restrict__ X, int64_t M,
+                                                                    int64_t K, int64_t ldx,
+                                                                    linear_pair_problem plain,
+                                                                    linear_pair_problem gated,
+                                                                    int64_t gated_tiles) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char gsm[];
+  const int64_t L = blockIdx.x;
+  if (L < gated_tiles)
+    linear_pair_tile<256, 1>(L, gsm, X, gated.w, gated.y, M, gated.N, K, ldx, gated.ldw, gated.ldy, nullptr, 0);
+  else
+    linear_pair_tile<BN0, 0>(L - gated_tiles, gsm, X, plain.w, plain.y, M, plain.N, K, ldx, plain.ldw, plain.ldy,
+                             nullptr, 0);
+}
+
+template <int BN, int EPI>
 static int launch_pair(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, int64_t N, int64_t K,
                        int64_t ldx, int64_t ldw, int64_t ldy, hipStream_t s,
                        const bf16_t* r = nullptr, int64_t ldr = 0) {
@@ -1104,6 +1138,19 @@ static int launch_pair(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, i
   constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;
   dim3 grid((unsigned)(((N + OUT_COLS - 1) / OUT_COLS) * ((M + 255) / 256)));
   MVPA_LAUNCH(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy, r, ldr);
+  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+}
+
+template <int BN0>
+static int launch_pair_dual(const bf16_t* x, int64_t M, int64_t K, int64_t ldx, const mvpa::linear_pair_problem& plain,
+                            const mvpa::linear_pair_problem& gated, hipStream_t s) {
+  constexpr int LDS = 2 * (256 + 256) * 128;
+  auto kern = linear_bf16_pair_dual_kernel<BN0>;
+  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+  const int64_t mt = (M + 255) / 256;
+  const int64_t gated_tiles = mt * ((gated.N + 127) / 128), plain_tiles = mt * ((plain.N + BN0 - 1) / BN0);
+  MVPA_LAUNCH(kern, dim3((unsigned)(gated_tiles + plain_tiles)), dim3(512), LDS, s, x, M, K, ldx, plain, gated,
+              gated_tiles);
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 
@@ -1516,6 +1563,31 @@ extern "C" int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M
     MVPA_LAUNCH(linear_bf16_kernel<0>, grid, dim3(256), 0, s, xp, wp, yp, M, N, K, ldx, ldw, ldy);
   }
   return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+}
+
+// y0 = x w0^T and y1 = silu(x wg^T) * (x wu^T) in one launch (w1 holds the gate rows [0, N1) and
+// the up rows [N1, 2 N1)): the two products that read ln_1(x) in the parallel block.  Large
+// shapes only: at least 512 rows, K a multiple of 64; MVPA_ERR_UNSUPPORTED otherwise.
+extern "C" int mvpa_linear_bf16_dual(const void* x, const void* w0, void* y0, const void* w1, void* y1,
+                                     int64_t M, int64_t N0, int64_t N1, int64_t K, int64_t ldx,
+                                     int64_t ldw0, int64_t ldy0, int64_t ldw1, int64_t ldy1, void* stream) {
+  if (!x || !w0 || !y0 || !w1 || !y1) return MVPA_ERR_NULL;
+  if (M <= 0 || N0 <= 0 || N1 <= 0 || K <= 0 || ldx < K || ldw0 < K || ldw1 < K || ldy0 < N0 || ldy1 < N1)
+    return MVPA_ERR_SHAPE;
+  if ((((uintptr_t)x | (uintptr_t)w0 | (uintptr_t)w1) & 15) || (ldx & 7) || (ldw0 & 7) || (ldw1 & 7))
+    return MVPA_ERR_ALIGN;
+  if (((uintptr_t)y0 | (uintptr_t)y1) & 1) return MVPA_ERR_ALIGN;
+  const bool ok = M >= 512 && (K & 63) == 0 && K >= 128 && 256 * ldx < ((int64_t)1 << 30) &&
+                  256 * ldw0 < ((int64_t)1 << 30) && 2 * N1 * ldw1 < ((int64_t)1 << 30);
+  if (!ok) return MVPA_ERR_UNSUPPORTED;
+  const mvpa::linear_pair_problem plain{(const bf16_t*)w0, (bf16_t*)y0, N0, ldw0, ldy0};
+  const mvpa::linear_pair_problem gated{(const bf16_t*)w1, (bf16_t*)y1, N1, ldw1, ldy1};
+  // the plain product's tile width: the one that wastes the fewest padded columns
+  const int64_t pad256 = (N0 + 255) / 256 * 256, pad192 = (N0 + 191) / 192 * 192, pad128 = (N0 + 127) / 128 * 128;
+  hipStream_t s = (hipStream_t)stream;
+  if (pad256 <= pad192 && pad256 <= pad128) return launch_pair_dual<256>((const bf16_t*)x, M, K, ldx, plain, gated, s);
+  if (pad192 <= pad128) return launch_pair_dual<192>((const bf16_t*)x, M, K, ldx, plain, gated, s);
+  return launch_pair_dual<128>((const bf16_t*)x, M, K, ldx, plain, gated, s);
 }
 
 // Y = X W^T + R in one kernel (the large-tile ring kernel only): at least 512 rows, K a multiple

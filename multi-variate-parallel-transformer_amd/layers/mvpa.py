@@ -300,9 +300,10 @@ class MVPFormerGQAAttention(torch.nn.Module):
         return bool(self.global_att)                       # layers/mvpa.py:188-222, 230
 
     def _attend(self, hidden_states, positional_embedding, channel_embedding, attention_mask,
-                head_mask, use_cache, window, layer_past=None, merged_out=None):
+                head_mask, use_cache, window, layer_past=None, merged_out=None, qkv=None):
         """merged_out: a [B, T*C, H, Dh] view (unit last stride, any row pitch) that receives the
-        merged heads; c_proj is then left to the caller and merged_out is what comes back."""
+        merged heads; c_proj is then left to the caller and merged_out is what comes back.
+        qkv: hidden_states @ [q_attn; c_attn]^T when the caller has already formed it."""
         if self.training and (self.attn_dropout.p > 0 or self.resid_dropout.p > 0):
             raise NotImplementedError("MVPA HIP layer: dropout/training is not implemented; call .eval()")
         if self.is_cross_attention:
@@ -319,7 +320,8 @@ class MVPFormerGQAAttention(torch.nn.Module):
             return self._attend_step(hidden_states, positional_embedding, channel_embedding,
                                      attention_mask, head_mask, use_cache, window, layer_past)
         with torch.no_grad():
-            qkv = _linear(hidden_states, self._qkv_weight(dt))          # [B,T,C,E+2kvE]
+            if qkv is None:
+                qkv = _linear(hidden_states, self._qkv_weight(dt))      # [B,T,C,E+2kvE]
             row = e + 2 * kv
             qkv = qkv.view(bsz, n, row)
             q = qkv[:, :, :e].view(bsz, n, h, dh).permute(0, 2, 1, 3)        # views, no copy
@@ -454,14 +456,20 @@ class MVPFormerGQAAttention(torch.nn.Module):
 
 
     def forward_merged(self, hidden_states, positional_embedding, channel_embedding, merged_out,
-                       attention_mask=None, head_mask=None, use_cache=False):
+                       attention_mask=None, head_mask=None, use_cache=False, qkv=None):
         """forward() up to the merged heads: they are written into merged_out ([B, T*C, H, Dh], unit
         last stride, any row pitch) and c_proj (layers/mvpa.py:400) is left to the caller, who can
-        fold it into a later product.  Returns (merged_out, present)."""
+        fold it into a later product.  qkv: the fused q/kv projection of hidden_states
+        (hidden_states @ qkv_weight()^T, contiguous) if the caller has formed it with another
+        product.  Returns (merged_out, present)."""
         if not self._honours_masks:
             attention_mask, head_mask = None, None
         return self._attend(hidden_states, positional_embedding, channel_embedding, attention_mask,
-                            head_mask, use_cache, window=10, merged_out=merged_out)
+                            head_mask, use_cache, window=10, merged_out=merged_out, qkv=qkv)
+
+    def qkv_weight(self, dtype=torch.bfloat16) -> torch.Tensor:
+        """[q_attn; c_attn] stacked (adapters folded in), cached until a weight changes."""
+        return self._qkv_weight(dtype)
 
 
 class MVPFormerGQAFlashAttention(MVPFormerGQAAttention):

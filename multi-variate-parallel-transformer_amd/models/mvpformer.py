@@ -98,6 +98,10 @@ class GatedMLP(nn.Module):
         mid = mvpa_hip.linear(x, self._gate_up(), gated=True)
         return mvpa_hip.linear(mid, self.down_proj.weight.to(torch.bfloat16))
 
+    def gate_up_weight(self) -> torch.Tensor:
+        """[gate_proj; up_proj] stacked in bf16, cached until a weight changes."""
+        return self._gate_up()
+
     @torch.no_grad()
     def activations_into(self, x, out):
         """silu(gate(x)) * up(x) written into out, a [rows, intermediate] view of any row pitch:
@@ -162,9 +166,17 @@ class MVPFormerBlock(nn.Module):
             h, dh = self.attn.num_heads, self.attn.head_dim
             both = torch.empty((rows, e + inner), dtype=torch.bfloat16, device=residual.device)
             merged = both[:, :e].unflatten(0, (bsz, t_len * c_len)).unflatten(2, (h, dh))
-            _, present = self.attn.forward_merged(normed, positional_embedding, channel_embedding, merged,
-                                                  attention_mask=attention_mask, use_cache=use_cache)
-            self.mlp.activations_into(normed.reshape(rows, e), both[:, e:])
+            if mvpa_hip.linear_dual_supported(rows, e):
+                # the two products that read ln_1(x), q/kv and gate/up, as one grid of tiles
+                qkv, _ = mvpa_hip.linear_dual(normed.reshape(rows, e), self.attn.qkv_weight(),
+                                              self.mlp.gate_up_weight(), out_gated=both[:, e:])
+                _, present = self.attn.forward_merged(normed, positional_embedding, channel_embedding, merged,
+                                                      attention_mask=attention_mask, use_cache=use_cache,
+                                                      qkv=qkv)
+            else:
+                _, present = self.attn.forward_merged(normed, positional_embedding, channel_embedding, merged,
+                                                      attention_mask=attention_mask, use_cache=use_cache)
+                self.mlp.activations_into(normed.reshape(rows, e), both[:, e:])
             hidden_states = mvpa_hip.linear(both, self._tail_weight(),
                                             residual=residual.reshape(rows, e)).view(residual.shape)
             next_normed = next_norm(hidden_states) if next_norm is not None else None

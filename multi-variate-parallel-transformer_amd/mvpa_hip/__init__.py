@@ -112,6 +112,8 @@ def load_library() -> ctypes.CDLL:
     lib.mvpa_debug_maps.argtypes = [i32, i32, i32, u32, vp, vp, vp, vp, vp]
     lib.mvpa_linear_bf16.restype = ctypes.c_int
     lib.mvpa_linear_bf16.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, i32, vp]
+    lib.mvpa_linear_bf16_dual.restype = ctypes.c_int
+    lib.mvpa_linear_bf16_dual.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, i64, vp]
     lib.mvpa_cosine_rows_bf16.restype = ctypes.c_int
     lib.mvpa_cosine_rows_bf16.argtypes = [vp, vp, vp, i64, i64, i32, i64, i64, i64, i64, ctypes.c_float, vp]
     lib.mvpa_linear_bf16_residual.restype = ctypes.c_int
@@ -384,6 +386,39 @@ def debug_maps(T: int, C: int, window: int = 10, flags: int = 15, chan_valid=Non
 def linear_residual_supported(M: int, K: int) -> bool:
     """Shapes mvpa_linear_bf16_residual takes (the large-tile kernel: see include/mvpa_hip.h)."""
     return M >= 512 and K % 32 == 0 and K >= 96
+
+
+def linear_dual_supported(M: int, K: int) -> bool:
+    """Shapes mvpa_linear_bf16_dual takes (see include/mvpa_hip.h)."""
+    return M >= 512 and K % 64 == 0 and K >= 128
+
+
+def linear_dual(x: torch.Tensor, w_plain: torch.Tensor, w_gated: torch.Tensor,
+                out_plain: Optional[torch.Tensor] = None, out_gated: Optional[torch.Tensor] = None):
+    """(x @ w_plain.T, silu(x @ gate.T) * (x @ up.T)) from ONE launch; w_gated stacks [gate; up]
+    rows.  x is [rows, K] (or any shape with K last, contiguous); the outputs are 2-D, and either
+    may be a given [rows, N] view with unit last stride (a column slice of a wider buffer)."""
+    lib = load_library()
+    _need_cuda(x, w_plain, w_gated)
+    if x.dtype != torch.bfloat16 or w_plain.dtype != torch.bfloat16 or w_gated.dtype != torch.bfloat16:
+        raise TypeError("linear_dual: bf16 only")
+    K = x.shape[-1]
+    x2 = x if x.dim() == 2 and x.stride(-1) == 1 else x.reshape(-1, K)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    M, N0, N1 = x2.shape[0], w_plain.shape[0], w_gated.shape[0] // 2
+    assert w_plain.shape[1] == K and w_gated.shape[1] == K and w_plain.stride(1) == 1 and w_gated.stride(1) == 1
+    outs = []
+    for o, n in ((out_plain, N0), (out_gated, N1)):
+        if o is None:
+            o = torch.empty((M, n), dtype=torch.bfloat16, device=x.device)
+        elif o.dim() != 2 or tuple(o.shape) != (M, n) or o.stride(1) != 1 or o.dtype != torch.bfloat16:
+            raise ValueError("linear_dual: outputs must be bf16 [rows, N] tensors or views with unit last stride")
+        outs.append(o)
+    _check(lib.mvpa_linear_bf16_dual(x2.data_ptr(), w_plain.data_ptr(), outs[0].data_ptr(), w_gated.data_ptr(),
+                                     outs[1].data_ptr(), M, N0, N1, K, x2.stride(0), w_plain.stride(0),
+                                     outs[0].stride(0), w_gated.stride(0), outs[1].stride(0), _stream()))
+    return outs[0], outs[1]
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None,

@@ -105,6 +105,9 @@ def test_dense_entry_points_reject_bad_arguments(lib):
     assert lib.mvpa_linear_bf16_residual(None, None, None, None, 1, 1, 1, 1, 1, 1, 1, None) == -1
     assert lib.mvpa_linear_bf16_residual(p16, p16, p16, p16, 4, 4, 8, 8, 8, 2, 4, None) == -5     # ldr < N
     assert lib.mvpa_linear_bf16_residual(p16, p16, p16, p16, 4, 4, 8, 8, 8, 4, 4, None) < 0        # too small for the tiled kernel
+    assert lib.mvpa_linear_bf16_dual(None, None, None, None, None, 1, 1, 1, 1, 1, 1, 1, 1, 1, None) == -1
+    assert lib.mvpa_linear_bf16_dual(p16, p16, p16, p16, p16, 4, 4, 4, 8, 8, 8, 2, 8, 4, None) == -5   # ldy0 < N0
+    assert lib.mvpa_linear_bf16_dual(p16, p16, p16, p16, p16, 4, 4, 4, 8, 8, 8, 4, 8, 4, None) < 0      # too small
     assert lib.mvpa_cosine_rows_bf16(None, None, None, 1, 1, 8, 8, 8, 8, 8, 1e-8, None) == -1
     assert lib.mvpa_cosine_rows_bf16(p16, p16, p16, 1, 1, 12, 16, 16, 16, 16, 1e-8, None) == -7   # cols not a multiple of 8
     assert lib.mvpa_rmsnorm(None, None, None, 1, 1, 1, 1, 1e-5, 0, 0, None) == -1

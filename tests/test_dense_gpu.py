@@ -92,6 +92,30 @@ def test_cosine_similarity_of_consecutive_steps(B, T, C, E):
         assert (out.double() - ref).abs().max().item() <= 2e-6
 
 
+@pytest.mark.parametrize("M,N0,N1,K", [(16384, 1280, 1728, 768), (1024, 520, 300, 128), (600, 192, 64, 192),
+                                       (4096, 4096, 5632, 2048)])
+def test_two_products_of_one_launch_equal_the_separate_ones(M, N0, N1, K):
+    """mvpa_linear_bf16_dual against the two single launches, bit for bit (same kernels' tiles),
+    with the gated output a column slice of a wider buffer."""
+    g = torch.Generator().manual_seed(M + N0 + N1 + K)
+    x = torch.randn(M, K, generator=g).bfloat16().cuda()
+    w0 = (torch.randn(N0, K, generator=g) * 0.05).bfloat16().cuda()
+    w1 = (torch.randn(2 * N1, K, generator=g) * 0.05).bfloat16().cuda()
+    wide = torch.full((M, N1 + 72), 3.0, dtype=torch.bfloat16, device="cuda")
+    y0, y1 = mvpa_hip.linear_dual(x, w0, w1, out_gated=wide[:, 8:8 + N1])
+    assert torch.equal(y0, mvpa_hip.linear(x, w0))
+    assert torch.equal(y1, mvpa_hip.linear(x, w1, gated=True))
+    assert (wide[:, :8] == 3.0).all() and (wide[:, 8 + N1:] == 3.0).all()
+
+
+def test_two_products_of_one_launch_refuse_small_shapes():
+    x = torch.zeros(64, 768, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(768, 768, dtype=torch.bfloat16, device="cuda")
+    assert not mvpa_hip.linear_dual_supported(64, 768) and not mvpa_hip.linear_dual_supported(1024, 96)
+    with pytest.raises(mvpa_hip.MvpaError):
+        mvpa_hip.linear_dual(x, w, w)
+
+
 def test_linear_into_a_column_slice():
     """The gated product written into a column slice of a wider buffer (the block's tail operand)."""
     g = torch.Generator().manual_seed(9)
