@@ -165,6 +165,52 @@ def test_mvpformer_s_full_size_properties():
     assert not torch.equal(out2[:, -9:], out[:, -9:])
 
 
+@pytest.mark.parametrize("flash", [True, False], ids=["flash", "masked"])
+def test_block_with_fused_products_matches_the_separate_ones(flash, monkeypatch):
+    """A parallel block at 640 rows: the path that forms q/kv + gate/up in one launch and the block's
+    tail (c_proj + down + residual) as one product, against the same block with every product on
+    its own (the path of small inputs), with an attention mask (honoured by the masked class only)
+    and use_cache: hidden states to bf16 rounding of the different summation order, presents equal."""
+    import mvpa_hip
+    from models.mvpformer import MVPFormerBlock, MVPFormerConfig
+    torch.manual_seed(7)
+    cfg = MVPFormerConfig(n_positions=16, n_channels=64, n_embd=128, n_layer=1, n_head=4, n_head_kv=2, n_inner=320)
+    blk = MVPFormerBlock(cfg, layer_idx=0, flash=flash).to(device="cuda", dtype=torch.bfloat16).eval()
+    for p in blk.parameters():
+        p.data.normal_(0, 0.05)
+    blk.ln_1.weight.data.fill_(1.0)
+    B, T, C, E = 1, 16, 40, 128
+    x = torch.randn(B, T, C, E, device="cuda").bfloat16()
+    pos = (torch.randn(1, T, E, device="cuda") * 0.3).bfloat16()
+    chan = (torch.randn(1, C, E, device="cuda") * 0.3).bfloat16()
+    valid = torch.ones(B, T, C, device="cuda")
+    valid[:, :, 5] = 0
+    valid[:, :, 33:] = 0
+    mask = ((1.0 - valid.view(B, -1)) * torch.finfo(torch.bfloat16).min)[:, None, None, :].to(torch.bfloat16)
+
+    def run():
+        with torch.no_grad():
+            (h, present), normed = blk.forward_fused(x, None, blk.ln_2, pos, chan, attention_mask=mask, use_cache=True)
+        return h, present, normed
+
+    assert mvpa_hip.linear_residual_supported(B * T * C, E + 320) and mvpa_hip.linear_dual_supported(B * T * C, E)
+    h1, p1, n1 = run()
+    monkeypatch.setattr(mvpa_hip, "linear_residual_supported", lambda *a: False)
+    h0, p0, n0 = run()
+    assert torch.equal(p1[0], p0[0]) and torch.equal(p1[1], p0[1])
+    live = valid.bool()[..., None]
+    err = ((h1.float() - h0.float()) * live).abs().max().item()
+    assert err <= 2 ** -6 * h0.float().abs().max().item(), err
+    assert ((n1.float() - n0.float()) * live).abs().max().item() <= 5e-2
+    if not flash:           # the mask reaches the kernel: an absent channel's keys change nothing
+        x2 = x.clone()
+        x2[:, :, 33:] += 1.0
+        monkeypatch.undo()
+        with torch.no_grad():
+            (h2, _), _ = blk.forward_fused(x2, None, blk.ln_2, pos, chan, attention_mask=mask, use_cache=True)
+        assert torch.equal(h2[:, :, :5], h1[:, :, :5])
+
+
 def test_base_classification_bf16_then_fp8():
     """Base-size dims (E2048 H16 Hkv8 Dh128 n_inner5632, C=128) cut to two layers and 12 segments:
     binary-head logits in bf16 and with fp8 QK^T against the fp32 oracle stack.  Tolerances are
