@@ -716,7 +716,7 @@ __device__ inline void staged_epilogue(const f32x16 (&acc)[BN / 64][2], unsigned
               v[e] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
             }
           }
-          *(u32x4*)dst = v;
+          __builtin_nontemporal_store(v, (u32x4*)dst);   // (streamed out: the operand panels keep the L2)
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e)

@@ -685,15 +685,47 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
   wait_vmcnt_imm<0>();                   // (the far requests past the end)
 
   // =========================== epilogue ===========================
+  // In the accumulators a lane holds 4 consecutive output columns of its query (8 bytes) for each
+  // of 8 column groups: stored from there, an instruction writes 16 bytes to each of 32 rows.
+  // Staged through the wave's slab memory (idle by now), a tile leaves as whole 128-byte rows, 16
+  // bytes per lane, 8 lanes side by side on a row; the stores are streamed (non-temporal).
+  constexpr int OPITCH = DH * 2 + 16;                    // staged row pitch in bytes (+16: rows spread over the banks)
+  static_assert(32 * OPITCH <= STB_WAVE, "a staged tile fits the wave's slab memory");
+  unsigned char* ostage = (unsigned char*)stb_wave;
+  const bool ovec = (a.o_stride_n & 7) == 0 && (a.o_stride_b & 7) == 0 && (a.o_stride_h & 7) == 0 &&
+                    ((uintptr_t)a.o & 15) == 0;
 #pragma unroll
   for (int x = 0; x < 2; ++x) {
     if (x == 1 && last_wg) break;
-    const int cq = (x == 0 ? cb0 : cb1) + ln;
+    const int cq0 = x == 0 ? cb0 : cb1, cq = cq0 + ln;
     const float ltot = qt[x].l + __shfl_xor(qt[x].l, 32);
-    if (active && cq < C_) {
-      const float inv = 1.f / ltot;
-      const int64_t n = (int64_t)tq * C_ + cq;
-      bf16_t* orow = (bf16_t*)a.o + b * a.o_stride_b + h * a.o_stride_h + n * a.o_stride_n;
+    const float inv = 1.f / ltot;
+    bf16_t* obase = (bf16_t*)a.o + b * a.o_stride_b + h * a.o_stride_h;
+    if (a.lse && active && cq < C_ && hh == 0)
+      a.lse[((int64_t)b * a.H + h) * ((int64_t)T_ * C_) + (int64_t)tq * C_ + cq] = qt[x].m + log2f(ltot);
+    if (ovec) {
+      wave_lds_sync();                                 // (the slab memory's last readers / the tile before)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) {
+          bf16x4 w;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) w[r] = (__bf16)(qt[x].acc[mt][a4 * 4 + r] * inv);
+          *(bf16x4*)(ostage + ln * OPITCH + (mt * 32 + a4 * 8 + hh * 4) * 2) = w;
+        }
+      wave_lds_sync();
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int row = it * 8 + (lane >> 3), ch = lane & 7;
+        const u32x4 v = *(const u32x4*)(ostage + row * OPITCH + ch * 16);
+        if (active && cq0 + row < C_) {
+          const int64_t n = (int64_t)tq * C_ + cq0 + row;
+          __builtin_nontemporal_store(v, (u32x4*)(obase + n * a.o_stride_n + ch * 8));
+        }
+      }
+    } else if (active && cq < C_) {
+      bf16_t* orow = obase + ((int64_t)tq * C_ + cq) * a.o_stride_n;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -704,7 +736,6 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
           for (int r = 0; r < 4; ++r) w[r] = (__bf16)(qt[x].acc[mt][a4 * 4 + r] * inv);
           *(bf16x4*)(orow + d0) = w;
         }
-      if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * ((int64_t)T_ * C_) + n] = qt[x].m + log2f(ltot);
     }
   }
 }
