@@ -39,7 +39,7 @@ BF16_DENSE_PEAK_TFLOPS = 2500.0       # MI355X published dense bf16 MFMA peak
 # HBM bytes per launch of the attention kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by
 # what the same counters read for a plain device copy of known size; the profile summary named
 # beside each figure holds the two counter runs.
-MEASURED_TRAFFIC_BYTES = {"c2": (734.3e6, "profiles/mvpa_mfma64_kernel_c2.md"),
+MEASURED_TRAFFIC_BYTES = {"c2": (702.9e6, "profiles/mvpa_mfma64_kernel_c2.md"),
                           "c3": (4.68e9, "profiles/mvpa_mfma128_kernel_c3.md"),
                           "c5attn": (11.51e9, "profiles/mvpa_mfma128_kernel_c5attn.md")}
 PREWARM_LAUNCHES = 150
