@@ -13,6 +13,8 @@ pytestmark = pytest.mark.gpu
                                    (16384, 768, 1728),
                                    # tile rows a multiple of 32: the XCD-aware tile order, with ragged N and a K tail
                                    (8192, 1000, 200), (16384, 520, 72),
+                                   # K a multiple of 64: the 64-wide two-stage kernel, ragged rows and columns, two k-blocks only
+                                   (600, 130, 128), (1000, 200, 192), (5000, 333, 256), (513, 257, 1024),
                                    # at most 128 rows: the K-split kernel of a decoding step
                                    (64, 1280, 768), (64, 768, 1728), (33, 130, 550), (1, 768, 768), (20, 100, 72),
                                    (32, 2048, 5632), (128, 2048, 2048), (100, 3072, 2048), (65, 96, 24)])
@@ -33,7 +35,8 @@ def test_linear_bf16(M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(200, 96, 64), (1024, 1728, 768), (700, 200, 136), (4096, 64, 768),
                                    (64, 1728, 768), (20, 70, 136), (40, 33, 552), (7, 5632, 2048), (128, 5632, 2048), (97, 40, 72),
-                                   (8192, 300, 136)])      # the XCD-aware tile order
+                                   (8192, 300, 136),       # the XCD-aware tile order
+                                   (700, 200, 128), (2100, 70, 320)])   # the 64-wide two-stage kernel, ragged
 def test_linear_gated(M, N, K):
     g = torch.Generator().manual_seed(3)
     x = torch.randn(M, K, generator=g).bfloat16()
