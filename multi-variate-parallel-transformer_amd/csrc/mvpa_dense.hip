@@ -448,200 +448,6 @@ __device__ inline void tile_of_workgroup(int64_t L, int64_t mt, int64_t nt, int6
   *tn = __builtin_amdgcn_readfirstlane((int)n);
 }
 
-template <int BN, int EPI>
-__global__ __launch_bounds__(512) void linear_bf16_big_kernel(const bf16_t* __restrict__ X,
-                                                              const bf16_t* __restrict__ W,
-                                                              bf16_t* __restrict__ Y, int64_t M,
-                                                              int64_t N, int64_t K, int64_t ldx,
-                                                              int64_t ldw, int64_t ldy) {
-  constexpr int BM = 256, BK = 64, ROWB = BK * 2;
-  constexpr int WN = BN / 2, NB = WN / 32;            // per-wave extent over w rows
-  constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
-  constexpr int A_LOADS = A_BYTES / 1024 / 8, B_LOADS = B_BYTES / 1024 / 8;   // per wave
-  static_assert(EPI != 1 || NB % 2 == 0, "gate/up pairs need an even number of sub-blocks");
-  extern __shared__ __attribute__((aligned(1024))) unsigned char gsm[];
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int ln = lane & 31, hh = lane >> 5;
-  const int wm = wave >> 1, wc = wave & 1;
-  constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;    // output columns per workgroup
-  const int64_t mt = (M + BM - 1) / BM, nt = (N + OUT_COLS - 1) / OUT_COLS;
-
-  int64_t m0 = 0, n0 = 0;                             // first x row / output column of the tile
-  const bf16_t* asrc[A_LOADS];
-  const bf16_t* bsrc[B_LOADS];
-  auto w_row = [&](int r) -> int64_t {                // which w row feeds tile row r
-    if (EPI == 1) {
-      const int wcol = r / WN, nb = (r % WN) / 32, i = r & 31;
-      const int64_t col = n0 + wcol * (WN / 2) + (nb >> 1) * 32 + i;
-      return ((nb & 1) ? N : 0) + (col < N ? col : N - 1);
-    }
-    const int64_t n = n0 + r;
-    return n < N ? n : N - 1;
-  };
-  // per-lane source rows of this wave's loads (row clamped into range: such rows are never stored)
-  auto set_tile = [&](int64_t L) {
-    int64_t tile_m, tile_n;
-    tile_of_workgroup(L, mt, nt, &tile_m, &tile_n);
-    m0 = tile_m * BM;
-    n0 = tile_n * OUT_COLS;
-    const int rsub = lane >> 3, phys = lane & 7;
-#pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-      const int row = (wave * A_LOADS + i) * 8 + rsub;
-      const int64_t m = m0 + row;
-      asrc[i] = X + (m < M ? m : M - 1) * ldx + ((phys ^ ((row >> 1) & 7)) << 3);
-    }
-#pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) {
-      const int row = (wave * B_LOADS + i) * 8 + rsub;
-      bsrc[i] = W + w_row(row) * ldw + ((phys ^ ((row >> 1) & 7)) << 3);
-    }
-  };
-  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)gsm;
-  auto issue = [&](int kt, int stage) {
-    const int64_t k0 = (int64_t)kt * BK;
-    const uint32_t base = lds0 + stage * STAGE;
-    if (k0 + BK <= K) {                               // (uniform) a whole k-block: nothing but the loads
-#pragma unroll
-      for (int i = 0; i < A_LOADS; ++i) dma_to_lds_16(asrc[i] + k0, base + (wave * A_LOADS + i) * 1024);
-#pragma unroll
-      for (int i = 0; i < B_LOADS; ++i) dma_to_lds_16(bsrc[i] + k0, base + A_BYTES + (wave * B_LOADS + i) * 1024);
-      return;
-    }
-    // the tail block of K: chunks past the end are zero-filled
-#pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-      const uint32_t dst = base + (wave * A_LOADS + i) * 1024;
-      const int row = (wave * A_LOADS + i) * 8 + (lane >> 3);
-      const int64_t kk = k0 + (((lane & 7) ^ ((row >> 1) & 7)) << 3);
-      if (kk < K) dma_to_lds_16(asrc[i] + k0, dst);
-      else *(u32x4*)(gsm + (dst - lds0) + lane * 16) = u32x4{0u, 0u, 0u, 0u};
-    }
-#pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) {
-      const uint32_t dst = base + A_BYTES + (wave * B_LOADS + i) * 1024;
-      const int row = (wave * B_LOADS + i) * 8 + (lane >> 3);
-      const int64_t kk = k0 + (((lane & 7) ^ ((row >> 1) & 7)) << 3);
-      if (kk < K) dma_to_lds_16(bsrc[i] + k0, dst);
-      else *(u32x4*)(gsm + (dst - lds0) + lane * 16) = u32x4{0u, 0u, 0u, 0u};
-    }
-  };
-
-  // loop-invariant fragment offsets: row ln of a 32-row block, chunk (2ks+hh) ^ swizzle(ln)
-  int frag_off[4];
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) frag_off[ks] = ln * ROWB + (((2 * ks + hh) ^ ((ln >> 1) & 7)) << 4);
-
-  const int nkt = (int)((K + BK - 1) / BK);
-  typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-  int stage = 0;                                      // ring stage of the k-block to multiply next
-  set_tile(blockIdx.x);
-  issue(0, 0);
-  {
-    const int64_t cm0 = m0, cn0 = n0;
-    f32x16 acc[NB][2];
-#pragma unroll
-    for (int i = 0; i < NB; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-    for (int kt = 0; kt < nkt; ++kt) {
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      const unsigned char* sa = gsm + stage * STAGE + (wm * 64) * ROWB;
-      const unsigned char* sb = gsm + stage * STAGE + A_BYTES + (wc * WN) * ROWB;
-      // the first fragments are requested before the next block's loads, whose issue covers their
-      // latency; inside the block the fragments of k-step s+1 are requested before the products of s
-      bf16x8 xf[2][2], wf[2][NB];
-#pragma unroll
-      for (int j = 0; j < 2; ++j) xf[0][j] = *(const bf16x8*)(sa + j * 32 * ROWB + frag_off[0]);
-#pragma unroll
-      for (int i = 0; i < NB; ++i) wf[0][i] = *(const bf16x8*)(sb + i * 32 * ROWB + frag_off[0]);
-      __builtin_amdgcn_sched_barrier(0);
-      if (kt + 1 < nkt) issue(kt + 1, stage ^ 1);
-      stage ^= 1;
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const int cur = ks & 1, nxt = cur ^ 1;
-        if (ks + 1 < 4) {
-#pragma unroll
-          for (int j = 0; j < 2; ++j) xf[nxt][j] = *(const bf16x8*)(sa + j * 32 * ROWB + frag_off[ks + 1]);
-#pragma unroll
-          for (int i = 0; i < NB; ++i) wf[nxt][i] = *(const bf16x8*)(sb + i * 32 * ROWB + frag_off[ks + 1]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < NB; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[cur][i], xf[cur][j], acc[i][j], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-
-    // epilogue: lane = x row (ln) of block j; accumulator quad a4 = w rows 8*a4 + 4*hh + 0..3
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int64_t m = cm0 + wm * 64 + j * 32 + ln;
-      if (m >= M) continue;
-      bf16_t* yrow = Y + m * ldy;
-      if (EPI == 1) {
-#pragma unroll
-        for (int p = 0; p < NB / 2; ++p)
-#pragma unroll
-          for (int a4 = 0; a4 < 4; ++a4) {
-            const int64_t n = cn0 + wc * (WN / 2) + p * 32 + a4 * 8 + hh * 4;
-            bf16x4 o;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const float gte = acc[2 * p][j][a4 * 4 + r], up = acc[2 * p + 1][j][a4 * 4 + r];
-              o[r] = (__bf16)(gte / (1.f + __expf(-gte)) * up);
-            }
-            if (n + 3 < N) {
-              *(bf16x4*)(yrow + n) = o;
-            } else {
-#pragma unroll
-              for (int r = 0; r < 4; ++r)
-                if (n + r < N) ((__bf16*)yrow)[n + r] = o[r];
-            }
-          }
-      } else {
-#pragma unroll
-        for (int i = 0; i < NB; ++i)
-#pragma unroll
-          for (int a4 = 0; a4 < 4; ++a4) {
-            const int64_t n = cn0 + wc * WN + i * 32 + a4 * 8 + hh * 4;
-            bf16x4 o;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][a4 * 4 + r];
-            if (n + 3 < N) {
-              *(bf16x4*)(yrow + n) = o;
-            } else {
-#pragma unroll
-              for (int r = 0; r < 4; ++r)
-                if (n + r < N) ((__bf16*)yrow)[n + r] = o[r];
-            }
-          }
-      }
-    }
-  }
-}
-
-template <int BN, int EPI>
-static int launch_big(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, int64_t N, int64_t K,
-                      int64_t ldx, int64_t ldw, int64_t ldy, hipStream_t s) {
-  constexpr int LDS = 2 * (256 + BN) * 128;
-  auto kern = linear_bf16_big_kernel<BN, EPI>;
-  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
-  constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;
-  dim3 grid((unsigned)(((N + OUT_COLS - 1) / OUT_COLS) * ((M + 255) / 256)));
-  MVPA_LAUNCH(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
-}
-
 // ---- epilogue of the large-tile kernels, through LDS (LDS_BYTES of it, idle by now).
 // In the accumulators a lane holds 4 consecutive output columns of one x row (quad a4 = w rows
 // 8*a4 + 4*hh + 0..3 of sub-block i, x row ln of block j): stored from there, an instruction writes
@@ -732,6 +538,155 @@ __device__ inline void staged_epilogue(const f32x16 (&acc)[BN / 64][2], unsigned
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
+}
+
+template <int BN, int EPI>
+__global__ __launch_bounds__(512) void linear_bf16_big_kernel(const bf16_t* __restrict__ X,
+                                                              const bf16_t* __restrict__ W,
+                                                              bf16_t* __restrict__ Y, int64_t M,
+                                                              int64_t N, int64_t K, int64_t ldx,
+                                                              int64_t ldw, int64_t ldy) {
+  constexpr int BM = 256, BK = 64, ROWB = BK * 2;
+  constexpr int WN = BN / 2, NB = WN / 32;            // per-wave extent over w rows
+  constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_LOADS = A_BYTES / 1024 / 8, B_LOADS = B_BYTES / 1024 / 8;   // per wave
+  static_assert(EPI != 1 || NB % 2 == 0, "gate/up pairs need an even number of sub-blocks");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char gsm[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 31, hh = lane >> 5;
+  const int wm = wave >> 1, wc = wave & 1;
+  constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;    // output columns per workgroup
+  const int64_t mt = (M + BM - 1) / BM, nt = (N + OUT_COLS - 1) / OUT_COLS;
+
+  int64_t m0 = 0, n0 = 0;                             // first x row / output column of the tile
+  const bf16_t* asrc[A_LOADS];
+  const bf16_t* bsrc[B_LOADS];
+  auto w_row = [&](int r) -> int64_t {                // which w row feeds tile row r
+    if (EPI == 1) {
+      const int wcol = r / WN, nb = (r % WN) / 32, i = r & 31;
+      const int64_t col = n0 + wcol * (WN / 2) + (nb >> 1) * 32 + i;
+      return ((nb & 1) ? N : 0) + (col < N ? col : N - 1);
+    }
+    const int64_t n = n0 + r;
+    return n < N ? n : N - 1;
+  };
+  // per-lane source rows of this wave's loads (row clamped into range: such rows are never stored)
+  auto set_tile = [&](int64_t L) {
+    int64_t tile_m, tile_n;
+    tile_of_workgroup(L, mt, nt, &tile_m, &tile_n);
+    m0 = tile_m * BM;
+    n0 = tile_n * OUT_COLS;
+    const int rsub = lane >> 3, phys = lane & 7;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int row = (wave * A_LOADS + i) * 8 + rsub;
+      const int64_t m = m0 + row;
+      asrc[i] = X + (m < M ? m : M - 1) * ldx + ((phys ^ ((row >> 1) & 7)) << 3);
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+      const int row = (wave * B_LOADS + i) * 8 + rsub;
+      bsrc[i] = W + w_row(row) * ldw + ((phys ^ ((row >> 1) & 7)) << 3);
+    }
+  };
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)gsm;
+  auto issue = [&](int kt, int stage) {
+    const int64_t k0 = (int64_t)kt * BK;
+    const uint32_t base = lds0 + stage * STAGE;
+    if (k0 + BK <= K) {                               // (uniform) a whole k-block: nothing but the loads
+#pragma unroll
+      for (int i = 0; i < A_LOADS; ++i) dma_to_lds_16(asrc[i] + k0, base + (wave * A_LOADS + i) * 1024);
+#pragma unroll
+      for (int i = 0; i < B_LOADS; ++i) dma_to_lds_16(bsrc[i] + k0, base + A_BYTES + (wave * B_LOADS + i) * 1024);
+      return;
+    }
+    // the tail block of K: chunks past the end are zero-filled
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const uint32_t dst = base + (wave * A_LOADS + i) * 1024;
+      const int row = (wave * A_LOADS + i) * 8 + (lane >> 3);
+      const int64_t kk = k0 + (((lane & 7) ^ ((row >> 1) & 7)) << 3);
+      if (kk < K) dma_to_lds_16(asrc[i] + k0, dst);
+      else *(u32x4*)(gsm + (dst - lds0) + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+      const uint32_t dst = base + A_BYTES + (wave * B_LOADS + i) * 1024;
+      const int row = (wave * B_LOADS + i) * 8 + (lane >> 3);
+      const int64_t kk = k0 + (((lane & 7) ^ ((row >> 1) & 7)) << 3);
+      if (kk < K) dma_to_lds_16(bsrc[i] + k0, dst);
+      else *(u32x4*)(gsm + (dst - lds0) + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+    }
+  };
+
+  // loop-invariant fragment offsets: row ln of a 32-row block, chunk (2ks+hh) ^ swizzle(ln)
+  int frag_off[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) frag_off[ks] = ln * ROWB + (((2 * ks + hh) ^ ((ln >> 1) & 7)) << 4);
+
+  const int nkt = (int)((K + BK - 1) / BK);
+  int stage = 0;                                      // ring stage of the k-block to multiply next
+  set_tile(blockIdx.x);
+  issue(0, 0);
+  {
+    const int64_t cm0 = m0, cn0 = n0;
+    f32x16 acc[NB][2];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    for (int kt = 0; kt < nkt; ++kt) {
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      const unsigned char* sa = gsm + stage * STAGE + (wm * 64) * ROWB;
+      const unsigned char* sb = gsm + stage * STAGE + A_BYTES + (wc * WN) * ROWB;
+      // the first fragments are requested before the next block's loads, whose issue covers their
+      // latency; inside the block the fragments of k-step s+1 are requested before the products of s
+      bf16x8 xf[2][2], wf[2][NB];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) xf[0][j] = *(const bf16x8*)(sa + j * 32 * ROWB + frag_off[0]);
+#pragma unroll
+      for (int i = 0; i < NB; ++i) wf[0][i] = *(const bf16x8*)(sb + i * 32 * ROWB + frag_off[0]);
+      __builtin_amdgcn_sched_barrier(0);
+      if (kt + 1 < nkt) issue(kt + 1, stage ^ 1);
+      stage ^= 1;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int cur = ks & 1, nxt = cur ^ 1;
+        if (ks + 1 < 4) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) xf[nxt][j] = *(const bf16x8*)(sa + j * 32 * ROWB + frag_off[ks + 1]);
+#pragma unroll
+          for (int i = 0; i < NB; ++i) wf[nxt][i] = *(const bf16x8*)(sb + i * 32 * ROWB + frag_off[ks + 1]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[cur][i], xf[cur][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+
+    staged_epilogue<BN, EPI, 2 * STAGE>(acc, gsm, wave, lane, cm0, cn0, M, N, Y, ldy, nullptr, 0);
+  }
+}
+
+template <int BN, int EPI>
+static int launch_big(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, int64_t N, int64_t K,
+                      int64_t ldx, int64_t ldw, int64_t ldy, hipStream_t s) {
+  constexpr int LDS = 2 * (256 + BN) * 128;
+  auto kern = linear_bf16_big_kernel<BN, EPI>;
+  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+  constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;
+  dim3 grid((unsigned)(((N + OUT_COLS - 1) / OUT_COLS) * ((M + 255) / 256)));
+  MVPA_LAUNCH(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy);
+  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
 }
 
 // -----------------------------------------------------------------------------------------
