@@ -23,8 +23,21 @@ Pinning status (what independent evidence fixes each function):
                                float64 brute force (windowed, GQA, masks); invariants
                                (row-stochastic, causality, window locality, GQA == MHA).
   mvpa_direct                : equality with rel_attn on every small configuration.
-  attention_layer_forward    : composition of torch.nn.functional.linear and rel_attn;
-                               pinned through rel_attn.
+  split_heads / merge_heads  : explicit index check, feature h*Dh+d of token (b,t,c) lands at
+                               [b,h,t,c,d]; merge is the inverse (tests/test_oracle_stack.py).
+  attention_layer_forward    : an einsum statement that never calls split/merge heads (named
+                               head/dim axes, K = first half of c_attn, V = second) around the
+                               float64 brute force; with and without the additive key mask; a
+                               swapped K/V split is shown to fail (tests/test_oracle_stack.py).
+  rmsnorm                    : torch.nn.functional.rms_norm and torch.nn.RMSNorm, fp32 and bf16,
+                               plus a tiny-norm row that fixes eps inside the root.
+  wave_encoder_forward       : torch.nn.RMSNorm + torch.nn.Linear around the pad + conv1d
+                               statement of the wavelet transform.
+  mvpformer_forward          : a composition of library modules (torch.nn.RMSNorm, Linear,
+                               Embedding, transformers' LlamaMLP with mlp_bias=False) wired as
+                               models/mvpformer.py:104-147, 246-283, 380 state it (parallel
+                               block, both branches read ln_1(x), ln_2 unused, ln_f last), with
+                               and without a token mask; a sequential block is shown to differ.
   wavedec_db4_periodic       : the reference delegates to ptwt.wavedec (ptwt==0.1.9 with
                                PyWavelets' db4 filters, models/fftencoder.py:62, 70-88), not
                                installed here.  Its published algorithm - circular pad of
