@@ -266,15 +266,15 @@ def main():
                             "outputs": "dq (content share), dk, dv, dbias_time, dbias_chan (fp32)"}
     if not args.no_model:
         try:
-            from models.bench_model import mvpformer_s_windows_per_s
+            from bench_model import mvpformer_s_windows_per_s
             line["mvpformer_s"] = mvpformer_s_windows_per_s()
             if not args.no_stream:
-                from models.bench_model import mvpformer_s_stream_step_ms
+                from bench_model import mvpformer_s_stream_step_ms
                 line["mvpformer_s_stream"] = mvpformer_s_stream_step_ms()
         except ImportError:
             line["mvpformer_s"] = None
     if args.base_model:
-        from models.bench_model import mvpformer_base_forward_ms
+        from bench_model import mvpformer_base_forward_ms
         line["mvpformer_base"] = mvpformer_base_forward_ms(stream=not args.no_stream)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(cfg)

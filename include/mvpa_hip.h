@@ -181,6 +181,12 @@ int mvpa_forward(const mvpa_fwd_args* args, void* stream);
 #define MVPA_STATIC_WS_BYTES (16u << 20)
 int mvpa_forward_last_step_static(const mvpa_fwd_args* args, void* stream);
 size_t mvpa_static_ws_bytes(void);
+/* Set-up for the entry point above, once per GPU with that GPU current and outside any stream
+ * capture: resolves and keeps the array's address on that GPU, so that the first
+ * mvpa_forward_last_step_static call may itself be recorded into a graph.  (A first call that
+ * finds the address unresolved resolves it itself, which is a runtime query mid-capture.)
+ * Returns MVPA_OK or MVPA_ERR_LAUNCH.  No counterpart in the reference. */
+int mvpa_static_ws_init(void);
 
 /* ---- backward ------------------------------------------------------------------------------
  * Argument block of mvpa_backward: the boundary of FlashMVPA.backward
@@ -275,8 +281,8 @@ int mvpa_linear_bf16_residual(const void* x, const void* w, const void* r, void*
  * with w1 holding the gate rows [0,N1) and the up rows [N1,2*N1) - the fused q/kv projection
  * (layers/mvpa.py:354-356) and the MLP's gate/up product (models/mvpformer.py:146), which both read
  * ln_1(x) in the parallel block.  Launched separately each product ends on a partly filled round
- * of tiles; in one grid only their sum does.  Large shapes only: M >= 512, K a multiple of 64;
- * MVPA_ERR_UNSUPPORTED otherwise. */
+ * of tiles; in one grid only their sum does.  Large shapes only: M >= 512, K a multiple of 64 and
+ * at least 128 (two k-blocks: the kernel's two-stage pipeline); MVPA_ERR_UNSUPPORTED otherwise. */
 int mvpa_linear_bf16_dual(const void* x, const void* w0, void* y0, const void* w1, void* y1, int64_t M,
                           int64_t N0, int64_t N1, int64_t K, int64_t ldx, int64_t ldw0, int64_t ldy0,
                           int64_t ldw1, int64_t ldy1, void* stream);

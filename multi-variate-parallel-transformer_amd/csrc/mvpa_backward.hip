@@ -285,14 +285,14 @@ static int launch_bwd_t(const mvpa_bwd_args* a, hipStream_t stream, bool query_p
   if (lds_q > 160 * 1024) return MVPA_ERR_UNSUPPORTED;
   auto kq = mvpa_bwd_query_kernel<T, DH>;
   auto kk = mvpa_bwd_key_kernel<T, DH>;
-  (void)hipFuncSetAttribute((const void*)kq, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_q);
+  mvpa::want_dynamic_lds((const void*)kq, (int)lds_q);
   const unsigned nb = (unsigned)((N + BWD_THREADS - 1) / BWD_THREADS);
   if (query_pass) {
     MVPA_LAUNCH(kq, dim3(nb, a->B * a->H), dim3(BWD_THREADS), lds_q, stream, *a);
-    if (hipGetLastError() != hipSuccess) return MVPA_ERR_LAUNCH;
+    if (mvpa::take_launch_status() != MVPA_OK) return MVPA_ERR_LAUNCH;
   }
   MVPA_LAUNCH(kk, dim3(nb, a->B * a->Hkv), dim3(BWD_THREADS), lds_k, stream, *a);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 template <typename T>

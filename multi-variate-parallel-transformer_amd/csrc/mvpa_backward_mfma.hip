@@ -674,7 +674,7 @@ static void launch_query(const mvpa_bwd_args* a, hipStream_t stream, int q0, int
   const size_t lds = (size_t)QSTAGES * 3 * cp * ROWB + (size_t)nw * WAVE_SCRATCH * sizeof(float);
   dim3 grid((unsigned)(nt * a->B * a->H));
   auto kern = mvpa_bwd_query_mfma_kernel<NCT>;
-  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  mvpa::want_dynamic_lds((const void*)kern, (int)lds);
   MVPA_LAUNCH(kern, grid, dim3(nw * 64), lds, stream, *a, q0, k0, accum);
 }
 
@@ -1013,7 +1013,7 @@ static void launch_key(const mvpa_bwd_args* a, hipStream_t stream, int k0, int q
   const size_t lds = (size_t)KSTAGES * (4 * cp * ROWB + cp * cp * 4 + (kt + 1) * 256);
   dim3 grid((unsigned)(((a->T + kt - 1) / kt) * a->B * a->Hkv));
   auto kern = mvpa_bwd_key_mfma_kernel<NCT, MASKED>;
-  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  mvpa::want_dynamic_lds((const void*)kern, (int)lds);
   MVPA_LAUNCH(kern, grid, dim3(nw * 64), lds, stream, *a, k0, q0, accum);
 }
 
@@ -1039,5 +1039,5 @@ int mvpa_launch_bwd_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
         else launch_key<2, true>(a, stream, k0, q0, qp > 0);
       }
   }
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }

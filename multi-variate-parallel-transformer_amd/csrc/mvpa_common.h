@@ -4,6 +4,11 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+#include <tuple>
+#include <unordered_map>
+#include <utility>
+
 #include "mvpa_hip.h"
 
 namespace mvpa {
@@ -74,13 +79,61 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 }  // namespace mvpa
 
-// A launch whose status is this call's own: HIP keeps the last error until it is read, so an
-// error left by unrelated earlier work would otherwise be reported as a failure of this launch.
-#define MVPA_LAUNCH(...)            \
-  do {                              \
-    (void)hipGetLastError();        \
-    hipLaunchKernelGGL(__VA_ARGS__); \
-  } while (0)
+// ---- launches ------------------------------------------------------------------------------
+// A launch reports its OWN status: hipLaunchKernel's return value.  The runtime's global
+// last-error slot is neither read nor cleared, so an error that unrelated earlier work of the
+// host application left pending stays where that application will look for it.
+namespace mvpa {
+
+template <typename... KArgs, size_t... I>
+inline hipError_t launch_impl(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t s,
+                              std::tuple<KArgs...>& vals, std::index_sequence<I...>) {
+  void* ptrs[] = {(void*)&std::get<I>(vals)..., nullptr};
+  return hipLaunchKernel((const void*)kern, grid, block, ptrs, lds, s);
+}
+
+template <typename... KArgs, typename... Args>
+inline hipError_t launch(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t s,
+                         Args&&... args) {
+  static_assert(sizeof...(KArgs) == sizeof...(Args), "kernel argument count");
+  std::tuple<KArgs...> vals{static_cast<KArgs>(args)...};    // converted to the parameter types
+  return launch_impl(kern, grid, block, lds, s, vals, std::index_sequence_for<KArgs...>{});
+}
+
+// Status of the launches this thread made since the last take_launch_status().
+inline int& pending_launch_status() {
+  static thread_local int st = MVPA_OK;
+  return st;
+}
+inline void note_launch(hipError_t e) {
+  if (e != hipSuccess) pending_launch_status() = MVPA_ERR_LAUNCH;
+}
+inline int take_launch_status() {
+  const int st = pending_launch_status();
+  pending_launch_status() = MVPA_OK;
+  return st;
+}
+
+// hipFuncAttributeMaxDynamicSharedMemorySize, set once per (kernel, device) instead of on every
+// launch: the call costs about as much as the launch itself on the decoding path.
+inline void want_dynamic_lds(const void* kern, int bytes) {
+  static std::mutex mu;
+  static std::unordered_map<uint64_t, int> seen;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  const uint64_t key = (uint64_t)(uintptr_t)kern * 64u + (uint64_t)(dev & 63);
+  {
+    std::lock_guard<std::mutex> g(mu);
+    auto it = seen.find(key);
+    if (it != seen.end() && it->second >= bytes) return;
+    seen[key] = bytes;
+  }
+  (void)hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+}  // namespace mvpa
+
+#define MVPA_LAUNCH(...) mvpa::note_launch(mvpa::launch(__VA_ARGS__))
 
 // ---- launchers implemented by the kernel translation units ----------------------------------
 int mvpa_launch_generic(const mvpa_fwd_args* a, hipStream_t stream);

@@ -682,11 +682,11 @@ static int launch_big(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, in
                       int64_t ldx, int64_t ldw, int64_t ldy, hipStream_t s) {
   constexpr int LDS = 2 * (256 + BN) * 128;
   auto kern = linear_bf16_big_kernel<BN, EPI>;
-  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+  mvpa::want_dynamic_lds((const void*)kern, (int)LDS);
   constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;
   dim3 grid((unsigned)(((N + OUT_COLS - 1) / OUT_COLS) * ((M + 255) / 256)));
   MVPA_LAUNCH(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 // -----------------------------------------------------------------------------------------
@@ -870,11 +870,11 @@ static int launch_ring(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, i
                        const bf16_t* r = nullptr, int64_t ldr = 0) {
   constexpr int LDS = 4 * (256 + BN) * 64;
   auto kern = linear_bf16_ring_kernel<BN, EPI>;
-  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+  mvpa::want_dynamic_lds((const void*)kern, (int)LDS);
   constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;
   dim3 grid((unsigned)(((N + OUT_COLS - 1) / OUT_COLS) * ((M + 255) / 256)));
   MVPA_LAUNCH(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy, r, ldr);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 // -----------------------------------------------------------------------------------------
@@ -1089,11 +1089,11 @@ static int launch_pair(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, i
                        const bf16_t* r = nullptr, int64_t ldr = 0) {
   constexpr int LDS = 2 * (256 + BN) * 128;
   auto kern = linear_bf16_pair_kernel<BN, EPI>;
-  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+  mvpa::want_dynamic_lds((const void*)kern, (int)LDS);
   constexpr int OUT_COLS = EPI == 1 ? BN / 2 : BN;
   dim3 grid((unsigned)(((N + OUT_COLS - 1) / OUT_COLS) * ((M + 255) / 256)));
   MVPA_LAUNCH(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy, r, ldr);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 template <int BN0>
@@ -1101,12 +1101,12 @@ static int launch_pair_dual(const bf16_t* x, int64_t M, int64_t K, int64_t ldx, 
                             const mvpa::linear_pair_problem& gated, hipStream_t s) {
   constexpr int LDS = 2 * (256 + 256) * 128;
   auto kern = linear_bf16_pair_dual_kernel<BN0>;
-  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+  mvpa::want_dynamic_lds((const void*)kern, (int)LDS);
   const int64_t mt = (M + 255) / 256;
   const int64_t gated_tiles = mt * ((gated.N + 127) / 128), plain_tiles = mt * ((plain.N + BN0 - 1) / BN0);
   MVPA_LAUNCH(kern, dim3((unsigned)(gated_tiles + plain_tiles)), dim3(512), LDS, s, x, M, K, ldx, plain, gated,
               gated_tiles);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 // -----------------------------------------------------------------------------------------
@@ -1407,9 +1407,9 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M,
   constexpr int lds = SK_WAVES * XT * 16 * 64 * (int)sizeof(float);
   auto kern = linear_bf16_skinny_kernel<EPI, XT>;
   if (lds > 64 * 1024)
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    mvpa::want_dynamic_lds((const void*)kern, (int)lds);
   MVPA_LAUNCH(kern, dim3((unsigned)((N + 31) / 32)), dim3(SK_WAVES * 64), lds, s, x, w, y, M, N, K, ldx, ldw, ldy);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 // K slices per workgroup and the number of workgroup rows that follows: as few partial tiles as
@@ -1444,7 +1444,7 @@ extern "C" int mvpa_linear_bf16_splitk(const void* x, const void* w, void* y, in
   const int64_t nw = epilogue == 1 ? 2 * N : N;
   int per_group, slices;          // slices: partial tiles per output tile = workgroup rows
   splitk_groups(nw, K, &per_group, &slices);
-  (void)hipFuncSetAttribute((const void*)linear_splitk_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SPK_LDS_BYTES);
+  mvpa::want_dynamic_lds((const void*)linear_splitk_kernel, (int)SPK_LDS_BYTES);
   MVPA_LAUNCH(linear_splitk_kernel, dim3((unsigned)((nw + SPK_COLS - 1) / SPK_COLS), (unsigned)slices), dim3(256),
                      SPK_LDS_BYTES, s, (const bf16_t*)x, (const bf16_t*)w, (float*)ws, M, nw, K, ldx, ldw, per_group);
   const int64_t items = M * ((N + 3) / 4);
@@ -1454,7 +1454,7 @@ extern "C" int mvpa_linear_bf16_splitk(const void* x, const void* w, void* y, in
   else
     MVPA_LAUNCH(linear_splitk_reduce_kernel<0>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
                        (const float*)ws, (bf16_t*)y, M, N, nw, slices, ldy);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 extern "C" int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M, int64_t N,
@@ -1517,7 +1517,7 @@ extern "C" int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M
     dim3 grid((unsigned)((N + GBN - 1) / GBN), (unsigned)((M + GBM - 1) / GBM));
     MVPA_LAUNCH(linear_bf16_kernel<0>, grid, dim3(256), 0, s, xp, wp, yp, M, N, K, ldx, ldw, ldy);
   }
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 // y0 = x w0^T and y1 = silu(x wg^T) * (x wu^T) in one launch (w1 holds the gate rows [0, N1) and
@@ -1596,7 +1596,7 @@ extern "C" int mvpa_rmsnorm(const void* x, const float* weight, void* y, int64_t
       MVPA_LAUNCH((rmsnorm_rows_kernel<bf16_t, bf16_t>), vgrid, block, 0, s, (const bf16_t*)x, weight, (bf16_t*)y, rows, cols, ldx, ldy, eps);
     else
       MVPA_LAUNCH((rmsnorm_rows_kernel<bf16_t, float>), vgrid, block, 0, s, (const bf16_t*)x, weight, (float*)y, rows, cols, ldx, ldy, eps);
-    return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+    return mvpa::take_launch_status();
   }
   if (in_dtype == MVPA_F32 && out_dtype == MVPA_F32)
     MVPA_LAUNCH((rmsnorm_kernel<float, float>), grid, block, 0, s, (const float*)x, weight, (float*)y, cols, ldx, ldy, eps);
@@ -1608,7 +1608,7 @@ extern "C" int mvpa_rmsnorm(const void* x, const float* weight, void* y, int64_t
     MVPA_LAUNCH((rmsnorm_kernel<bf16_t, float>), grid, block, 0, s, (const bf16_t*)x, weight, (float*)y, cols, ldx, ldy, eps);
   else
     return MVPA_ERR_DTYPE;
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 extern "C" int mvpa_cosine_rows_bf16(const void* a, const void* b, float* out, int64_t groups,
@@ -1624,7 +1624,7 @@ extern "C" int mvpa_cosine_rows_bf16(const void* a, const void* b, float* out, i
   MVPA_LAUNCH(cosine_rows_bf16_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
               (const bf16_t*)a, (const bf16_t*)b, out, rows, rows_per_group, cols, lda, ldb,
               group_stride_a, group_stride_b, eps);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 extern "C" int mvpa_add3_bf16(const void* a, const void* b, const void* c, void* out, int64_t n,
@@ -1636,12 +1636,12 @@ extern "C" int mvpa_add3_bf16(const void* a, const void* b, const void* c, void*
     MVPA_LAUNCH(add3_bf16_vec_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)c,
                        (bf16_t*)out, n8);
-    return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+    return mvpa::take_launch_status();
   }
   MVPA_LAUNCH(add3_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)c,
                      (bf16_t*)out, n);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 extern "C" int mvpa_ring_append_bf16(const void* k_new, const void* v_new, void* k_ring, void* v_ring,
@@ -1657,7 +1657,7 @@ extern "C" int mvpa_ring_append_bf16(const void* k_new, const void* v_new, void*
   MVPA_LAUNCH(ring_append_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)k_new, (const bf16_t*)v_new, (bf16_t*)k_ring,
                      (bf16_t*)v_ring, head, Hkv, C, Dh, steps, stride_b, stride_h, stride_c, total);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 extern "C" int mvpa_add3_rmsnorm_bf16(const void* a, const void* b, const void* c,
@@ -1673,7 +1673,7 @@ extern "C" int mvpa_add3_rmsnorm_bf16(const void* a, const void* b, const void* 
   MVPA_LAUNCH(kern, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)c,
                      weight, (bf16_t*)sum, (bf16_t*)norm, rows, cols, eps);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 extern "C" int mvpa_wavedec_db4(const float* x, float* coeffs, int64_t M, int32_t L,
@@ -1686,9 +1686,8 @@ extern "C" int mvpa_wavedec_db4(const float* x, float* coeffs, int64_t M, int32_
   if (total != dwt_size) return MVPA_ERR_SHAPE;
   // two ping-pong rows of L floats: past 64 KiB of dynamic LDS the kernel has to be told
   if (2 * L * sizeof(float) > 64 * 1024)
-    (void)hipFuncSetAttribute((const void*)wavedec_db4_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)(2 * L * sizeof(float)));
+    mvpa::want_dynamic_lds((const void*)wavedec_db4_kernel, (int)(2 * L * sizeof(float)));
   MVPA_LAUNCH(wavedec_db4_kernel, dim3((unsigned)M), dim3(256), 2 * L * sizeof(float),
                      (hipStream_t)stream, x, coeffs, L, levels, dwt_size, ldc);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }

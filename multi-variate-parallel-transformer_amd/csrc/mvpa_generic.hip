@@ -194,11 +194,11 @@ static int launch_generic_t(const mvpa_fwd_args* a, hipStream_t stream) {
   const int chan_table = (base + table <= 150 * 1024) ? 1 : 0;
   const size_t lds = base + (chan_table ? table : 0);
   auto kern = mvpa_generic_kernel<T, DH>;
-  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  mvpa::want_dynamic_lds((const void*)kern, (int)lds);
   const int n_rows = (a->flags & MVPA_FLAG_LAST_STEP) ? a->C : N;
   dim3 grid((n_rows + GEN_THREADS - 1) / GEN_THREADS, a->B * a->H);
   MVPA_LAUNCH(kern, grid, dim3(GEN_THREADS), lds, stream, *a, chan_table);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 template <typename T>
@@ -230,5 +230,5 @@ extern "C" int mvpa_debug_maps(int32_t T, int32_t C, int32_t window, uint32_t fl
   dim3 grid((N + 255) / 256, N);
   MVPA_LAUNCH(mvpa::mvpa_debug_maps_kernel, grid, dim3(256), 0, (hipStream_t)stream, T, C,
                      window, flags, chan_valid, time_idx, chan_idx, mask_bits);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }

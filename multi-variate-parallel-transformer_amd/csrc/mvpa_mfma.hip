@@ -890,8 +890,7 @@ static int launch_one(const mvpa_fwd_args* a, hipStream_t stream) {
   if (!content) n_split = 1;
   auto kern = (n_split > 1 || ring) ? mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH, true>
                           : mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH, false>;
-  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)G::LDS_BYTES);
+  mvpa::want_dynamic_lds((const void*)kern, (int)G::LDS_BYTES);
   const int nt = (G::TQW == 2 && STAGES == 4 && KH == 1) ? 1 + a->T / 2 : (a->T + G::TQW - 1) / G::TQW;   // as in the kernel
   dim3 grid((unsigned)((last ? n_split : nt) * a->B * a->H));
   MVPA_LAUNCH(kern, grid, dim3(G::THREADS), G::LDS_BYTES, stream, *a);
@@ -899,7 +898,7 @@ static int launch_one(const mvpa_fwd_args* a, hipStream_t stream) {
     const int rows = a->B * a->H * a->C;
     MVPA_LAUNCH(mvpa_split_merge_kernel<DH>, dim3((unsigned)((rows + 2048 / DH - 1) / (2048 / DH))), dim3(256), 0, stream, *a);
   }
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 template <int DH, int NCT, int NW, int STAGES, int MINB = 1, int KH = 1>
@@ -926,6 +925,9 @@ int mvpa_mfma_supported(const mvpa_fwd_args* a) {
   // per-sample element offsets are kept in 32 bits inside the kernel
   const int64_t n = (int64_t)a->T * a->C;
   if (n * a->k_stride_n >= ((int64_t)1 << 31) || n * a->v_stride_n >= ((int64_t)1 << 31)) return 0;
+  // so are the byte offsets of q and o rows (2 bytes per element)
+  const int64_t nq = (a->flags & MVPA_FLAG_LAST_STEP) ? a->C : n;
+  if (nq * a->q_stride_n >= ((int64_t)1 << 30) || nq * a->o_stride_n >= ((int64_t)1 << 30)) return 0;
   return 1;
 }
 

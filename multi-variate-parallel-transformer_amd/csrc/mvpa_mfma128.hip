@@ -672,10 +672,10 @@ static int launch128(const mvpa_fwd_args* a, hipStream_t stream) {
   using namespace mvpa::d128;
   using G = Geo<DH, NCT>;
   auto kern = mvpa_mfma128_kernel<DH, NCT, FP8>;
-  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
+  mvpa::want_dynamic_lds((const void*)kern, (int)G::LDS_BYTES);
   const int nt = (a->T + G::TQW - 1) / G::TQW;
   MVPA_LAUNCH(kern, dim3((unsigned)(nt * a->B * a->H)), dim3(NW * 64), G::LDS_BYTES, stream, *a);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }
 
 int mvpa_launch_mfma128(const mvpa_fwd_args* a, hipStream_t stream) {

@@ -754,9 +754,9 @@ int mvpa_mfma64_supported(const mvpa_fwd_args* a) {
 
 int mvpa_launch_mfma64(const mvpa_fwd_args* a, hipStream_t stream) {
   using namespace mvpa::q64;
-  (void)hipFuncSetAttribute((const void*)mvpa_mfma64_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+  mvpa::want_dynamic_lds((const void*)mvpa_mfma64_kernel, (int)LDS_BYTES);
   const bool own_last = (a->flags & MVPA_FLAG_CONTENT) && a->T > 1;       // as in the kernel
   const int nt = ((own_last ? a->T - 1 : a->T) + TQW - 1) / TQW + (own_last ? 1 : 0);
   MVPA_LAUNCH(mvpa_mfma64_kernel, dim3((unsigned)(nt * a->B * a->H)), dim3(NW * 64), LDS_BYTES, stream, *a);
-  return hipGetLastError() == hipSuccess ? MVPA_OK : MVPA_ERR_LAUNCH;
+  return mvpa::take_launch_status();
 }

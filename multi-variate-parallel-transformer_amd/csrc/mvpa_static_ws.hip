@@ -23,16 +23,17 @@ void* scratch_on_current_device() {
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
   void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
   if (p) return p;
-  if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
-    (void)hipGetLastError();
-    return nullptr;
-  }
+  if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
   g_scratch_ptr[dev].store(p, std::memory_order_release);   // racing first calls store the same value
   return p;
 }
 }  // namespace
 
 extern "C" size_t mvpa_static_ws_bytes(void) { return (size_t)MVPA_STATIC_WS_BYTES; }
+
+// Set-up call: looks the array's address on the current device up and keeps it, so that no later
+// call has to ask the runtime for it - in particular not the first call under stream capture.
+extern "C" int mvpa_static_ws_init(void) { return scratch_on_current_device() ? MVPA_OK : MVPA_ERR_LAUNCH; }
 
 extern "C" int mvpa_forward_last_step_static(const mvpa_fwd_args* a, void* stream) {
   if (!a) return MVPA_ERR_NULL;

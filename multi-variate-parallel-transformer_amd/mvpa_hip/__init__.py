@@ -106,6 +106,8 @@ def load_library() -> ctypes.CDLL:
     lib.mvpa_forward_last_step_static.argtypes = [ctypes.POINTER(MvpaFwdArgs), vp]
     lib.mvpa_static_ws_bytes.restype = ctypes.c_size_t
     lib.mvpa_static_ws_bytes.argtypes = []
+    lib.mvpa_static_ws_init.restype = ctypes.c_int
+    lib.mvpa_static_ws_init.argtypes = []
     lib.mvpa_backward.restype = ctypes.c_int
     lib.mvpa_backward.argtypes = [ctypes.POINTER(MvpaBwdArgs), vp]
     lib.mvpa_debug_maps.restype = ctypes.c_int
@@ -297,6 +299,7 @@ def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float]
         if n > 1:
             a.n_split = n
             if static_ws:
+                static_ws_init(q.device)
                 _check(lib.mvpa_forward_last_step_static(ctypes.byref(a), _stream()))
                 return (out, lse) if return_lse else out
             ws = torch.empty(lib.mvpa_split_ws_bytes(ctypes.byref(a)), dtype=torch.uint8, device=q.device)
@@ -305,6 +308,21 @@ def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float]
         raise ValueError("static_ws needs last_step_only on the bf16 matrix-core kernel with more than one key run")
     _check(lib.mvpa_forward(ctypes.byref(a), _stream()))
     return (out, lse) if return_lse else out
+
+
+_static_ws_ready = set()
+
+
+def static_ws_init(device=None) -> None:
+    """Set-up of mvpa_forward_last_step_static on a GPU (mvpa_static_ws_init with that GPU
+    current): call it once per GPU before recording the step into a graph."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    if idx in _static_ws_ready:
+        return
+    with torch.cuda.device(idx):
+        _check(load_library().mvpa_static_ws_init())
+    _static_ws_ready.add(idx)
 
 
 def mvpa_backward(q, k, v, o, d_o, lse, u, vb, z, k_time, k_chan, *,

@@ -91,6 +91,26 @@ def test_validate_key_split_arguments(lib):
         assert n >= 1 and (n - 1) * ((T + n - 1) // n) < T
 
 
+def test_wide_row_pitch_leaves_the_matrix_core_kernels(lib):
+    """The matrix-core kernels keep the offsets of q and o rows of a sample in 32 bits: a view whose
+    row pitch makes them wrap must not be taken by them (AUTO falls back to the row-per-lane
+    kernel, a forced matrix-core selector is refused).  Host-side only: nothing is launched."""
+    a, keep = _args(B=1, H=2, Hkv=2, T=64, C=64, Dh=64, dtype=torch.bfloat16)
+    assert lib.mvpa_select_kernel(ctypes.byref(a)) == mvpa_hip.KERNEL_MFMA
+    for field in ("q_stride_n", "o_stride_n", "k_stride_n", "v_stride_n"):
+        a, keep = _args(B=1, H=2, Hkv=2, T=64, C=64, Dh=64, dtype=torch.bfloat16)
+        setattr(a, field, 1 << 20)                              # 4096 rows x 2^20 elements
+        assert lib.mvpa_select_kernel(ctypes.byref(a)) == mvpa_hip.KERNEL_GENERIC, field
+        for forced in (mvpa_hip.KERNEL_MFMA, mvpa_hip.KERNEL_MFMA_STEP, mvpa_hip.KERNEL_MFMA_SPLIT):
+            a.kernel = forced
+            assert lib.mvpa_validate(ctypes.byref(a)) == -8, field
+    # the pitch of a fused projection output at the largest benchmark shape stays inside
+    a, keep = _args(B=1, H=2, Hkv=2, T=64, C=64, Dh=64, dtype=torch.bfloat16)
+    a.T, a.C, a.q_stride_n, a.o_stride_n = 512, 128, 4096, 2048
+    a.k_stride_n = a.v_stride_n = 4096
+    assert lib.mvpa_select_kernel(ctypes.byref(a)) == mvpa_hip.KERNEL_MFMA
+
+
 def test_null_block(lib):
     assert lib.mvpa_validate(None) == -1
 

@@ -149,7 +149,7 @@ def test_mvpformer_s_full_size_properties():
     through properties that need no oracle: finite scores, and time-causality of the whole stack,
     bit for bit - changing the last k segments leaves the hidden states of every earlier segment
     untouched."""
-    from models.bench_model import build_mvpformer_s
+    from bench_model import build_mvpformer_s
     model = build_mvpformer_s(512)
     x = make_ieeg(4, 64, 64, 512, seed=0).cuda()
     out, _ = model._common_forward(x)

@@ -73,3 +73,54 @@ def test_static_workspace_limits():
                                 key_splits=8, static_ws=True, out=out)
     want = mvpa_hip.mvpa_forward(inp.q[:, :, -128:], inp.k, inp.v, *tabs, last_step_only=True, key_splits=8)
     assert torch.equal(got, want)
+
+
+def test_static_step_allocates_nothing_and_replays_in_a_graph():
+    """With every buffer in place beforehand the entry point leaves the allocator's counters where
+    they were, and a step recorded into a HIP graph (after mvpa_static_ws_init, so that nothing is
+    looked up during capture) gives on every replay what the eager caller-workspace step gives on
+    the same cache contents - replays with eager work and synchronisations between them."""
+    lib = mvpa_hip.load_library()
+    cfg = dict(B=2, C=64, T=40, H=4, Hkv=2, Dh=64)
+    B, C, T, H, Dh = cfg["B"], cfg["C"], cfg["T"], cfg["H"], cfg["Dh"]
+    inp = make_mvpa_inputs(seed=61, qkv_unit=True, **cfg).to("cuda", torch.bfloat16)
+    q_last = inp.q[:, :, -C:].contiguous()
+    out = torch.zeros((B, H, C, Dh), dtype=torch.bfloat16, device="cuda")
+    tabs = [t.contiguous() for t in (inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan)]
+    a = mvpa_hip.make_args(q_last, inp.k, inp.v, out, *tabs, T=T, C=C, sm_scale=Dh ** -0.5,
+                           flags=15 | mvpa_hip.FLAG_LAST_STEP, kernel=mvpa_hip.KERNEL_MFMA, n_split=5)
+    assert lib.mvpa_static_ws_init() == 0
+    stream = torch.cuda.current_stream().cuda_stream
+    torch.cuda.synchronize()
+    before = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+    assert lib.mvpa_forward_last_step_static(ctypes.byref(a), stream) == 0
+    torch.cuda.synchronize()
+    assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == before
+    eager = out.clone()
+
+    def caller_ws_step():
+        res = torch.empty_like(out)
+        b = mvpa_hip.make_args(q_last, inp.k, inp.v, res, *tabs, T=T, C=C, sm_scale=Dh ** -0.5,
+                               flags=15 | mvpa_hip.FLAG_LAST_STEP, kernel=mvpa_hip.KERNEL_MFMA, n_split=5)
+        ws = torch.empty(lib.mvpa_split_ws_bytes(ctypes.byref(b)), dtype=torch.uint8, device="cuda")
+        b.split_ws = ws.data_ptr()
+        assert lib.mvpa_forward(ctypes.byref(b), torch.cuda.current_stream().cuda_stream) == 0
+        torch.cuda.synchronize()
+        return res
+
+    assert torch.equal(eager, caller_ws_step())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        st = lib.mvpa_forward_last_step_static(ctypes.byref(a), torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    for i in range(4):
+        # new cache contents and a new query in the same buffers, written by eager work
+        fresh = make_mvpa_inputs(seed=70 + i, qkv_unit=True, **cfg).to("cuda", torch.bfloat16)
+        inp.k.copy_(fresh.k)
+        inp.v.copy_(fresh.v)
+        q_last.copy_(fresh.q[:, :, -C:])
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, caller_ws_step()), f"replay {i}"
