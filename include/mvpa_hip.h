@@ -242,6 +242,14 @@ int mvpa_backward(const mvpa_bwd_args* args, void* stream);
  * MVPA_KERNEL_MFMA (or a negative status). */
 int mvpa_select_kernel(const mvpa_fwd_args* args);
 
+/* Host-only: the order in which the matrix-core forward kernels hand their work out.  Workgroup L
+ * of a launch with n_bh (batch, head) pairs and n_tiles time tiles each takes time tile tile[L] of
+ * pair bh[L]; workgroups whose ids are equal mod 8 run on one XCD (one L2), and the map keeps the
+ * heads of a kv group (heads_per_kv = H / Hkv neighbours in bh) on one XCD and side by side in
+ * time.  The reference's grid is (query tiles, B*H) in plain order (attentions/attn.py:1048).
+ * bh and tile hold n_bh * n_tiles entries.  Launches nothing. */
+int mvpa_debug_block_order(int32_t n_bh, int32_t n_tiles, int32_t heads_per_kv, int32_t* bh, int32_t* tile);
+
 /*
  * Index/mask maps exactly as the kernels compute them, for bit-exact tests against
  * layers/mvpa.py:127-159 (shifts) and :230-264 (window and causal masks).

@@ -2,6 +2,7 @@
 // Nothing here touches device memory, so mvpa_validate / mvpa_select_kernel work on a machine
 // without a GPU.
 #include "mvpa_common.h"
+#include "mvpa_mfma_tools.h"
 
 extern "C" int mvpa_version(void) { return MVPA_ABI_VERSION; }
 
@@ -83,6 +84,19 @@ extern "C" int mvpa_validate(const mvpa_fwd_args* a) {
 extern "C" size_t mvpa_split_ws_bytes(const mvpa_fwd_args* a) {
   if (!a || a->n_split <= 1) return 0;
   return (size_t)a->n_split * a->B * a->H * a->C * ((size_t)a->Dh * 2 + sizeof(float));
+}
+
+extern "C" int mvpa_debug_block_order(int32_t n_bh, int32_t n_tiles, int32_t heads_per_kv, int32_t* bh,
+                                      int32_t* tile) {
+  if (!bh || !tile) return MVPA_ERR_NULL;
+  if (n_bh <= 0 || n_tiles <= 0 || heads_per_kv <= 0) return MVPA_ERR_SHAPE;
+  for (int L = 0; L < n_bh * n_tiles; ++L) {
+    int x, y;
+    mvpa::map_block(L, n_bh, n_tiles, heads_per_kv, x, y);
+    bh[L] = x;
+    tile[L] = y;
+  }
+  return MVPA_OK;
 }
 
 extern "C" int mvpa_select_kernel(const mvpa_fwd_args* a) {

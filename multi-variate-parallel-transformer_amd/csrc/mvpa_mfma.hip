@@ -110,7 +110,6 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   constexpr bool SPLIT = G::TQW == 2 && STAGES == 4 && KH == 1;
   const int nt = SPLIT ? 1 + T_ / 2 : (T_ + G::TQW - 1) / G::TQW;
   const int nbh = a.B * a.H;
-  constexpr int TAIL_MERGE = 2;
   // MVPA_FLAG_LAST_STEP: only the workgroup of the last time step runs, one per (b, h); q, o and
   // lse are indexed by channel alone
   const bool last_only = a.flags & MVPA_FLAG_LAST_STEP;
@@ -120,40 +119,8 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     if (last_only) {
       bh = n_split > 1 ? L % nbh : L;
       tile = nt - 1;
-    } else if ((nbh & 7) == 0 && nt > 1) {
-      if (L < nbh) {
-        bh = L;                          // L & 7 is the XCD, the same one as below for this (b, h)
-        tile = nt - 1;
-      } else {
-        // the other nt-1 tiles: one (b, h) of the XCD after the other, long tiles first; the
-        // last TAIL_MERGE (b, h) of the XCD are interleaved tile by tile so that the grid does
-        // not end on the long tiles of a single (b, h)
-        const int L2 = L - nbh;
-        const int xcd = L2 & 7, per_xcd = nbh >> 3, s = L2 >> 3;
-        const int merged = per_xcd < TAIL_MERGE ? per_xcd : TAIL_MERGE;
-        const int plain = (per_xcd - merged) * (nt - 1);
-        if (s < plain) {
-          bh = xcd + 8 * (s / (nt - 1));
-          tile = nt - 2 - s % (nt - 1);
-        } else {
-          const int r = s - plain;
-          bh = xcd + 8 * (per_xcd - merged + r % merged);
-          tile = nt - 2 - r / merged;
-        }
-      }
-    } else if (nt > 1) {
-      // no XCD affinity to keep (the (b, h) do not divide over the 8 XCDs): last tiles first,
-      // then (b, h) by (b, h)
-      if (L < nbh) {
-        bh = L;
-        tile = nt - 1;
-      } else {
-        bh = (L - nbh) / (nt - 1);
-        tile = nt - 2 - (L - nbh) % (nt - 1);
-      }
     } else {
-      bh = L;
-      tile = 0;
+      map_block(L, nbh, nt, a.H / a.Hkv, bh, tile);
     }
   }
   const int b = bh / a.H, h = bh % a.H;

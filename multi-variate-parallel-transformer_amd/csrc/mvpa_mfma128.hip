@@ -80,41 +80,8 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
   // (b, h) of an XCD are interleaved so that the grid does not end on the long steps of one.
   const int nt = (T_ + TQW - 1) / TQW;
   const int nbh = a.B * a.H;
-  constexpr int TAIL_MERGE = 2;
   int bh, tile;
-  {
-    const int L = blockIdx.x;
-    if ((nbh & 7) == 0 && nt > 1) {
-      if (L < nbh) {
-        bh = L;
-        tile = nt - 1;
-      } else {
-        const int L2 = L - nbh;
-        const int xcd = L2 & 7, per_xcd = nbh >> 3, s = L2 >> 3;
-        const int merged = per_xcd < TAIL_MERGE ? per_xcd : TAIL_MERGE;
-        const int plain = (per_xcd - merged) * (nt - 1);
-        if (s < plain) {
-          bh = xcd + 8 * (s / (nt - 1));
-          tile = nt - 2 - s % (nt - 1);
-        } else {
-          const int r = s - plain;
-          bh = xcd + 8 * (per_xcd - merged + r % merged);
-          tile = nt - 2 - r / merged;
-        }
-      }
-    } else if (nt > 1) {
-      if (L < nbh) {
-        bh = L;
-        tile = nt - 1;
-      } else {
-        bh = (L - nbh) / (nt - 1);
-        tile = nt - 2 - (L - nbh) % (nt - 1);
-      }
-    } else {
-      bh = L;
-      tile = 0;
-    }
-  }
+  map_block(blockIdx.x, nbh, nt, a.H / a.Hkv, bh, tile);
   const int b = bh / a.H, h = bh % a.H;
   const int g = h / (a.H / a.Hkv);
   const int tq0 = tile * TQW, tq_hi = min(T_ - 1, tq0 + TQW - 1);

@@ -64,41 +64,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
   const int t_main = own_last ? T_ - 1 : T_;
   const int nt = (t_main + TQW - 1) / TQW + (own_last ? 1 : 0);
   const int nbh = a.B * a.H;
-  constexpr int TAIL_MERGE = 2;
   int bh, tile;
-  {
-    const int L = blockIdx.x;
-    if ((nbh & 7) == 0 && nt > 1) {
-      if (L < nbh) {
-        bh = L;
-        tile = nt - 1;
-      } else {
-        const int L2 = L - nbh;
-        const int xcd = L2 & 7, per_xcd = nbh >> 3, s = L2 >> 3;
-        const int merged = per_xcd < TAIL_MERGE ? per_xcd : TAIL_MERGE;
-        const int plain = (per_xcd - merged) * (nt - 1);
-        if (s < plain) {
-          bh = xcd + 8 * (s / (nt - 1));
-          tile = nt - 2 - s % (nt - 1);
-        } else {
-          const int r = s - plain;
-          bh = xcd + 8 * (per_xcd - merged + r % merged);
-          tile = nt - 2 - r / merged;
-        }
-      }
-    } else if (nt > 1) {
-      if (L < nbh) {
-        bh = L;
-        tile = nt - 1;
-      } else {
-        bh = (L - nbh) / (nt - 1);
-        tile = nt - 2 - (L - nbh) % (nt - 1);
-      }
-    } else {
-      bh = L;
-      tile = 0;
-    }
-  }
+  map_block(blockIdx.x, nbh, nt, a.H / a.Hkv, bh, tile);
   const int b = bh / a.H, h = bh % a.H;
   const int g = h / (a.H / a.Hkv);
   const bool last_wg = own_last && tile == nt - 1;

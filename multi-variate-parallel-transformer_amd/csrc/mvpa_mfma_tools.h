@@ -157,4 +157,60 @@ template <int DH> __device__ inline int swz_v(int row) {
   return DH == 64 ? (((row >> 1) & 1) << 2) : DH == 128 ? ((row & 3) << 2) : 0;
 }
 
+// ---- workgroup id -> ((b, h), time tile) ---------------------------------------------------
+// Workgroup ids that are equal mod 8 run on one XCD and share its L2.  An XCD is given a
+// contiguous range of (b, h) - with grouped-query attention the heads of one kv group are
+// neighbours there, so the K/V of a kv head fill ONE L2, once - and walks it in this order:
+//   * first the LAST time tile of every (b, h) it owns (the last time step keeps the content
+//     term for every key step, layers/mvpa.py:244, and takes several times longer than any other
+//     tile: it must not be what the grid ends on);
+//   * then unit by unit, a unit being the heads of one kv group (one head without grouping),
+//     late (= long) tiles first, the heads of the unit side by side on a tile so that they
+//     stream the same K/V tiles at the same time;
+//   * the last two units are interleaved tile by tile, so that the grid does not end on the long
+//     tiles of a single unit.
+// Without XCD affinity to keep (the (b, h) do not divide over 8 XCDs): last tiles first, then
+// (b, h) by (b, h).
+__host__ __device__ inline void map_block(int L, int nbh, int nt, int grp, int& bh, int& tile) {
+  constexpr int TAIL_MERGE = 2;
+  if (nt <= 1) {
+    bh = L;
+    tile = 0;
+    return;
+  }
+  if ((nbh & 7) != 0) {
+    if (L < nbh) {
+      bh = L;
+      tile = nt - 1;
+    } else {
+      bh = (L - nbh) / (nt - 1);
+      tile = nt - 2 - (L - nbh) % (nt - 1);
+    }
+    return;
+  }
+  const int per_xcd = nbh >> 3;
+  if (L < nbh) {
+    bh = (L & 7) * per_xcd + (L >> 3);
+    tile = nt - 1;
+    return;
+  }
+  const int L2 = L - nbh;
+  const int xcd = L2 & 7, s = L2 >> 3;
+  const int u = (grp > 1 && per_xcd % grp == 0) ? grp : 1;      // heads per unit
+  const int n_units = per_xcd / u, items = u * (nt - 1);
+  const int merged = n_units < TAIL_MERGE ? n_units : TAIL_MERGE;
+  const int plain = (n_units - merged) * items;
+  int unit, i;
+  if (s < plain) {
+    unit = s / items;
+    i = s % items;
+  } else {
+    const int r = s - plain;
+    unit = n_units - merged + r % merged;
+    i = r / merged;
+  }
+  bh = xcd * per_xcd + unit * u + i % u;
+  tile = nt - 2 - i / u;
+}
+
 }  // namespace mvpa

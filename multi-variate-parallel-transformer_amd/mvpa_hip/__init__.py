@@ -110,6 +110,8 @@ def load_library() -> ctypes.CDLL:
     lib.mvpa_static_ws_init.argtypes = []
     lib.mvpa_backward.restype = ctypes.c_int
     lib.mvpa_backward.argtypes = [ctypes.POINTER(MvpaBwdArgs), vp]
+    lib.mvpa_debug_block_order.restype = ctypes.c_int
+    lib.mvpa_debug_block_order.argtypes = [i32, i32, i32, vp, vp]
     lib.mvpa_debug_maps.restype = ctypes.c_int
     lib.mvpa_debug_maps.argtypes = [i32, i32, i32, u32, vp, vp, vp, vp, vp]
     lib.mvpa_linear_bf16.restype = ctypes.c_int

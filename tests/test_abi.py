@@ -111,6 +111,37 @@ def test_wide_row_pitch_leaves_the_matrix_core_kernels(lib):
     assert lib.mvpa_select_kernel(ctypes.byref(a)) == mvpa_hip.KERNEL_MFMA
 
 
+@pytest.mark.parametrize("B,H,Hkv,nt", [(4, 16, 16, 33), (4, 12, 4, 33), (1, 16, 8, 512), (8, 16, 16, 128),
+                                        (2, 8, 2, 5), (3, 5, 5, 7), (1, 4, 1, 9), (2, 16, 4, 1), (1, 16, 8, 2)])
+def test_block_order_is_a_permutation_and_keeps_kv_groups_on_one_xcd(lib, B, H, Hkv, nt):
+    """Every (pair, tile) is handed out exactly once; the last tile of every pair goes out first;
+    and where the pairs divide over the 8 XCDs, the heads of a kv group share an XCD whenever an
+    XCD's share of heads is a whole number of groups."""
+    import numpy as np
+    nbh, grp = B * H, H // Hkv
+    bh = np.full(nbh * nt, -1, dtype=np.int32)
+    tile = np.full(nbh * nt, -1, dtype=np.int32)
+    assert lib.mvpa_debug_block_order(nbh, nt, grp, bh.ctypes.data, tile.ctypes.data) == 0
+    seen = set(zip(bh.tolist(), tile.tolist()))
+    assert len(seen) == nbh * nt and min(bh) == 0 and max(bh) == nbh - 1 and min(tile) == 0 and max(tile) == nt - 1
+    if nt > 1:
+        assert set(tile[:nbh].tolist()) == {nt - 1} and (nt - 1) not in set(tile[nbh:].tolist())
+    if nbh % 8 == 0 and nt > 1:
+        xcd = np.arange(nbh * nt) % 8
+        owner = {}
+        for x, p in zip(xcd.tolist(), bh.tolist()):
+            assert owner.setdefault(p, x) == x, "a (b, h) pair is split over two XCDs"
+        if (nbh // 8) % grp == 0:
+            for p, x in owner.items():
+                assert owner[(p // grp) * grp] == x, "a kv group is split over two XCDs"
+            # within a group the heads take a tile side by side
+            first = nbh + int(np.argmax(xcd[nbh:] == 0))
+            if grp > 1:
+                run = [(int(bh[first + 8 * i]), int(tile[first + 8 * i])) for i in range(grp * (2 if nbh // 8 // grp == 2 else 1))]   # two units: interleaved
+                mine = [(p, t) for p, t in run if p // grp == run[0][0] // grp]
+                assert len({p for p, _ in mine}) == grp and len({t for _, t in mine}) == 1
+
+
 def test_null_block(lib):
     assert lib.mvpa_validate(None) == -1
 
