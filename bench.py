@@ -1,8 +1,9 @@
 #!/usr/bin/env python3
 """Benchmark of the MVPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3] [--no-cpu] [--no-model]
-                    [--no-stream] [--no-backward] [--base-model] [--copy-probe] [--prewarm P]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c5attn] [--no-cpu]
+                    [--no-model] [--no-stream] [--no-backward] [--no-extra] [--no-base-model]
+                    [--base-stream] [--copy-probe] [--prewarm P]
 
 A step is one fused MVPA forward (one kernel launch) over one batch of synthetic inputs that
 are already resident in HBM.  The default workload is the configuration the headline metric
@@ -13,7 +14,10 @@ restatement of the reference PyTorch path on this box's host cores).  Beside the
 of `value`: `backward` (one mvpa_backward call on the same workload), `mvpformer_s` (the
 MVPFormer-S forward in windows per second, with the oracle stack on the host cores beside it),
 `mvpformer_s_stream` (one new segment of a stream against cached keys and values, beside the
-full forward over the same window) and, on request, `mvpformer_base`.
+full forward over the same window), `mvpa_c3` and `mvpa_c5attn` (the irregular-channel
+configuration and the base model's attention shape, a few launches each: time, algorithmic
+TFLOP/s, fraction of the bf16 peak, kernel) and `mvpformer_base` (the base-size classification
+forward at B1 C128 T512, bf16 and fp8 QK^T, with the logit gap between the two).
 
 The GPU's clocks take a few dozen milliseconds of work to reach their steady state after a
 process starts.  Before the W warm-up steps the benchmark therefore runs a fixed number of
@@ -74,6 +78,41 @@ def algorithmic_flops(B, H, T, C, Dh, window=10):
     else:
         p_window = p_causal
     return B * H * 2 * Dh * (p_causal + p_window + n * (T + C))
+
+
+def _extra_workload(key, warmup=3, steps=5):
+    """One of the other benchmark shapes on the library's own kernel choice: HIP-event time per
+    launch over `steps` launches, algorithmic TFLOP/s and the fraction of the dense bf16 peak."""
+    import torch
+    import mvpa_hip
+    from mvpa_hip.synthetic import make_mvpa_inputs
+
+    cfg = WORKLOADS[key]
+    B, C, T, H, Hkv, Dh = (cfg[k] for k in ("B", "C", "T", "H", "Hkv", "Dh"))
+    d = make_mvpa_inputs(B=B, C=C, T=T, H=H, Hkv=Hkv, Dh=Dh, seed=0, qkv_unit=True,
+                         validity=cfg["validity"]).to("cuda:0", torch.bfloat16)
+    out = torch.empty_like(d.q)
+
+    def step():
+        mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
+                              chan_valid=d.chan_valid, out=out)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    ms = ev0.elapsed_time(ev1) / steps
+    flops = algorithmic_flops(B, H, T, C, Dh)
+    tf = flops / (ms * 1e-3) / 1e12
+    return {"workload": f"B={B} C={C} T={T} H={H} Hkv={Hkv} Dh={Dh}"
+                        + (", per-sample channel validity" if cfg["validity"] else ""),
+            "ms": round(ms, 4), "steps": steps, "tflops": round(tf, 1),
+            "frac": round(tf / BF16_DENSE_PEAK_TFLOPS, 4), "algorithmic_flops": flops,
+            "kernel": _forward_kernel_name(cfg)}
 
 
 def cpu_baseline(cfg, budget_s=8.0):
@@ -147,16 +186,17 @@ def cpu_baseline_model(B=1, C=64, T=64, seg=512):
     with torch.no_grad():
         O.mvpformer_forward(x[:, :8], params, dict(n_layer=1, n_head=H, n_head_kv=Hkv))   # thread pool warm-up
         for n_layer in (0, 1):
-            t0 = time.perf_counter()
-            O.mvpformer_forward(x, params, dict(n_layer=n_layer, n_head=H, n_head_kv=Hkv))
-            times[n_layer] = time.perf_counter() - t0
+            for _ in range(2):      # the second call is the one reported: the first also pays for
+                t0 = time.perf_counter()         # allocator and thread-pool warm-up at this size
+                O.mvpformer_forward(x, params, dict(n_layer=n_layer, n_head=H, n_head_kv=Hkv))
+                times[n_layer] = time.perf_counter() - t0
     per_block = max(times[1] - times[0], 1e-9)
     full = times[0] + MVPFORMER_S["n_layer"] * per_block
     return {"value": round(B / full, 4), "unit": "windows/s", "cores": torch.get_num_threads(),
             "kind": "port",
             "sample": f"oracle stack, fp32, B={B} C={C} T={T} segments of {seg} samples: encoder + final "
-                      f"norm {times[0]:.2f} s, one block {per_block:.2f} s (timed once, first call at this "
-                      f"size); extrapolated to 12 blocks: {full:.1f} s per window"}
+                      f"norm {times[0]:.2f} s, one block {per_block:.2f} s (each timed twice, the second "
+                      f"call reported); extrapolated to 12 blocks: {full:.1f} s per window"}
 
 
 def main():
@@ -171,8 +211,12 @@ def main():
     ap.add_argument("--no-model", action="store_true", help="skip the MVPFormer-S forward leg")
     ap.add_argument("--no-stream", action="store_true", help="skip the MVPFormer-S streamed-segment leg")
     ap.add_argument("--no-backward", action="store_true", help="skip the MVPA backward leg")
-    ap.add_argument("--base-model", action="store_true",
-                    help="also time the base-size classification forward (B1 C128 T512, bf16 and fp8 QK^T)")
+    ap.add_argument("--no-extra", action="store_true", help="skip the c3 and c5-attention legs")
+    ap.add_argument("--no-base-model", action="store_true",
+                    help="skip the base-size classification forward (B1 C128 T512, bf16 and fp8 QK^T)")
+    ap.add_argument("--base-model", action="store_true", help=argparse.SUPPRESS)   # (now the default)
+    ap.add_argument("--base-stream", action="store_true",
+                    help="with the base-size forward: also time its streamed segments")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 256 MiB device copy (calibrates HBM traffic counters)")
     args = ap.parse_args()
@@ -264,6 +308,13 @@ def main():
         line["backward"] = {"ms_per_step": round(ev0.elapsed_time(ev1) / n_bwd, 4), "steps": n_bwd,
                             "kernels": "mvpa_bwd_query_mfma_kernel + mvpa_bwd_key_mfma_kernel",
                             "outputs": "dq (content share), dk, dv, dbias_time, dbias_chan (fp32)"}
+    if not args.no_extra:
+        # the other attention shapes of the benchmark set, a few launches each, beside the headline
+        # and never part of `value`: the irregular-channel configuration and the attention shape of
+        # the base model
+        for key in ("c3", "c5attn"):
+            if key != args.workload:
+                line["mvpa_" + key] = _extra_workload(key)
     if not args.no_model:
         try:
             from bench_model import mvpformer_s_windows_per_s
@@ -273,9 +324,9 @@ def main():
                 line["mvpformer_s_stream"] = mvpformer_s_stream_step_ms()
         except ImportError:
             line["mvpformer_s"] = None
-    if args.base_model:
+    if not args.no_base_model:
         from bench_model import mvpformer_base_forward_ms
-        line["mvpformer_base"] = mvpformer_base_forward_ms(stream=not args.no_stream)
+        line["mvpformer_base"] = mvpformer_base_forward_ms(stream=args.base_stream)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(cfg)
         if line.get("mvpformer_s"):

@@ -241,6 +241,42 @@ def test_base_classification_bf16_then_fp8():
     assert e16 <= 3e-2 and e8 <= 6e-2
 
 
+def test_base_classification_full_size_properties():
+    """The base-size classification forward at the benchmark's full size (B1 C128 T512 segments of
+    512 samples, 24 layers, Dh 128), through properties that need no oracle: finite logits,
+    time-causality of the whole stack bit for bit, and the bf16 / fp8-QK^T logit gap inside the
+    stated 6e-2 of the logit spread."""
+    from models.configs import MVPFORMER_BASE
+    from models.fftencoder import WaveEncoder
+    from models.mvpformer import HMVPFormer, MVPFormerConfig, MVPFormerHead
+    T, C = 512, 128
+    x = make_ieeg(1, C, T, 512, seed=7).cuda()
+    x2 = x.clone()
+    x2[:, -40:] = x2[:, -40:].flip(-1) * 1.5
+    logits = {}
+    for fp8 in (False, True):
+        torch.manual_seed(3)
+        cfg = MVPFormerConfig(**dict(MVPFORMER_BASE, n_positions=T), fp8_qk=fp8)
+        model = HMVPFormer(cfg, WaveEncoder(512, cfg.n_embd), MVPFormerHead(cfg.n_embd, 2))
+        model = model.to(device="cuda", dtype=torch.bfloat16).eval()
+        assert len(model.mvpformer.h) == 24
+        out, _ = model._common_forward(x)
+        assert out.shape == (1, T, C, 2048) and torch.isfinite(out.float()).all()
+        logits[fp8] = model.classify(x).float().cpu()
+        assert logits[fp8].shape == (1, 2) and torch.isfinite(logits[fp8]).all()
+        if not fp8:
+            out2, _ = model._common_forward(x2)
+            assert torch.equal(out2[:, :-40], out[:, :-40])
+            assert not torch.equal(out2[:, -40:], out[:, -40:])
+            del out2
+        del model, out
+        torch.cuda.empty_cache()
+    spread = logits[False].abs().max().item() + 1e-6
+    gap = (logits[True] - logits[False]).abs().max().item() / spread
+    print(f"base model, full size: logits {logits[False].flatten().tolist()}, fp8 gap {gap:.3e} of the spread")
+    assert gap <= 6e-2
+
+
 @pytest.mark.parametrize("flash", [True, False], ids=["flash", "masked"])
 def test_layer_incremental_step_matches_full_forward(flash):
     """use_cache / layer_past: the layer run on T-1 time steps with use_cache, then on the last

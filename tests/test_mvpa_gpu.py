@@ -945,3 +945,18 @@ def test_bf16_base_attention_shape_full_size(kern):
     o3 = mvpa_hip.mvpa_forward(d.q, k3, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, chan_valid=d.chan_valid, kernel=kern)
     same = (o3 == out).flatten(0, 1).all(-1).view(-1, T, C).all(0).all(-1).cpu()
     assert same.tolist() == [not (t <= 10 or t == T - 1) for t in range(T)]
+    # the fp8 content term at this length (far steps, 512 time-bias rows): the same sampled rows
+    # against the oracle within the stated fp8 tolerance, and the masks bit for bit
+    o8 = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
+                               chan_valid=d.chan_valid, kernel=kern, fp8_qk=True)
+    assert not torch.equal(o8, out)
+    tol = FP8_TOL[True]
+    for (r0, r1) in ranges:
+        got = o8[0, 11, r0:r1].float().cpu().view(-1, C, 128) * live
+        want = ref[0, 11, r0:r1].view(-1, C, 128) * live
+        err, rel = (got - want).abs().max().item(), _rel_l2(got, want)
+        assert err <= tol["max_abs"] and rel <= tol["rel_l2"], f"fp8 rows {r0}: max-abs {err:.3e}, rel-L2 {rel:.3e}"
+    # (values only: the keys enter the per-head fp8 scales, which are computed over every row)
+    o82 = mvpa_hip.mvpa_forward(d.q, d.k, v2, d.u, d.vb, d.z, d.k_time, d.k_chan, chan_valid=d.chan_valid,
+                                kernel=kern, fp8_qk=True)
+    assert torch.equal(o82[:, :, :-40 * C], o8[:, :, :-40 * C])
