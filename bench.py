@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MVPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c5attn] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4attn|c5attn] [--no-cpu]
                     [--no-model] [--no-stream] [--no-backward] [--no-extra] [--no-base-model]
                     [--base-stream] [--copy-probe] [--prewarm P]
 
@@ -53,6 +53,8 @@ WORKLOADS = {
     "c3": dict(B=8, C=117, T=256, H=16, Hkv=16, Dh=64, validity=True),
     # the attention shape inside configuration c5 (the base model: one sample, 128 channels, 512 segments)
     "c5attn": dict(B=1, C=128, T=512, H=16, Hkv=8, Dh=128, validity=False),
+    # the attention shape inside configuration c4 (MVPFormer-S: 64 channels, 64 segments, 3 heads per kv head)
+    "c4attn": dict(B=4, C=64, T=64, H=12, Hkv=4, Dh=64, validity=False),
 }
 
 

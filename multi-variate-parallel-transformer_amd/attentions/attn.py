@@ -25,34 +25,34 @@ class FlashMVPA(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, u, vb, z, k, k_time, k_chan, v, causal, sm_scale, window, time_bias,
-                chan_bias, chan_valid):
+                chan_bias, chan_valid, content=True, key_bias=None):
         out, lse = mvpa_hip.mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, sm_scale=sm_scale,
-                                         window=window, causal=causal, content=True,
+                                         window=window, causal=causal, content=content,
                                          time_bias=time_bias, chan_bias=chan_bias,
-                                         chan_valid=chan_valid, return_lse=True)
+                                         chan_valid=chan_valid, key_bias=key_bias, return_lse=True)
         ctx.save_for_backward(q, u, vb, z, k, k_time, k_chan, v, out, lse)
-        ctx.conf = (causal, sm_scale, window, time_bias, chan_bias, chan_valid)
+        ctx.conf = (causal, sm_scale, window, time_bias, chan_bias, chan_valid, content, key_bias)
         return out
 
     @staticmethod
     def backward(ctx, d_out):
         q, u, vb, z, k, k_time, k_chan, v, out, lse = ctx.saved_tensors
-        causal, sm_scale, window, time_bias, chan_bias, chan_valid = ctx.conf
+        causal, sm_scale, window, time_bias, chan_bias, chan_valid, content, key_bias = ctx.conf
         dq_c, dk, dv, dbt, dbc = mvpa_hip.mvpa_backward(
             q, k, v, out, d_out.contiguous(), lse, u, vb, z, k_time, k_chan, sm_scale=sm_scale,
-            window=window, causal=causal, content=True, time_bias=time_bias, chan_bias=chan_bias,
-            chan_valid=chan_valid)
+            window=window, causal=causal, content=content, time_bias=time_bias, chan_bias=chan_bias,
+            chan_valid=chan_valid, key_bias=key_bias)
         B, H, N, Dh = q.shape
         Hkv = k.shape[1]
         grp = H // Hkv
-        qf = q.float().view(B, Hkv, grp, N, Dh)
+        qf = q.float().reshape(B, Hkv, grp, N, Dh)
         # time table (q+vb) @ k_time^T and channel table (q+z) @ k_chan^T, per kv head g
         dbt = dbt.view(B, Hkv, grp, N, -1)
         dbc = dbc.view(B, Hkv, grp, N, -1)
         rt, ec = k_time.float(), k_chan.float()                    # [Hkv,T,Dh], [Hkv,C,Dh]
         dq_cv = dq_c.view(B, Hkv, grp, N, Dh)
         dq = dq_cv
-        du = dq_cv.sum(dim=(0, 2, 3))
+        du = dq_cv.sum(dim=(0, 2, 3)) if content else torch.zeros_like(u, dtype=torch.float32)
         # a bias term that is switched off takes no part in the forward: its table, its query
         # bias and the query get nothing through it
         if time_bias:
@@ -71,7 +71,7 @@ class FlashMVPA(torch.autograd.Function):
             dz, dk_chan = torch.zeros_like(z, dtype=torch.float32), torch.zeros_like(ec)
         return (dq.view(B, H, N, Dh).to(q.dtype), du.to(u.dtype), dvb.to(vb.dtype), dz.to(z.dtype),
                 dk.to(k.dtype), dk_time.to(k_time.dtype), dk_chan.to(k_chan.dtype), dv.to(v.dtype),
-                None, None, None, None, None, None)
+                None, None, None, None, None, None, None, None)
 
 
 def flash_mvpa(

@@ -1,5 +1,5 @@
-from .mvpa import (MvpaKVCache, MvpaRingCache, MvpaRingClock, MVPFormerGQAAttention,
+from .mvpa import (KeyMask, MvpaKVCache, MvpaRingCache, MvpaRingClock, MVPFormerGQAAttention,
                    MVPFormerGQAFlashAttention)
 
-__all__ = ["MvpaKVCache", "MvpaRingCache", "MvpaRingClock", "MVPFormerGQAAttention",
+__all__ = ["KeyMask", "MvpaKVCache", "MvpaRingCache", "MvpaRingClock", "MVPFormerGQAAttention",
            "MVPFormerGQAFlashAttention"]

@@ -125,6 +125,30 @@ class MvpaRingCache:
         mvpa_hip.ring_append(k_new, v_new, self.k, self.v, self.clock.head32)
 
 
+class KeyMask:
+    """An additive key mask ([B,1,1,N], zeros and finfo.min: models/mvpformer.py:262-268) together
+    with what the kernels make of it, worked out ONCE for all the layers that receive it.  A mask
+    that is the same at every time step is a per-channel validity mask [B,C], which the bf16
+    kernels apply exactly; anything else goes on as an additive key bias [B,N] (fp32 kernel).
+    Built with chan_valid given, nothing is inspected and nothing synchronises with the device,
+    so a forward with such a mask can be recorded into a graph."""
+
+    def __init__(self, additive: Optional[torch.Tensor] = None, chan_valid: Optional[torch.Tensor] = None):
+        if additive is None and chan_valid is None:
+            raise ValueError("KeyMask needs the additive mask or the channel-validity mask")
+        self.additive = additive
+        self.chan_valid = chan_valid
+        self._resolved = chan_valid is not None
+
+    def resolve(self, bsz, t_len, c_len):
+        if not self._resolved:
+            self.chan_valid = MVPFormerGQAAttention._as_channel_validity(self.additive, bsz, t_len, c_len)
+            self._resolved = True
+        if self.chan_valid is not None:
+            return self.chan_valid, None
+        return None, self.additive.reshape(bsz, t_len * c_len).to(torch.float32)
+
+
 class _LoRALinear(torch.nn.Linear):
     """Bias-free Linear with low-rank adapters under the parameter names the reference's
     adapter library uses (lora_A, lora_B; layers/mvpa.py:43-62, 86-93).  `enable` marks which
@@ -275,6 +299,17 @@ class MVPFormerGQAAttention(torch.nn.Module):
         return self._tables
 
     @staticmethod
+    def _resolve_mask(attention_mask, bsz, t_len, c_len):
+        """(chan_valid, key_bias) for the kernels.  A KeyMask was analysed by whoever made it (the
+        stack does that once per forward, or is told the validity mask outright: no device
+        synchronisation here); a plain additive tensor is analysed now."""
+        if attention_mask is None:
+            return None, None
+        if isinstance(attention_mask, KeyMask):
+            return attention_mask.resolve(bsz, t_len, c_len)
+        return KeyMask(attention_mask).resolve(bsz, t_len, c_len)
+
+    @staticmethod
     def _as_channel_validity(attention_mask, bsz, t_len, c_len):
         """An additive key mask built from a 0/1 mask (models/mvpformer.py:262-268: zeros and
         finfo.min) that is the same at every time step is a per-channel validity mask, which the
@@ -305,7 +340,8 @@ class MVPFormerGQAAttention(torch.nn.Module):
         merged heads; c_proj is then left to the caller and merged_out is what comes back.
         qkv: hidden_states @ [q_attn; c_attn]^T when the caller has already formed it."""
         if self.training and (self.attn_dropout.p > 0 or self.resid_dropout.p > 0):
-            raise NotImplementedError("MVPA HIP layer: dropout/training is not implemented; call .eval()")
+            raise NotImplementedError("MVPA HIP layer: dropout is not implemented; train with "
+                                      "attn_pdrop = resid_pdrop = 0 or call .eval()")
         if self.is_cross_attention:
             raise NotImplementedError(
                 "MVPA HIP layer: without the time-causal mask the relative-time shift of the "
@@ -319,6 +355,9 @@ class MVPFormerGQAAttention(torch.nn.Module):
                 raise NotImplementedError("merged_out goes with a whole-sequence forward")
             return self._attend_step(hidden_states, positional_embedding, channel_embedding,
                                      attention_mask, head_mask, use_cache, window, layer_past)
+        if merged_out is None and qkv is None and self._wants_grad(hidden_states):
+            return self._attend_autograd(hidden_states, positional_embedding, channel_embedding,
+                                         attention_mask, head_mask, use_cache, window)
         with torch.no_grad():
             if qkv is None:
                 qkv = _linear(hidden_states, self._qkv_weight(dt))      # [B,T,C,E+2kvE]
@@ -329,11 +368,7 @@ class MVPFormerGQAAttention(torch.nn.Module):
             v = qkv[:, :, e + kv:].view(bsz, n, hkv, dh).permute(0, 2, 1, 3)
             k_time, k_chan = self._key_tables(positional_embedding, channel_embedding)
             u, vb, z = (b.view(hkv, dh) for b in self.attn_bias.split(kv, dim=0))
-            chan_valid, key_bias = None, None
-            if attention_mask is not None:
-                chan_valid = self._as_channel_validity(attention_mask, bsz, t_len, c_len)
-                if chan_valid is None:
-                    key_bias = attention_mask.reshape(bsz, n).to(torch.float32)
+            chan_valid, key_bias = self._resolve_mask(attention_mask, bsz, t_len, c_len)
             merged = merged_out if merged_out is not None else \
                 torch.empty((bsz, n, h, dh), dtype=dt, device=hidden_states.device)
             mvpa_hip.mvpa_forward(
@@ -352,6 +387,46 @@ class MVPFormerGQAAttention(torch.nn.Module):
                 _linear(merged.view(bsz, t_len, c_len, e), self.c_proj.weight)
         present = None
         if use_cache is True:                               # layers/mvpa.py:318-321
+            present = (k.reshape(bsz, hkv, t_len, c_len, dh), v.reshape(bsz, hkv, t_len, c_len, dh))
+        return out, present
+
+    def _wants_grad(self, hidden_states) -> bool:
+        """Gradients are produced when grad mode is on and either the input carries a graph or the
+        module is in train() mode (then for its parameters too); an eval() forward on a plain
+        input stays on the fused inference path even outside torch.no_grad()."""
+        return torch.is_grad_enabled() and (hidden_states.requires_grad or self.training)
+
+    def _attend_autograd(self, hidden_states, positional_embedding, channel_embedding, attention_mask,
+                         head_mask, use_cache, window):
+        """The whole-sequence forward of layers/mvpa.py:280-337 as a differentiable graph: the four
+        projections and c_proj through the library's GEMM (backward: two more GEMMs each), the
+        attention through FlashMVPA (backward: mvpa_backward).  Same kernels as the inference path,
+        launched one by one instead of fused."""
+        from attentions.attn import FlashMVPA
+        from mvpa_hip import autograd as AG
+        bsz, t_len, c_len, e = hidden_states.shape
+        h, hkv, dh, kv = self.num_heads, self.num_kv_heads, self.head_dim, self.embed_kv_dim
+        n = t_len * c_len
+        dt = hidden_states.dtype
+        w_qkv = torch.cat([_weight_of(self.q_attn), _weight_of(self.c_attn)], 0)
+        qkv = AG.linear(hidden_states, w_qkv).reshape(bsz, n, e + 2 * kv)
+        q = qkv[:, :, :e].reshape(bsz, n, h, dh).permute(0, 2, 1, 3)
+        k = qkv[:, :, e:e + kv].reshape(bsz, n, hkv, dh).permute(0, 2, 1, 3)
+        v = qkv[:, :, e + kv:].reshape(bsz, n, hkv, dh).permute(0, 2, 1, 3)
+        k_time = AG.linear(positional_embedding, self.position_net.weight).reshape(t_len, hkv, dh).permute(1, 0, 2)
+        k_chan = AG.linear(channel_embedding, self.channel_net.weight).reshape(c_len, hkv, dh).permute(1, 0, 2)
+        u, vb, z = (b.reshape(hkv, dh).to(dt) for b in self.attn_bias.split(kv, dim=0))
+        chan_valid, key_bias = self._resolve_mask(attention_mask, bsz, t_len, c_len)
+        out = FlashMVPA.apply(q, u, vb, z, k, k_time.contiguous(), k_chan.contiguous(), v, True,
+                              self._scale(), window, True, True, chan_valid, self._content(), key_bias)
+        merged = out.permute(0, 2, 1, 3)                                      # [B,N,H,Dh]
+        if head_mask is not None:                                            # layers/mvpa.py:274-275
+            if head_mask.numel() != h:
+                raise NotImplementedError("head_mask must hold one factor per head")
+            merged = merged * head_mask.to(dt).reshape(1, 1, h, 1)
+        out = AG.linear(merged.reshape(bsz, t_len, c_len, e), self.c_proj.weight)
+        present = None
+        if use_cache is True:
             present = (k.reshape(bsz, hkv, t_len, c_len, dh), v.reshape(bsz, hkv, t_len, c_len, dh))
         return out, present
 
@@ -402,11 +477,7 @@ class MVPFormerGQAAttention(torch.nn.Module):
                 v = torch.cat([past_v.to(dt), v_new.unsqueeze(2)], dim=2)
             k_time, k_chan = self._key_tables(positional_embedding, channel_embedding)
             u, vb, z = (b.view(hkv, dh) for b in self.attn_bias.split(kv, dim=0))
-            chan_valid, key_bias = None, None
-            if attention_mask is not None:
-                chan_valid = self._as_channel_validity(attention_mask, bsz, t_len, c_len)
-                if chan_valid is None:
-                    key_bias = attention_mask.reshape(bsz, t_len * c_len).to(torch.float32)
+            chan_valid, key_bias = self._resolve_mask(attention_mask, bsz, t_len, c_len)
             merged = torch.empty((bsz, c_len, h, dh), dtype=dt, device=hidden_states.device)
             mvpa_hip.mvpa_forward(
                 q, k.reshape(bsz, hkv, t_len * c_len, dh), v.reshape(bsz, hkv, t_len * c_len, dh),

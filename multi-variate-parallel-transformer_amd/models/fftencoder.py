@@ -8,6 +8,7 @@ import torch
 from torch import Tensor, nn
 
 import mvpa_hip
+from mvpa_hip import autograd as AG
 from models import BrainEncoder
 
 
@@ -20,6 +21,8 @@ class RMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(size))
 
     def forward(self, x: Tensor) -> Tensor:
+        if torch.is_grad_enabled() and (x.requires_grad or self.training):
+            return AG.rmsnorm(x, self.weight, self.eps)
         return mvpa_hip.rmsnorm(x, self.weight, self.eps)
 
 
@@ -60,9 +63,24 @@ class WaveEncoder(BrainEncoder):
             self._proj_padded, self._proj_key = buf, key
         return self._proj_padded
 
-    @torch.no_grad()
     def forward(self, x: Tensor) -> Tensor:
-        """x [M, L] -> [M, size_output]; bf16 output (the model's compute dtype)."""
+        """x [M, L] -> [M, size_output]; bf16 output (the model's compute dtype).  In train() mode
+        under grad the norm and the projection are differentiable; the wavelet transform has no
+        parameters and carries no gradient (models/fftencoder.py:80: no_grad)."""
+        if torch.is_grad_enabled() and self.training:
+            return self._forward_autograd(x)
+        with torch.no_grad():
+            return self._forward_fused(x)
+
+    def _forward_autograd(self, x: Tensor) -> Tensor:
+        pad = self._padded_k() - self.dwt_size
+        coeffs = self.block(x)                                                  # fp32, no gradient
+        normed = AG.rmsnorm(coeffs, self.ln.weight, 1e-5, out_dtype=torch.bfloat16)
+        # whole 64-element k-blocks, as on the inference path: the zero columns contribute nothing
+        return AG.linear(torch.nn.functional.pad(normed, (0, pad)),
+                         torch.nn.functional.pad(self.proj.weight.to(torch.bfloat16), (0, pad)))
+
+    def _forward_fused(self, x: Tensor) -> Tensor:
         m = x.shape[0]
         kp = self._padded_k()
         coeffs = mvpa_hip.wavedec_db4(x.float(), pitch=kp, zero_pad=False)   # [M, dwt] view, pitch kp
@@ -72,4 +90,5 @@ class WaveEncoder(BrainEncoder):
         w = self._padded_weight()
         return mvpa_hip.linear(normed, w)          # the zero padding contributes nothing
 
-    encode = forward
+    def encode(self, x: Tensor) -> Tensor:
+        return self.forward(x)

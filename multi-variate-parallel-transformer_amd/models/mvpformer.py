@@ -1,7 +1,14 @@
 """MVPFormer stack on the HIP library: config, parallel block, model, head and the inference
 wrapper, with the reference's class names, constructor arguments and state-dict keys
 (models/mvpformer.py:37-152, 155-402, 405-479, 596-607, 979-989) but without the training
-harness (no Lightning, no HF base classes).  Inference / eval only, bf16 on the GPU.
+harness (no Lightning, no HF base classes).  bf16 on the GPU.
+
+Two paths through every module.  Inference (eval() mode, or under torch.no_grad()): fused
+launches, nothing kept for a backward.  Differentiable (grad mode on and either train() mode or
+an input that carries a graph): the same kernels one product at a time through
+mvpa_hip.autograd and attentions.attn.FlashMVPA, so that gradients reach the input and every
+parameter as they do through models/mvpformer.py:132-147 and layers/mvpa.py:280-337.  Dropout is
+not implemented: the *_pdrop values must be 0 in train() mode.
 """
 from __future__ import annotations
 
@@ -11,7 +18,8 @@ import torch
 from torch import nn
 
 import mvpa_hip
-from layers import (MvpaKVCache, MvpaRingCache, MvpaRingClock, MVPFormerGQAAttention,
+from mvpa_hip import autograd as AG
+from layers import (KeyMask, MvpaKVCache, MvpaRingCache, MvpaRingClock, MVPFormerGQAAttention,
                     MVPFormerGQAFlashAttention)
 from models import BrainDecider, BrainEncoder, BrainModel
 from models.fftencoder import RMSNorm
@@ -93,10 +101,13 @@ class GatedMLP(nn.Module):
             self._gu_key = key
         return self._gu
 
-    @torch.no_grad()
     def forward(self, x):
-        mid = mvpa_hip.linear(x, self._gate_up(), gated=True)
-        return mvpa_hip.linear(mid, self.down_proj.weight.to(torch.bfloat16))
+        if torch.is_grad_enabled() and (x.requires_grad or self.training):
+            mid = torch.nn.functional.silu(AG.linear(x, self.gate_proj.weight)) * AG.linear(x, self.up_proj.weight)
+            return AG.linear(mid, self.down_proj.weight)
+        with torch.no_grad():
+            mid = mvpa_hip.linear(x, self._gate_up(), gated=True)
+            return mvpa_hip.linear(mid, self.down_proj.weight.to(torch.bfloat16))
 
     def gate_up_weight(self) -> torch.Tensor:
         """[gate_proj; up_proj] stacked in bf16, cached until a weight changes."""
@@ -150,6 +161,16 @@ class MVPFormerBlock(nn.Module):
         already has it, `next_norm` the RMSNorm that will consume this block's output (the next
         block's ln_1, or ln_f).  Returns (outputs, next_norm(output) or None); the residual sum and
         that norm come out of one kernel."""
+        if layer_past is None and torch.is_grad_enabled() and (hidden_states.requires_grad or self.training):
+            # differentiable path (models/mvpformer.py:132-147 op by op; both branches read ln_1(x))
+            if normed is None:
+                normed = self.ln_1(hidden_states)
+            attn_outputs = self.attn(normed, positional_embedding, channel_embedding,
+                                     attention_mask=attention_mask, head_mask=head_mask,
+                                     use_cache=use_cache, output_attentions=output_attentions)
+            hidden_states = hidden_states + self.mlp(normed) + attn_outputs[0]
+            outputs = (hidden_states,) + (attn_outputs[1:] if use_cache else attn_outputs[2:])
+            return outputs, (next_norm(hidden_states) if next_norm is not None else None)
         residual = hidden_states
         if normed is None:
             normed = self.ln_1(hidden_states)
@@ -240,9 +261,9 @@ class MVPFormerModel(nn.Module):
         return tuple(MvpaKVCache(batch, self.num_kv_heads, channels, self.head_dim, max_steps,
                                  dtype=dtype, device=device) for _ in self.h)
 
-    @torch.no_grad()
     def forward(self, input_ids=None, past_key_values=None, inputs_embeds=None, attention_mask=None,
-                head_mask=None, use_cache=None, output_attentions=None, position_end=None, **unused):
+                head_mask=None, use_cache=None, output_attentions=None, position_end=None,
+                channel_validity=None, **unused):
         """forward(inputs_embeds=[B,T,C,E]) -> last_hidden_state [B,T,C,E]; with use_cache also the
         per-block `present`s, as the reference returns them in `past_key_values`
         (models/mvpformer.py:290-398).  With past_key_values (one entry per block: the (k, v)
@@ -253,11 +274,25 @@ class MVPFormerModel(nn.Module):
         embedding instead of rows [0, T).  Row j of the T rows in use stands for the distance
         T-1-j between query and key step (layers/mvpa.py:223), so with rows [0, T) the row of a
         given distance moves as a sequence grows; a stream keeps it in place by always ending at
-        the same row (MvpaKVCache entries imply position_end = their max_steps)."""
+        the same row (MvpaKVCache entries imply position_end = their max_steps).
+
+        channel_validity (extension): [B,C], 1 = channel present; stands for an attention_mask that
+        repeats the same 0/1 pattern at every time step, without a look at its values.
+
+        Gradients: with grad mode on and either train() mode or an inputs_embeds that carries a
+        graph, the whole-sequence forward is differentiable (dropout must be 0)."""
         if inputs_embeds is None:
             raise NotImplementedError
-        if self.training:
-            raise NotImplementedError("MVPFormer HIP stack: inference only; call .eval()")
+        if self.training and self.drop.p > 0:
+            raise NotImplementedError("MVPFormer HIP stack: dropout is not implemented; train with "
+                                      "embd_pdrop = 0 or call .eval()")
+        grad = torch.is_grad_enabled() and past_key_values is None and (self.training or inputs_embeds.requires_grad)
+        with torch.set_grad_enabled(grad):
+            return self._forward(past_key_values, inputs_embeds, attention_mask, use_cache, position_end,
+                                 channel_validity)
+
+    def _forward(self, past_key_values, inputs_embeds, attention_mask, use_cache, position_end,
+                 channel_validity):
         use_cache = bool(use_cache)      # None = off whatever config.use_cache says: a tensor comes back
         bsz, t_len, c_len, _ = inputs_embeds.shape
         if past_key_values is not None:
@@ -279,6 +314,14 @@ class MVPFormerModel(nn.Module):
             dt = inputs_embeds.dtype
             attention_mask = attention_mask.view(bsz, -1)[:, None, None, :].to(dtype=dt)
             attention_mask = (1.0 - attention_mask) * torch.finfo(dt).min
+            # analysed once for all blocks (one device synchronisation per forward, none per layer)
+            attention_mask = KeyMask(attention_mask)
+            attention_mask.resolve(bsz, t_len, c_len)
+        elif channel_validity is not None:
+            # extension: the per-channel validity mask [B,C] (1 = present) handed over as such -
+            # what a 0/1 attention_mask that repeats over the time steps amounts to, without the
+            # look at its values, so nothing here synchronises with the device
+            attention_mask = KeyMask(chan_valid=channel_validity.to(torch.bool))
         # ids are arange(T) / arange(C) (models/mvpformer.py:246-261), so the lookups
         # (models/mvpformer.py:282-283) are leading slices of the embedding tables
         if t_len > self.positional_embedding.num_embeddings or c_len > self.channel_embedding.num_embeddings:
@@ -311,10 +354,12 @@ class MVPFormerHead(BrainDecider):
         super().__init__()
         self.head = nn.Linear(size, size_out if size_out is not None else size, bias=False)
 
-    @torch.no_grad()
     def forward(self, x: torch.Tensor):
         if x.is_cuda and x.dtype == torch.bfloat16:
-            return mvpa_hip.linear(x, self.head.weight.to(torch.bfloat16))
+            if torch.is_grad_enabled() and (x.requires_grad or self.training):
+                return AG.linear(x, self.head.weight)
+            with torch.no_grad():
+                return mvpa_hip.linear(x, self.head.weight.to(torch.bfloat16))
         return self.head(x)
 
 
@@ -351,9 +396,16 @@ class HMVPFormer(BrainModel):
         self._load_checkpoint(base_model_sd, head_model_sd)
         return self
 
-    @torch.no_grad()
+    def _grad_mode(self):
+        """Grad mode of the scoring methods: on only in train() mode under an enabled grad mode."""
+        return torch.set_grad_enabled(torch.is_grad_enabled() and self.training)
+
     def _common_forward(self, batch: torch.Tensor, attention_mask=None):
         """batch [B, n_seg, ch, len] -> (last_hidden_state [B,T,C,E], input_embeds [B,T,C,E])."""
+        with self._grad_mode():
+            return self._common_forward_impl(batch, attention_mask)
+
+    def _common_forward_impl(self, batch: torch.Tensor, attention_mask=None):
         bsz, seg_n, ch, seg = batch.shape
         out_enc = self.encoder(batch.reshape(bsz * seg_n * ch, seg))
         input_embeds = out_enc.view(bsz, seg_n, ch, -1)
@@ -452,12 +504,17 @@ class HMVPFormer(BrainModel):
             cache.append(k[:, :, 0], v[:, :, 0])
         return out, caches
 
-    @torch.no_grad()
     def predict_next_segment(self, batch: torch.Tensor):
         """Generative scoring of models/mvpformer.py:749-764: cosine similarity between the head's
         prediction at segment t and the encoding of segment t+1, per channel."""
+        with self._grad_mode():
+            return self._predict_next_segment(batch)
+
+    def _predict_next_segment(self, batch: torch.Tensor):
         out, enc = self._common_forward(batch)
         out = self.head(out)
+        if torch.is_grad_enabled():
+            return torch.cosine_similarity(enc[:, 1:].float(), out[:, :-1].float(), dim=-1)
         if enc.is_cuda and enc.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and enc.shape[-1] % 8 == 0:
             return mvpa_hip.cosine_similarity_steps(enc, out)
         return torch.cosine_similarity(enc[:, 1:].float(), out[:, :-1].float(), dim=-1)
@@ -485,12 +542,12 @@ class HMVPFormer(BrainModel):
         prediction = self.head(out[:, -1])
         return similarity, prediction, (caches, prediction)
 
-    @torch.no_grad()
     def classify(self, batch: torch.Tensor):
         """Classification scoring of models/mvpformer.py:947-953: head(mean over channels of the
         last segment's hidden state)."""
-        out, _ = self._common_forward(batch)
-        return self.head(out[:, -1].float().mean(dim=1).to(out.dtype))
+        with self._grad_mode():
+            out, _ = self._common_forward(batch)
+            return self.head(out[:, -1].float().mean(dim=1).to(out.dtype))
 
 
 def _load_weights(path: str):

@@ -1,0 +1,86 @@
+"""Differentiable wrappers of the library's dense ops, for gradients through the layer and stack
+modules (the reference trains through layers/mvpa.py:280-337 and models/mvpformer.py:132-147).
+
+Forward passes are the library's kernels; backward passes of the products are two more products
+on the same MFMA GEMM (dX = dY W, dW = dY^T X), the norm's backward is a few fp32 tensor ops.
+The attention operator itself is `attentions.attn.FlashMVPA` (mvpa_backward kernels).
+"""
+from __future__ import annotations
+
+import torch
+
+import mvpa_hip
+
+
+def wants_grad(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+def _k8(t: torch.Tensor) -> torch.Tensor:
+    """[rows, K] contiguous with K padded by zero columns to a multiple of 8 (the GEMM fetches rows
+    in 16-byte chunks); zero columns add nothing to a product."""
+    pad = (-t.shape[-1]) % 8
+    t = torch.nn.functional.pad(t, (0, pad)) if pad else t
+    return t.contiguous()
+
+
+class _LinearFn(torch.autograd.Function):
+    """y = x @ w^T, bf16 on the GPU library, any leading shape of x."""
+
+    @staticmethod
+    def forward(ctx, x, w):
+        ctx.save_for_backward(x, w)
+        return mvpa_hip.linear(x, w)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w = ctx.saved_tensors
+        k = x.shape[-1]
+        dy2 = dy.reshape(-1, dy.shape[-1]).contiguous()
+        dx = dw = None
+        if ctx.needs_input_grad[0]:
+            dx = mvpa_hip.linear(_k8(dy2), _k8(w.t())).view(x.shape)              # [M,N] @ [N,K]
+        if ctx.needs_input_grad[1]:
+            x2 = x.reshape(-1, k)
+            dw = mvpa_hip.linear(_k8(dy2.t()), _k8(x2.t()))                       # [N,M] @ [M,K]
+        return dx, dw
+
+
+def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """x @ w^T.  bf16 GPU tensors go through the library (differentiably when a gradient is
+    wanted); anything else is torch's own linear."""
+    if x.is_cuda and x.dtype == torch.bfloat16:
+        w = w.to(torch.bfloat16)
+        if wants_grad(x, w):
+            return _LinearFn.apply(x, w)
+        return mvpa_hip.linear(x, w.detach())
+    return torch.nn.functional.linear(x, w.to(x.dtype))
+
+
+class _RMSNormFn(torch.autograd.Function):
+    """y = x * rsqrt(mean(x^2) + eps) * w; forward on the library's kernel, backward in fp32."""
+
+    @staticmethod
+    def forward(ctx, x, w, eps, out_dtype):
+        ctx.save_for_backward(x, w)
+        ctx.eps = eps
+        return mvpa_hip.rmsnorm(x, w, eps, out_dtype=out_dtype)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w = ctx.saved_tensors
+        xf, wf, g = x.float(), w.float(), dy.float()
+        r = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + ctx.eps)
+        gw = g * wf
+        dx = dw = None
+        if ctx.needs_input_grad[0]:
+            dx = (r * gw - xf * r.pow(3) * (xf * gw).mean(-1, keepdim=True)).to(x.dtype)
+        if ctx.needs_input_grad[1]:
+            dw = (g * xf * r).reshape(-1, x.shape[-1]).sum(0).to(w.dtype)
+        return dx, dw, None, None
+
+
+def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype=None) -> torch.Tensor:
+    if wants_grad(x, w):
+        return _RMSNormFn.apply(x, w, eps, out_dtype)
+    return mvpa_hip.rmsnorm(x, w, eps, out_dtype=out_dtype)
