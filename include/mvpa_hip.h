@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define MVPA_ABI_VERSION 2
+#define MVPA_ABI_VERSION 3
 
 /* ---- status codes ---------------------------------------------------------------- */
 enum {
@@ -144,6 +144,12 @@ typedef struct mvpa_fwd_args {
   int32_t n_split;           /* 0 or 1 = no split; at most T                              */
   int32_t reserved0;
   const int32_t* ring_head;  /* MVPA_FLAG_RING: device pointer to the newest slot, in [0, T)  */
+  const void* k_fp8;         /* nullable, MVPA_FLAG_FP8_QK: the keys already rounded to e4m3,
+                                k / fp8_k_scale[g], contiguous [B,Hkv,N,Dh] bytes, 16-byte aligned
+                                (mvpa_fp8_prepare writes it).  The column-split build
+                                (MVPA_KERNEL_MFMA_SPLIT) streams these rows for its window steps
+                                and needs them for the fp8 content term; the general kernel rounds
+                                the bf16 keys itself and ignores the field.                      */
 } mvpa_fwd_args;
 
 /* ABI version of the loaded library. */
@@ -155,6 +161,17 @@ const char* mvpa_error_string(int status);
 /* Host-only check of an argument block; touches no device memory and needs no GPU.
  * Mirrors the asserts of attentions/attn.py:1041-1045, 1339, 1344. */
 int mvpa_validate(const mvpa_fwd_args* args);
+
+/* What MVPA_FLAG_FP8_QK needs besides the tensors themselves, from q, k, bias_u, sm_scale, the
+ * shapes and the strides of an argument block (its fp8_* and k_fp8 fields are not read):
+ *   q_scale[h] = max |q + u| over the head's rows * sm_scale * log2(e) / 224   (>= 1e-20)
+ *   k_scale[g] = max |k| over the kv head's rows / 224                          (>= 1e-20)
+ *   k_fp8      = e4m3(k / k_scale[g]), contiguous [B,Hkv,N,Dh] bytes (nullable: scales only)
+ * 224 keeps the largest magnitude inside the range of either e4m3 flavour.  With
+ * MVPA_FLAG_LAST_STEP q holds C rows per head.  bf16 tensors; a handful of small launches on
+ * `stream`, no allocation.  The reference has no fp8 path (attentions/attn.py:1064-1066 takes
+ * fp16 or bf16). */
+int mvpa_fp8_prepare(const mvpa_fwd_args* args, float* q_scale, float* k_scale, void* k_fp8, void* stream);
 
 /* Bytes of mvpa_fwd_args.split_ws for args->n_split runs: n_split * B * H * C partial output
  * rows of Dh bf16 values followed by as many float log-sum-exps.  0 if n_split <= 1. */

@@ -131,6 +131,27 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
     k_off[i] = (uint32_t)(rowc * a.k_stride_n) * 2u + ((phys ^ swz_k<DH>(row)) << 4);
     v_off[i] = (uint32_t)(rowc * a.v_stride_n) * 2u + ((phys ^ swz_v<DH>(row)) << 4);
   }
+  // fp8 content term: the window steps stream the e4m3 copy of the keys (a.k_fp8, one byte per
+  // element, contiguous [B,Hkv,N,DH]) into the K slot instead of the bf16 rows: rows of DH bytes
+  // in natural [key][dh] order, 16-byte chunks XOR-swizzled so that 8 lanes reading the same
+  // logical chunk of 8 consecutive rows cover all banks.  A key tile is K8_LOADS loads of 64 x 16
+  // bytes; with fewer of them than waves some waves fetch a chunk a second time (same bytes to
+  // the same place), so that every wave issues the same number of loads.
+  constexpr int K8_CHUNKS = DH / 16, K8_LOADS = G::CP * DH / 1024, LPW8 = (K8_LOADS + NW - 1) / NW;
+  auto swz8 = [](int row) -> int { return DH == 128 ? (row & 7) : ((row >> 1) & 3); };
+  uint32_t k8_off[LPW8], k8_dst[LPW8];
+  if (FP8) {
+#pragma unroll
+    for (int i = 0; i < LPW8; ++i) {
+      const int ld = (wave + NW * i) % K8_LOADS;
+      const int pc = ld * 64 + lane;
+      const int row = pc / K8_CHUNKS, phys = pc % K8_CHUNKS;
+      k8_off[i] = (uint32_t)(min(row, C_ - 1) * DH) + ((phys ^ swz8(row)) << 4);
+      k8_dst[i] = ld * 1024;
+    }
+  }
+  const unsigned char* k8base = FP8 ? (const unsigned char*)a.k_fp8 + ((int64_t)b * a.Hkv + g) * ((int64_t)T_ * C_ * DH) : nullptr;
+  const int64_t k8step = (int64_t)C_ * DH;
   const uint32_t ring_lds = (uint32_t)(uintptr_t)(LDS_PTR(unsigned char))smem_raw;
   // Tiles are requested in stream order - window steps NLO .. tq (K and V), then far steps
   // 0 .. far_max (V only) - whenever the slots they need are free.  `used` counts the slots of
@@ -139,16 +160,23 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
   int iss_pos = 0, iss_slot = 0, used = 0, issued = 0;
   const bf16_t* iss_k = kbase + (n_near > 0 ? NLO : 0) * kstep;
   const bf16_t* iss_v = vbase + (n_near > 0 ? NLO : 0) * vstep;
+  const unsigned char* iss_k8 = FP8 ? k8base + (n_near > 0 ? NLO : 0) * k8step : nullptr;
   auto issue_avail = [&]() {
     while (iss_pos < n_near) {
       const bool is_near = true;
       if (used + (is_near ? 2 : 1) > SLOTS) break;
       uint32_t slot = ring_lds + iss_slot * TILE_BYTES;
       if (is_near) {
+        if (FP8) {
 #pragma unroll
-        for (int i = 0; i < LPW; ++i) load_to_lds_16(iss_k, k_off[i], slot + (wave + NW * i) * 1024);
+          for (int i = 0; i < LPW8; ++i) load_to_lds_16(iss_k8, k8_off[i], slot + k8_dst[i]);
+          iss_k8 += k8step;
+        } else {
+#pragma unroll
+          for (int i = 0; i < LPW; ++i) load_to_lds_16(iss_k, k_off[i], slot + (wave + NW * i) * 1024);
+          iss_k += kstep;
+        }
         slot += TILE_BYTES;
-        iss_k += kstep;
       }
 #pragma unroll
       for (int i = 0; i < LPW; ++i) load_to_lds_16(iss_v, v_off[i], slot + (wave + NW * i) * 1024);
@@ -176,6 +204,13 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) k_lane[ks] = ln * ROWB + (((2 * ks + hh) ^ swz_k<DH>(ln)) << 4);
+    // fp8 keys: one 16-byte read serves two products.  Read p of a lane covers the head
+    // dimensions [(2p + hh) * 16, +16) of its key row: the low 8 bytes go to product 2p, the high
+    // 8 to product 2p + 1 (the query fragments are laid out to match).
+    if (FP8) {
+#pragma unroll
+      for (int p2 = 0; p2 < KS / 2; ++p2) k_lane[p2] = ln * DH + (((2 * p2 + hh) ^ swz8(ln)) << 4);
+    }
   }
   // Fragment addresses of a step: one register per output tile (V^T) / k-step (K) = lane part +
   // slot, formed once per step and made opaque to the compiler, so that everything else of an
@@ -247,15 +282,21 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
   // fp8 content term (FP8): q' = (q+u)*scale/sq and k' = k/sk are rounded to e4m3 with the
   // per-head amax scales sq, sk chosen by the caller; the MFMA accumulates in units of 1/(sq*sk),
   // the channel-bias tile is pre-divided accordingly for the window steps and the product sq*sk
-  // returns inside the exp2 fma.  K is converted on the fly from the bf16 tile.
+  // returns inside the exp2 fma.  K arrives rounded (a.k_fp8).
   f32x16 Bc[NCT];
   bf16x8 Qu[KS];
   long Qu8[KS];
-  float fp8_d = 1.f, fp8_inv_sk = 1.f;
+  float fp8_d = 1.f;
   if (FP8) {
     const float sq = a.fp8_q_scale[h], sk = a.fp8_k_scale[g];
     fp8_d = sq * sk;
-    fp8_inv_sk = 1.f / sk;
+    // product s = 2p + j contracts, in lane half hh, the head dimensions [(2p + hh) * 16 + 8j, +8)
+#pragma unroll
+    for (int s8 = 0; s8 < KS; ++s8) {
+      const int d0 = ((s8 >> 1) * 2 + hh) * 16 + (s8 & 1) * 8;
+      const u32x4 raw = *(const u32x4*)(qbase + (qoff - hh * 16) + d0 * 2);
+      Qu8[s8] = make_qfrag_fp8(raw, bu + d0, sc2 / sq);
+    }
   }
   {
     f32x16 sct[NCT];
@@ -272,8 +313,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
       for (int k4 = 0; k4 < 4; ++k4) {
         const int ks = kh + k4;
         const int d0 = ks * 16 + hh * 8;
-        if (FP8) Qu8[ks] = make_qfrag_fp8(raw[k4], bu + d0, sc2 / a.fp8_q_scale[h]);
-        else Qu[ks] = make_qfrag(raw[k4], bu + d0, sc2);
+        if (!FP8) Qu[ks] = make_qfrag(raw[k4], bu + d0, sc2);
         const bf16x8 qz = make_qfrag(raw[k4], bz + d0, sc2);
 #pragma unroll
         for (int t = 0; t < NCT; ++t) {
@@ -385,12 +425,16 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
     for (int t = 0; t < NCT; ++t) {
       f32x16 S = Bc[t];
       if (FP8) {
-        u32x4 kr[KS];
+        u32x4 kr[KS / 2];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) kr[ks] = *(LDS_PTR(const u32x4))(uintptr_t)(ka_.k[ks] + t * 32 * ROWB);
+        for (int p2 = 0; p2 < KS / 2; ++p2) kr[p2] = *(LDS_PTR(const u32x4))(uintptr_t)(ka_.k[p2] + t * 32 * DH);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-          S = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(kfrag_fp8(kr[ks], fp8_inv_sk), Qu8[ks], S, 0, 0, 0);
+        for (int p2 = 0; p2 < KS / 2; ++p2) {
+          const long lo = (long)(((unsigned long)kr[p2][1] << 32) | kr[p2][0]);
+          const long hi = (long)(((unsigned long)kr[p2][3] << 32) | kr[p2][2]);
+          S = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(lo, Qu8[2 * p2], S, 0, 0, 0);
+          S = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(hi, Qu8[2 * p2 + 1], S, 0, 0, 0);
+        }
       } else {
         bf16x8 ka[KS];
 #pragma unroll
@@ -445,7 +489,8 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
   for (int p = 0; p < n_near; ++p) {
     const int tk = NLO + p;
     need += 2;
-    wait_units<LPW>(issued - need);
+    if (FP8) wait_units<LPW + LPW8>((issued - need) / 2);     // (a window tile is LPW8 + LPW loads)
+    else wait_units<LPW>(issued - need);
     lds_barrier();
     used -= prev_slots;          // the previous tile is consumed by every wave
     prev_slots = 2;
@@ -631,6 +676,8 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
 int mvpa_mfma128_supported(const mvpa_fwd_args* a) {
   if ((a->Dh != 128 && a->Dh != 64) || a->C <= 32 || a->C > 128) return 0;
   if (a->flags & (MVPA_FLAG_LAST_STEP | MVPA_FLAG_RING)) return 0;
+  // the fp8 content term streams the keys' e4m3 copy (the general kernel rounds bf16 keys itself)
+  if ((a->flags & MVPA_FLAG_FP8_QK) && (!a->k_fp8 || ((uintptr_t)a->k_fp8 & 15))) return 0;
   return 1;
 }
 

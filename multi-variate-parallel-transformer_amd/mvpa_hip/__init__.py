@@ -44,7 +44,7 @@ class MvpaFwdArgs(ctypes.Structure):
         ("lse", ctypes.c_void_p),
         ("fp8_q_scale", ctypes.c_void_p), ("fp8_k_scale", ctypes.c_void_p),
         ("split_ws", ctypes.c_void_p), ("n_split", ctypes.c_int32), ("reserved0", ctypes.c_int32),
-        ("ring_head", ctypes.c_void_p),
+        ("ring_head", ctypes.c_void_p), ("k_fp8", ctypes.c_void_p),
     ]
 
 
@@ -110,6 +110,8 @@ def load_library() -> ctypes.CDLL:
     lib.mvpa_static_ws_init.argtypes = []
     lib.mvpa_backward.restype = ctypes.c_int
     lib.mvpa_backward.argtypes = [ctypes.POINTER(MvpaBwdArgs), vp]
+    lib.mvpa_fp8_prepare.restype = ctypes.c_int
+    lib.mvpa_fp8_prepare.argtypes = [ctypes.POINTER(MvpaFwdArgs), vp, vp, vp, vp]
     lib.mvpa_debug_block_order.restype = ctypes.c_int
     lib.mvpa_debug_block_order.argtypes = [i32, i32, i32, vp, vp]
     lib.mvpa_debug_maps.restype = ctypes.c_int
@@ -130,7 +132,7 @@ def load_library() -> ctypes.CDLL:
     lib.mvpa_add3_rmsnorm_bf16.argtypes = [vp, vp, vp, vp, vp, vp, i64, i32, f32, vp]
     lib.mvpa_wavedec_db4.restype = ctypes.c_int
     lib.mvpa_wavedec_db4.argtypes = [vp, vp, i64, i32, i32, i32, i64, vp]
-    if lib.mvpa_version() != 2:
+    if lib.mvpa_version() != 3:
         raise RuntimeError("libmvpa_hip ABI version mismatch")
     _lib = lib
     return lib
@@ -182,7 +184,7 @@ def make_args(q, k, v, out, u, vb, z, k_time, k_chan, *, T: int, C: int,
               sm_scale: float, window: int = 10, flags: int = 15,
               chan_valid=None, key_bias=None, lse=None, kernel: int = KERNEL_AUTO,
               fp8_q_scale=None, fp8_k_scale=None, split_ws=None, n_split: int = 0,
-              ring_head=None) -> MvpaFwdArgs:
+              ring_head=None, k_fp8=None) -> MvpaFwdArgs:
     """Fill the argument block from [B,H,N,Dh]-indexable tensors (any strides with a unit
     last stride).  Accepts meta/CPU tensors too so validation can be exercised without a GPU."""
     a = MvpaFwdArgs()
@@ -212,6 +214,7 @@ def make_args(q, k, v, out, u, vb, z, k_time, k_chan, *, T: int, C: int,
     a.split_ws = split_ws.data_ptr() if split_ws is not None else None
     a.n_split = n_split
     a.ring_head = ring_head.data_ptr() if ring_head is not None else None
+    a.k_fp8 = k_fp8.data_ptr() if k_fp8 is not None else None
     return a
 
 
@@ -285,17 +288,21 @@ def mvpa_forward(q, k, v, u, vb, z, k_time, k_chan, *, sm_scale: Optional[float]
         if ring_head.dtype != torch.int32 or not ring_head.is_cuda or ring_head.numel() != 1:
             raise TypeError("ring_head: one int32 element on the GPU")
     s = (1.0 / Dh ** 0.5) if sm_scale is None else float(sm_scale)
-    q_scale = k_scale = None
+    q_scale = k_scale = k8 = None
     if fp8_qk:
-        # per-head amax scales: the kernel rounds (q+u)*s*log2(e)/q_scale and k/k_scale to e4m3;
-        # 224 keeps the largest magnitude inside the range of either e4m3 flavour
-        grp = H // k.shape[1]
-        qf = q.float() + u.float().repeat_interleave(grp, 0)[None, :, None, :]
-        q_scale = (qf.abs().amax(dim=(0, 2, 3)) * (s * 1.4426950408889634 / 224.0)).clamp_min(1e-20).contiguous()
-        k_scale = (k.float().abs().amax(dim=(0, 2, 3)) / 224.0).clamp_min(1e-20).contiguous()
+        # per-head amax scales and the e4m3 copy of the keys, by the library (mvpa_fp8_prepare):
+        # the kernel rounds (q+u)*s*log2(e)/q_scale to e4m3 itself and multiplies it with k/k_scale
+        q_scale = torch.empty(H, dtype=torch.float32, device=q.device)
+        k_scale = torch.empty(k.shape[1], dtype=torch.float32, device=q.device)
+        if not last_step_only and 32 < C <= 128 and Dh in (64, 128):      # shapes of the column-split build
+            k8 = torch.empty((B, k.shape[1], N, Dh), dtype=torch.uint8, device=q.device)
+        pa = make_args(q, k, v, out, u, vb, z, k_time, k_chan, T=T, C=C, sm_scale=s, window=window,
+                       flags=flags)
+        _check(lib.mvpa_fp8_prepare(ctypes.byref(pa), q_scale.data_ptr(), k_scale.data_ptr(),
+                                    k8.data_ptr() if k8 is not None else None, _stream()))
     a = make_args(q, k, v, out, u, vb, z, k_time, k_chan, T=T, C=C, sm_scale=s, window=window,
                   flags=flags, chan_valid=chan_valid, key_bias=key_bias, lse=lse, kernel=kernel,
-                  fp8_q_scale=q_scale, fp8_k_scale=k_scale, ring_head=ring_head)
+                  fp8_q_scale=q_scale, fp8_k_scale=k_scale, ring_head=ring_head, k_fp8=k8)
     if last_step_only and lib.mvpa_select_kernel(ctypes.byref(a)) == KERNEL_MFMA:
         n = default_key_splits(B, H, T) if key_splits is None else int(key_splits)
         if n > 1:

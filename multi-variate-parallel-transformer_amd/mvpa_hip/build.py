@@ -13,7 +13,7 @@ INCLUDE = os.path.join(os.path.dirname(PKG), "include")
 LIB = os.path.join(HERE, "libmvpa_hip.so")
 
 SOURCES = ["mvpa_api.hip", "mvpa_generic.hip", "mvpa_mfma.hip", "mvpa_mfma64.hip", "mvpa_mfma128.hip", "mvpa_dense.hip", "mvpa_backward.hip",
-           "mvpa_backward_mfma.hip", "mvpa_static_ws.hip"]
+           "mvpa_backward_mfma.hip", "mvpa_static_ws.hip", "mvpa_fp8.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming packed fp32 VALU instructions.
 FLAGS = [

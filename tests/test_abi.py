@@ -24,7 +24,7 @@ def test_exports_every_declared_symbol(lib):
     assert "mvpa_forward" in names and "mvpa_linear_bf16" in names
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/mvpa_hip.h but not exported"
-    assert lib.mvpa_version() == 2
+    assert lib.mvpa_version() == 3
 
 
 def _args(B=2, H=4, Hkv=4, T=4, C=3, Dh=32, dtype=torch.float32, **kw):

@@ -767,6 +767,43 @@ def test_fp8_qk_on_the_column_split_build(cfg):
     assert ((o8 - og8) * live).abs().max().item() <= 2e-2
 
 
+@pytest.mark.parametrize("cfg", [dict(B=2, C=40, T=9, H=4, Hkv=2, Dh=64), dict(B=1, C=128, T=5, H=2, Hkv=1, Dh=128)])
+def test_fp8_prepare_scales_and_rounded_keys(cfg):
+    """mvpa_fp8_prepare: the per-head scales are max|q+u| * s*log2(e)/224 and max|k| / 224, and the
+    e4m3 copy of the keys is k * (1/k_scale) rounded to nearest even, byte for byte what torch's
+    float8_e4m3fn conversion gives - on strided views of a fused projection, as the layer passes
+    them."""
+    import ctypes
+    lib = mvpa_hip.load_library()
+    B, C, T, H, Hkv, Dh = (cfg[k] for k in ("B", "C", "T", "H", "Hkv", "Dh"))
+    N = T * C
+    torch.manual_seed(17)
+    qkv = (torch.randn(B, N, (H + 2 * Hkv) * Dh, device="cuda") * 1.7).to(torch.bfloat16)
+    q = qkv[:, :, :H * Dh].view(B, N, H, Dh).permute(0, 2, 1, 3)
+    k = qkv[:, :, H * Dh:(H + Hkv) * Dh].view(B, N, Hkv, Dh).permute(0, 2, 1, 3)
+    v = qkv[:, :, (H + Hkv) * Dh:].view(B, N, Hkv, Dh).permute(0, 2, 1, 3)
+    u = (torch.randn(Hkv, Dh, device="cuda") * 0.5).to(torch.bfloat16)
+    tab = torch.zeros(Hkv, max(T, C), Dh, dtype=torch.bfloat16, device="cuda")
+    out = torch.empty((B, H, N, Dh), dtype=torch.bfloat16, device="cuda")
+    s = Dh ** -0.5
+    a = mvpa_hip.make_args(q, k, v, out, u, u, u, tab, tab, T=T, C=C, sm_scale=s)
+    qs = torch.empty(H, dtype=torch.float32, device="cuda")
+    ks = torch.empty(Hkv, dtype=torch.float32, device="cuda")
+    k8 = torch.zeros((B, Hkv, N, Dh), dtype=torch.uint8, device="cuda")
+    assert lib.mvpa_fp8_prepare(ctypes.byref(a), qs.data_ptr(), ks.data_ptr(), k8.data_ptr(),
+                                torch.cuda.current_stream().cuda_stream) == 0
+    qf = q.float() + u.float().repeat_interleave(H // Hkv, 0)[None, :, None, :]
+    want_q = qf.abs().amax(dim=(0, 2, 3)) * torch.tensor(a.sm_scale * 1.4426950408889634 / 224.0, dtype=torch.float64).float().cuda()
+    want_k = k.float().abs().amax(dim=(0, 2, 3)) / 224.0
+    assert torch.allclose(qs, want_q, rtol=2e-7, atol=0) and torch.equal(ks, want_k)
+    want8 = (k.float() * (1.0 / ks)[None, :, None, None]).to(torch.float8_e4m3fn).view(torch.uint8)
+    assert torch.equal(k8, want8)
+    # scales only
+    assert lib.mvpa_fp8_prepare(ctypes.byref(a), qs.data_ptr(), ks.data_ptr(), None,
+                                torch.cuda.current_stream().cuda_stream) == 0
+    assert torch.equal(ks, want_k)
+
+
 def test_fp8_needs_mfma_kernel():
     inp = make_mvpa_inputs(B=1, C=4, T=6, H=1, Dh=32, seed=1)
     d = inp.to("cuda", torch.float32)
