@@ -302,6 +302,12 @@ int mvpa_linear_bf16_residual(const void* x, const void* w, const void* r, void*
                               int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldr,
                               int64_t ldy, void* stream);
 
+/* The same product in fp32 (fp32 in and out, fp32 MFMA): the projections of the fp32 layer path
+ * (layers/mvpa.py:303-313, 336 on fp32 tensors - the small plumbing configuration).  Any positive
+ * M, N, K; row strides in elements. */
+int mvpa_linear_f32(const float* x, const float* w, float* y, int64_t M, int64_t N, int64_t K,
+                    int64_t ldx, int64_t ldw, int64_t ldy, void* stream);
+
 /* Two products on one x in one launch: y0[M,N0] = x @ w0^T and y1[M,N1] = silu(x @ wg^T) * (x @ wu^T)
  * with w1 holding the gate rows [0,N1) and the up rows [N1,2*N1) - the fused q/kv projection
  * (layers/mvpa.py:354-356) and the MLP's gate/up product (models/mvpformer.py:146), which both read

@@ -1397,6 +1397,50 @@ __global__ __launch_bounds__(256) void ring_append_bf16_kernel(
   *(u32x4*)(v_ring + dst) = *(const u32x4*)(v_new + src);
 }
 
+// -----------------------------------------------------------------------------------------
+// y[M,N] = x[M,K] w[N,K]^T in fp32 (v_mfma_f32_32x32x2_f32): the projections of the fp32 layer
+// path (the small fp32 configuration: plumbing and golden outputs), so that they too run in this
+// library.  64 x 64 tile, 4 waves of one 32 x 32 block each, 32-wide k-blocks staged in LDS
+// (rows padded by one float against bank conflicts).  Any M, N, K.
+// -----------------------------------------------------------------------------------------
+constexpr int F32_BK = 32, F32_PITCH = F32_BK + 1;
+
+__global__ __launch_bounds__(256) void linear_f32_kernel(const float* __restrict__ X, const float* __restrict__ W,
+                                                         float* __restrict__ Y, int64_t M, int64_t N, int64_t K,
+                                                         int64_t ldx, int64_t ldw, int64_t ldy) {
+  __shared__ float xs[64 * F32_PITCH], ws[64 * F32_PITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int ln = lane & 31, hh = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int64_t m0 = (int64_t)blockIdx.y * 64, n0 = (int64_t)blockIdx.x * 64;
+  f32x16 acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+  for (int64_t k0 = 0; k0 < K; k0 += F32_BK) {
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int e = it * 256 + tid, r = e / F32_BK, c = e % F32_BK;
+      const int64_t k = k0 + c;
+      xs[r * F32_PITCH + c] = (m0 + r < M && k < K) ? X[(m0 + r) * ldx + k] : 0.f;
+      ws[r * F32_PITCH + c] = (n0 + r < N && k < K) ? W[(n0 + r) * ldw + k] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s2 = 0; s2 < F32_BK / 2; ++s2) {
+      const float av = xs[(wm * 32 + ln) * F32_PITCH + 2 * s2 + hh];
+      const float bv = ws[(wn * 32 + ln) * F32_PITCH + 2 * s2 + hh];
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0);
+    }
+  }
+  const int64_t n = n0 + wn * 32 + ln;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int64_t m = m0 + wm * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
+    if (m < M && n < N) Y[m * ldy + n] = acc[i];
+  }
+}
+
 }  // namespace mvpa
 
 using namespace mvpa;
@@ -1523,6 +1567,15 @@ extern "C" int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M
 // y0 = x w0^T and y1 = silu(x wg^T) * (x wu^T) in one launch (w1 holds the gate rows [0, N1) and
 // the up rows [N1, 2 N1)): the two products that read ln_1(x) in the parallel block.  Large
 // shapes only: at least 512 rows, K a multiple of 64; MVPA_ERR_UNSUPPORTED otherwise.
+extern "C" int mvpa_linear_f32(const float* x, const float* w, float* y, int64_t M, int64_t N, int64_t K,
+                               int64_t ldx, int64_t ldw, int64_t ldy, void* stream) {
+  if (!x || !w || !y) return MVPA_ERR_NULL;
+  if (M <= 0 || N <= 0 || K <= 0 || ldx < K || ldw < K || ldy < N) return MVPA_ERR_SHAPE;
+  MVPA_LAUNCH(mvpa::linear_f32_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64)), dim3(256), 0,
+              (hipStream_t)stream, x, w, y, M, N, K, ldx, ldw, ldy);
+  return mvpa::take_launch_status();
+}
+
 extern "C" int mvpa_linear_bf16_dual(const void* x, const void* w0, void* y0, const void* w1, void* y1,
                                      int64_t M, int64_t N0, int64_t N1, int64_t K, int64_t ldx,
                                      int64_t ldw0, int64_t ldy0, int64_t ldw1, int64_t ldy1, void* stream) {

@@ -191,9 +191,11 @@ def _weight_of(mod) -> torch.Tensor:
 
 
 def _linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """bf16 on the GPU goes through the library's MFMA GEMM; fp32 uses the BLAS GEMM."""
+    """GPU tensors go through the library's MFMA GEMMs, bf16 or fp32."""
     if x.is_cuda and x.dtype == torch.bfloat16:
         return mvpa_hip.linear(x, w.to(torch.bfloat16))
+    if x.is_cuda and x.dtype == torch.float32:
+        return mvpa_hip.linear_f32(x, w.to(torch.float32))
     return torch.nn.functional.linear(x, w.to(x.dtype))
 
 

@@ -110,6 +110,8 @@ def load_library() -> ctypes.CDLL:
     lib.mvpa_static_ws_init.argtypes = []
     lib.mvpa_backward.restype = ctypes.c_int
     lib.mvpa_backward.argtypes = [ctypes.POINTER(MvpaBwdArgs), vp]
+    lib.mvpa_linear_f32.restype = ctypes.c_int
+    lib.mvpa_linear_f32.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, vp]
     lib.mvpa_fp8_prepare.restype = ctypes.c_int
     lib.mvpa_fp8_prepare.argtypes = [ctypes.POINTER(MvpaFwdArgs), vp, vp, vp, vp]
     lib.mvpa_debug_block_order.restype = ctypes.c_int
@@ -501,6 +503,25 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = 
                                 x2.stride(0), weight.stride(0), out.stride(0),
                                 1 if gated else 0, _stream()))
     return out if given else out.view(*x.shape[:-1], N)
+
+
+def linear_f32(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """y = x @ weight.T in fp32 on the GPU library (x: any leading shape, K last)."""
+    lib = load_library()
+    _need_cuda(x, weight)
+    if x.dtype != torch.float32 or weight.dtype != torch.float32:
+        raise TypeError("linear_f32: fp32 only")
+    K = x.shape[-1]
+    x2 = x.reshape(-1, K)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    w = weight if weight.stride(-1) == 1 else weight.contiguous()
+    assert w.shape[1] == K
+    M, N = x2.shape[0], w.shape[0]
+    out = torch.empty((M, N), dtype=torch.float32, device=x.device)
+    _check(lib.mvpa_linear_f32(x2.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, x2.stride(0),
+                               w.stride(0), out.stride(0), _stream()))
+    return out.view(*x.shape[:-1], N)
 
 
 def cosine_similarity_steps(nxt: torch.Tensor, pred: torch.Tensor, eps: float = 1e-8) -> torch.Tensor:

@@ -46,14 +46,39 @@ class _LinearFn(torch.autograd.Function):
         return dx, dw
 
 
+class _LinearF32Fn(torch.autograd.Function):
+    """The same in fp32 (the library's fp32 MFMA product, forward and both backward products)."""
+
+    @staticmethod
+    def forward(ctx, x, w):
+        ctx.save_for_backward(x, w)
+        return mvpa_hip.linear_f32(x, w)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w = ctx.saved_tensors
+        dy2 = dy.reshape(-1, dy.shape[-1]).contiguous()
+        dx = dw = None
+        if ctx.needs_input_grad[0]:
+            dx = mvpa_hip.linear_f32(dy2, w.t().contiguous()).view(x.shape)
+        if ctx.needs_input_grad[1]:
+            dw = mvpa_hip.linear_f32(dy2.t().contiguous(), x.reshape(-1, x.shape[-1]).t().contiguous())
+        return dx, dw
+
+
 def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """x @ w^T.  bf16 GPU tensors go through the library (differentiably when a gradient is
-    wanted); anything else is torch's own linear."""
+    """x @ w^T on the GPU library, bf16 or fp32 (differentiably when a gradient is wanted);
+    tensors that are not on the GPU take torch's own linear."""
     if x.is_cuda and x.dtype == torch.bfloat16:
         w = w.to(torch.bfloat16)
         if wants_grad(x, w):
             return _LinearFn.apply(x, w)
         return mvpa_hip.linear(x, w.detach())
+    if x.is_cuda and x.dtype == torch.float32:
+        w = w.to(torch.float32)
+        if wants_grad(x, w):
+            return _LinearF32Fn.apply(x, w)
+        return mvpa_hip.linear_f32(x, w.detach())
     return torch.nn.functional.linear(x, w.to(x.dtype))
 
 

@@ -228,3 +228,18 @@ def test_linear_split_k_pair(M, N, K, gated):
     tol = (2 ** -7 if gated else 2 ** -8) * ref.abs().max().item() + 1e-5
     assert (y.double() - ref).abs().max().item() <= tol
     assert (y - y1).abs().max().item() <= 2 * tol
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 128, 128), (70, 33, 50), (1, 5, 3), (513, 96, 129)])
+def test_linear_f32_matches_float64_product(M, N, K):
+    """The fp32 product of the fp32 layer path (fp32 MFMA, fp32 accumulation) against a float64
+    matrix product: max-abs error <= 1e-5 on unit-scale operands, any M, N, K, row-pitched x."""
+    torch.manual_seed(M + N)
+    xw = torch.randn(M, K + 3, device="cuda")
+    x = xw[:, :K]                                   # a row-pitched view
+    w = torch.randn(N, K, device="cuda") / K ** 0.5
+    y = mvpa_hip.linear_f32(x, w)
+    ref = (x.double() @ w.double().t())
+    assert y.shape == (M, N) and (y.double() - ref).abs().max().item() <= 1e-5
+    y3 = mvpa_hip.linear_f32(x.reshape(1, M, K), w)
+    assert y3.shape == (1, M, N) and torch.equal(y3[0], y)
