@@ -318,6 +318,32 @@ int mvpa_linear_bf16_dual(const void* x, const void* w0, void* y0, const void* w
                           int64_t N0, int64_t N1, int64_t K, int64_t ldx, int64_t ldw0, int64_t ldy0,
                           int64_t ldw1, int64_t ldy1, void* stream);
 
+/* RMSNorm between two products without a pass of its own (models/mvpformer.py:133: ln_1 in front
+ * of the block's projections; :146-147: its input is the sum the previous block's tail product
+ * wrote).  The producer writes, beside its rows, their partial sums of squares; the consumer reads
+ * the RAW rows, multiplies them with weights whose columns already carry the norm's weight
+ * (w[n][k] * ln[k], folded by the caller), and scales every output row by
+ * rsqrt(sum of the row's partial sums / K + eps) while it converts it - before the SiLU gate.
+ *   mvpa_linear_sumsq_parts(M, N)      host-only: partial sums per row that the residual product
+ *                                      writes for an [M, N] output (two per column tile)
+ *   mvpa_linear_bf16_residual_sumsq    mvpa_linear_bf16_residual that also writes
+ *                                      sumsq[M][parts] (fp32; sums over the final bf16 values);
+ *                                      pair-kernel shapes: M >= 512, K a multiple of 64 and >= 128,
+ *                                      N a multiple of 8, y and r 16-byte aligned with row strides
+ *                                      that are multiples of 8
+ *   mvpa_row_sumsq_bf16                sumsq[rows] of plain bf16 rows (parts = 1): the statistics
+ *                                      of the first block's input
+ *   mvpa_linear_bf16_dual_normed       mvpa_linear_bf16_dual on raw rows x with sumsq[M][parts] */
+int32_t mvpa_linear_sumsq_parts(int64_t M, int64_t N);
+int mvpa_linear_bf16_residual_sumsq(const void* x, const void* w, const void* r, void* y, float* sumsq, int64_t M,
+                                    int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldr, int64_t ldy,
+                                    void* stream);
+int mvpa_row_sumsq_bf16(const void* x, float* sumsq, int64_t rows, int32_t cols, int64_t ldx, void* stream);
+int mvpa_linear_bf16_dual_normed(const void* x, const void* w0, void* y0, const void* w1, void* y1, int64_t M,
+                                 int64_t N0, int64_t N1, int64_t K, int64_t ldx, int64_t ldw0, int64_t ldy0,
+                                 int64_t ldw1, int64_t ldy1, const float* sumsq, int32_t parts, float eps,
+                                 void* stream);
+
 /* The same product for at most 128 rows of x against a large weight (the projections of one
  * decoding step of a wide model), with K split over workgroups: fp32 partial tiles go through the
  * caller's workspace ws (mvpa_linear_splitk_ws_bytes(M, N, K, epilogue) bytes, 16-byte aligned)

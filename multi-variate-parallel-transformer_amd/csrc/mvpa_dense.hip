@@ -454,11 +454,27 @@ __device__ inline void tile_of_workgroup(int64_t L, int64_t mt, int64_t nt, int6
 // 16 bytes to each of 32 rows.  Staged through LDS, a wave's 32 x WC outputs of a block j leave as
 // whole rows: 16 bytes per lane, a row's lanes side by side.  EPI 1: SiLU gate; EPI 2: the residual
 // rows R are added where the staged rows are read back.
-template <int BN, int EPI, int LDS_BYTES>
+// Row statistics that ride an epilogue, so that an RMSNorm between two products costs no pass of
+// its own (models/mvpformer.py:133: the norm in front of the block's projections):
+//   STATS 1  the product's x rows are RAW rows whose norm is still due: every output row is
+//            scaled by r = rsqrt(sum of the row's partial sums of squares / cols + eps) while it
+//            is converted (the norm's weight is folded into w's columns by the caller);
+//   STATS 2  the partial sums of squares of the rows this product writes (final bf16 values, this
+//            wave's columns) go to ss_out[m][2 * column tile + column half].
+struct row_stats {
+  const float* ss_in;      // [M][parts_in]
+  int32_t parts_in;
+  float inv_cols, eps;
+  float* ss_out;           // [M][parts_out]
+  int32_t parts_out;
+};
+
+template <int BN, int EPI, int LDS_BYTES, int STATS = 0>
 __device__ inline void staged_epilogue(const f32x16 (&acc)[BN / 64][2], unsigned char* gsm, int wave, int lane,
                                        int64_t m0, int64_t n0, int64_t M, int64_t N,
                                        bf16_t* __restrict__ Y, int64_t ldy,
-                                       const bf16_t* __restrict__ R, int64_t ldr) {
+                                       const bf16_t* __restrict__ R, int64_t ldr,
+                                       const row_stats* rs = nullptr, int64_t tile_n = 0) {
   typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
   constexpr int WN = BN / 2, NB = WN / 32;
   const int ln = lane & 31, hh = lane >> 5;
@@ -473,6 +489,12 @@ __device__ inline void staged_epilogue(const f32x16 (&acc)[BN / 64][2], unsigned
   const bool vec16 = (ldy & 7) == 0 && ((uintptr_t)Y & 15) == 0 &&
                      (EPI != 2 || ((ldr & 7) == 0 && ((uintptr_t)R & 15) == 0));
   const int64_t ncol0 = n0 + wc * WC;
+  float rnorm[2] = {1.f, 1.f};
+  if (STATS == 1) {        // the tile's 256 factors were put behind the ring when the tile began
+    const float* rstat = (const float*)(gsm + LDS_BYTES);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) rnorm[j] = rstat[wm * 64 + j * 32 + ln];
+  }
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     if (EPI == 1) {
@@ -483,7 +505,7 @@ __device__ inline void staged_epilogue(const f32x16 (&acc)[BN / 64][2], unsigned
           bf16x4 o;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const float gte = acc[2 * p2][j][a4 * 4 + r], up = acc[2 * p2 + 1][j][a4 * 4 + r];
+            const float gte = acc[2 * p2][j][a4 * 4 + r] * rnorm[j], up = acc[2 * p2 + 1][j][a4 * 4 + r] * rnorm[j];
             o[r] = (__bf16)(gte / (1.f + __expf(-gte)) * up);
           }
           *(bf16x4*)(stg + ln * PITCH + (p2 * 32 + a4 * 8 + hh * 4) * 2) = o;
@@ -495,7 +517,7 @@ __device__ inline void staged_epilogue(const f32x16 (&acc)[BN / 64][2], unsigned
         for (int a4 = 0; a4 < 4; ++a4) {
           bf16x4 o;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][a4 * 4 + r];
+          for (int r = 0; r < 4; ++r) o[r] = (__bf16)(STATS == 1 ? acc[i][j][a4 * 4 + r] * rnorm[j] : acc[i][j][a4 * 4 + r]);
           *(bf16x4*)(stg + ln * PITCH + (i * 32 + a4 * 8 + hh * 4) * 2) = o;
         }
     }
@@ -510,6 +532,7 @@ __device__ inline void staged_epilogue(const f32x16 (&acc)[BN / 64][2], unsigned
       u32x4 v = *(const u32x4*)(stg + row * PITCH + cc * 16);
       const int64_t m = m0 + wm * 64 + j * 32 + row;
       const int64_t n = ncol0 + cc * 8;
+      float sq = 0.f;
       if (m < M) {
         bf16_t* dst = Y + m * ldy + n;
         if (n + 7 < N && vec16) {
@@ -522,6 +545,13 @@ __device__ inline void staged_epilogue(const f32x16 (&acc)[BN / 64][2], unsigned
               v[e] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
             }
           }
+          if (STATS == 2) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float lo = __uint_as_float(v[e] << 16), hi = __uint_as_float(v[e] & 0xffff0000u);
+              sq += lo * lo + hi * hi;
+            }
+          }
           __builtin_nontemporal_store(v, (u32x4*)dst);   // (streamed out: the operand panels keep the L2)
         } else {
 #pragma unroll
@@ -532,6 +562,16 @@ __device__ inline void staged_epilogue(const f32x16 (&acc)[BN / 64][2], unsigned
               dst[e] = o;
             }
         }
+      }
+      if (STATS == 2) {
+        // the row's CPR lanes sit side by side: lane cc = 0 collects their sums (host side: this
+        // product only runs on shapes that take the 16-byte path above for every chunk)
+#pragma unroll
+        for (int off = 1; off < CPR; off <<= 1) {
+          const float o = __shfl_down(sq, off);
+          if (cc + off < CPR) sq += o;
+        }
+        if (cc == 0 && m < M) rs->ss_out[m * rs->parts_out + tile_n * 2 + wc] = sq;
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -890,12 +930,13 @@ static int launch_ring(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, i
 // the end the last block again, into a stage nobody reads), so the wait is a fixed vmcnt(0).
 // Same tile order, roles, row mapping and epilogues as the other large-tile kernels.
 // -----------------------------------------------------------------------------------------
-template <int BN, int EPI>
+template <int BN, int EPI, int STATS = 0>
 __device__ __forceinline__ void linear_pair_tile(int64_t tile, unsigned char* gsm,
                                                  const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                  bf16_t* __restrict__ Y, int64_t M, int64_t N, int64_t K,
                                                  int64_t ldx, int64_t ldw, int64_t ldy,
-                                                 const bf16_t* __restrict__ R, int64_t ldr) {
+                                                 const bf16_t* __restrict__ R, int64_t ldr,
+                                                 const row_stats* rs = nullptr) {
   constexpr int BM = 256, BK = 64, ROWB = BK * 2, STAGES = 2;
   constexpr int WN = BN / 2, NB = WN / 32;            // per-wave extent over w rows
   constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
@@ -970,9 +1011,38 @@ __device__ __forceinline__ void linear_pair_tile(int64_t tile, unsigned char* gs
   for (int sl = 0; sl < 4; ++sl) frag_off[sl] = ln * ROWB + (((2 * sl + hh) ^ ((ln >> 1) & 7)) << 4);
   const int a_lane = (wm * 64) * ROWB, b_lane = A_BYTES + (wc * WN) * ROWB;
 
+  // STATS 1: the norm factors of the tile's 256 rows, r = rsqrt(sum of the row's partial sums of
+  // squares / K + eps).  Two threads share a row and half of its partial sums each; the loads go
+  // out in front of the first blocks and are long back when those have landed.  The factors wait
+  // in LDS behind the ring for the epilogue.
+  float rpart = 0.f;
+  if (STATS == 1) {
+    const int row = tid >> 1, half = tid & 1;
+    const int64_t m = m0 + row;
+    const int parts = rs->parts_in;
+    if (m < M) {
+      const float* pp = rs->ss_in + m * parts;
+      if ((parts & 7) == 0 && parts <= 16) {
+        typedef __attribute__((ext_vector_type(4))) float f32x4;
+        const f32x4* q4 = (const f32x4*)(pp + half * (parts >> 1));
+        const f32x4 a = q4[0];
+        rpart = (a.x + a.y) + (a.z + a.w);
+        if (parts == 16) {
+          const f32x4 b4 = q4[1];
+          rpart += (b4.x + b4.y) + (b4.z + b4.w);
+        }
+      } else if (half == 0) {
+        for (int p2 = 0; p2 < parts; ++p2) rpart += pp[p2];
+      }
+    }
+  }
   issue_block();
   issue_block();
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(A_LOADS + B_LOADS) : "memory");
+  if (STATS == 1) {
+    rpart += __shfl_xor(rpart, 1);
+    if ((tid & 1) == 0) ((float*)(gsm + STAGES * STAGE))[tid >> 1] = rsqrtf(rpart * rs->inv_cols + rs->eps);
+  }
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   bf16x8 xf0[2], wf0[NB];
 #pragma unroll
@@ -1044,7 +1114,7 @@ __device__ __forceinline__ void linear_pair_tile(int64_t tile, unsigned char* gs
       }
     __builtin_amdgcn_sched_barrier(0);
   }
-  staged_epilogue<BN, EPI, STAGES * STAGE>(acc, gsm, wave, lane, m0, n0, M, N, Y, ldy, R, ldr);
+  staged_epilogue<BN, EPI, STAGES * STAGE, STATS>(acc, gsm, wave, lane, m0, n0, M, N, Y, ldy, R, ldr, rs, tile_n);
 }
 
 template <int BN, int EPI>
@@ -1081,6 +1151,82 @@ __global__ __launch_bounds__(512) void linear_bf16_pair_dual_kernel(const bf16_t
   else
     linear_pair_tile<BN0, 0>(L - gated_tiles, gsm, X, plain.w, plain.y, M, plain.N, K, ldx, plain.ldw, plain.ldy,
                              nullptr, 0);
+}
+
+// the residual product that also writes the partial sums of squares of its output rows
+template <int BN>
+__global__ __launch_bounds__(512) void linear_bf16_pair_sumsq_kernel(const bf16_t* __restrict__ X,
+                                                                     const bf16_t* __restrict__ W,
+                                                                     bf16_t* __restrict__ Y, int64_t M,
+                                                                     int64_t N, int64_t K, int64_t ldx,
+                                                                     int64_t ldw, int64_t ldy,
+                                                                     const bf16_t* __restrict__ R, int64_t ldr,
+                                                                     row_stats rs) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char gsm[];
+  linear_pair_tile<BN, 2, 2>(blockIdx.x, gsm, X, W, Y, M, N, K, ldx, ldw, ldy, R, ldr, &rs);
+}
+
+// the two products on raw rows whose RMSNorm is applied in the epilogue
+template <int BN0>
+__global__ __launch_bounds__(512) void linear_bf16_pair_dual_normed_kernel(const bf16_t* __restrict__ X, int64_t M,
+                                                                           int64_t K, int64_t ldx,
+                                                                           linear_pair_problem plain,
+                                                                           linear_pair_problem gated,
+                                                                           int64_t gated_tiles, row_stats rs) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char gsm[];
+  const int64_t L = blockIdx.x;
+  if (L < gated_tiles)
+    linear_pair_tile<256, 1, 1>(L, gsm, X, gated.w, gated.y, M, gated.N, K, ldx, gated.ldw, gated.ldy, nullptr, 0, &rs);
+  else
+    linear_pair_tile<BN0, 0, 1>(L - gated_tiles, gsm, X, plain.w, plain.y, M, plain.N, K, ldx, plain.ldw, plain.ldy,
+                                nullptr, 0, &rs);
+}
+
+// sums of squares of bf16 rows (one part per row): the statistics of the first block's input
+__global__ __launch_bounds__(256) void row_sumsq_bf16_kernel(const bf16_t* __restrict__ x, float* __restrict__ ss,
+                                                             int64_t rows, int32_t cols, int64_t ldx) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  float sq = 0.f;
+  for (int c = lane * 8; c < cols; c += 512) {
+    const u32x4 v = *(const u32x4*)(x + row * ldx + c);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float lo = __uint_as_float(v[e] << 16), hi = __uint_as_float(v[e] & 0xffff0000u);
+      sq += lo * lo + hi * hi;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sq += __shfl_xor(sq, off);
+  if (lane == 0) ss[row] = sq;
+}
+
+template <int BN>
+static int launch_pair_sumsq(const bf16_t* x, const bf16_t* w, bf16_t* y, int64_t M, int64_t N, int64_t K,
+                             int64_t ldx, int64_t ldw, int64_t ldy, hipStream_t s, const bf16_t* r, int64_t ldr,
+                             float* ss_out, int32_t parts) {
+  constexpr int LDS = 2 * (256 + BN) * 128;
+  auto kern = linear_bf16_pair_sumsq_kernel<BN>;
+  mvpa::want_dynamic_lds((const void*)kern, (int)LDS);
+  dim3 grid((unsigned)(((N + BN - 1) / BN) * ((M + 255) / 256)));
+  const mvpa::row_stats rs{nullptr, 0, 0.f, 0.f, ss_out, parts};
+  MVPA_LAUNCH(kern, grid, dim3(512), LDS, s, x, w, y, M, N, K, ldx, ldw, ldy, r, ldr, rs);
+  return mvpa::take_launch_status();
+}
+
+template <int BN0>
+static int launch_pair_dual_normed(const bf16_t* x, int64_t M, int64_t K, int64_t ldx,
+                                   const mvpa::linear_pair_problem& plain, const mvpa::linear_pair_problem& gated,
+                                   const mvpa::row_stats& rs, hipStream_t s) {
+  constexpr int LDS = 2 * (256 + 256) * 128 + 1024;     // ring + the tile's 256 norm factors
+  auto kern = linear_bf16_pair_dual_normed_kernel<BN0>;
+  mvpa::want_dynamic_lds((const void*)kern, (int)LDS);
+  const int64_t mt = (M + 255) / 256;
+  const int64_t gated_tiles = mt * ((gated.N + 127) / 128), plain_tiles = mt * ((plain.N + BN0 - 1) / BN0);
+  MVPA_LAUNCH(kern, dim3((unsigned)(gated_tiles + plain_tiles)), dim3(512), LDS, s, x, M, K, ldx, plain, gated,
+              gated_tiles, rs);
+  return mvpa::take_launch_status();
 }
 
 template <int BN, int EPI>
@@ -1564,9 +1710,6 @@ extern "C" int mvpa_linear_bf16(const void* x, const void* w, void* y, int64_t M
   return mvpa::take_launch_status();
 }
 
-// y0 = x w0^T and y1 = silu(x wg^T) * (x wu^T) in one launch (w1 holds the gate rows [0, N1) and
-// the up rows [N1, 2 N1)): the two products that read ln_1(x) in the parallel block.  Large
-// shapes only: at least 512 rows, K a multiple of 64; MVPA_ERR_UNSUPPORTED otherwise.
 extern "C" int mvpa_linear_f32(const float* x, const float* w, float* y, int64_t M, int64_t N, int64_t K,
                                int64_t ldx, int64_t ldw, int64_t ldy, void* stream) {
   if (!x || !w || !y) return MVPA_ERR_NULL;
@@ -1576,9 +1719,15 @@ extern "C" int mvpa_linear_f32(const float* x, const float* w, float* y, int64_t
   return mvpa::take_launch_status();
 }
 
-extern "C" int mvpa_linear_bf16_dual(const void* x, const void* w0, void* y0, const void* w1, void* y1,
-                                     int64_t M, int64_t N0, int64_t N1, int64_t K, int64_t ldx,
-                                     int64_t ldw0, int64_t ldy0, int64_t ldw1, int64_t ldy1, void* stream) {
+// y0 = x w0^T and y1 = silu(x wg^T) * (x wu^T) in one launch (w1 holds the gate rows [0, N1) and
+// the up rows [N1, 2 N1)): the two products that read ln_1(x) in the parallel block.  Large
+// shapes only: at least 512 rows, K a multiple of 64; MVPA_ERR_UNSUPPORTED otherwise.
+// With sumsq given, x holds the RAW rows and their RMSNorm happens in the epilogue
+// (mvpa_linear_bf16_dual_normed).
+static int linear_dual_impl(const void* x, const void* w0, void* y0, const void* w1, void* y1,
+                            int64_t M, int64_t N0, int64_t N1, int64_t K, int64_t ldx,
+                            int64_t ldw0, int64_t ldy0, int64_t ldw1, int64_t ldy1,
+                            const float* sumsq, int32_t parts, float eps, void* stream) {
   if (!x || !w0 || !y0 || !w1 || !y1) return MVPA_ERR_NULL;
   if (M <= 0 || N0 <= 0 || N1 <= 0 || K <= 0 || ldx < K || ldw0 < K || ldw1 < K || ldy0 < N0 || ldy1 < N1)
     return MVPA_ERR_SHAPE;
@@ -1593,9 +1742,75 @@ extern "C" int mvpa_linear_bf16_dual(const void* x, const void* w0, void* y0, co
   // the plain product's tile width: the one that wastes the fewest padded columns
   const int64_t pad256 = (N0 + 255) / 256 * 256, pad192 = (N0 + 191) / 192 * 192, pad128 = (N0 + 127) / 128 * 128;
   hipStream_t s = (hipStream_t)stream;
+  if (sumsq) {
+    const mvpa::row_stats rs{sumsq, parts, 1.f / (float)K, eps, nullptr, 0};
+    if (pad256 <= pad192 && pad256 <= pad128)
+      return mvpa::launch_pair_dual_normed<256>((const bf16_t*)x, M, K, ldx, plain, gated, rs, s);
+    if (pad192 <= pad128) return mvpa::launch_pair_dual_normed<192>((const bf16_t*)x, M, K, ldx, plain, gated, rs, s);
+    return mvpa::launch_pair_dual_normed<128>((const bf16_t*)x, M, K, ldx, plain, gated, rs, s);
+  }
   if (pad256 <= pad192 && pad256 <= pad128) return launch_pair_dual<256>((const bf16_t*)x, M, K, ldx, plain, gated, s);
   if (pad192 <= pad128) return launch_pair_dual<192>((const bf16_t*)x, M, K, ldx, plain, gated, s);
   return launch_pair_dual<128>((const bf16_t*)x, M, K, ldx, plain, gated, s);
+}
+
+extern "C" int mvpa_linear_bf16_dual(const void* x, const void* w0, void* y0, const void* w1, void* y1,
+                                     int64_t M, int64_t N0, int64_t N1, int64_t K, int64_t ldx,
+                                     int64_t ldw0, int64_t ldy0, int64_t ldw1, int64_t ldy1, void* stream) {
+  return linear_dual_impl(x, w0, y0, w1, y1, M, N0, N1, K, ldx, ldw0, ldy0, ldw1, ldy1, nullptr, 0, 0.f, stream);
+}
+
+extern "C" int mvpa_linear_bf16_dual_normed(const void* x, const void* w0, void* y0, const void* w1, void* y1,
+                                            int64_t M, int64_t N0, int64_t N1, int64_t K, int64_t ldx,
+                                            int64_t ldw0, int64_t ldy0, int64_t ldw1, int64_t ldy1,
+                                            const float* sumsq, int32_t parts, float eps, void* stream) {
+  if (!sumsq) return MVPA_ERR_NULL;
+  if (parts <= 0 || parts > 64) return MVPA_ERR_SHAPE;
+  return linear_dual_impl(x, w0, y0, w1, y1, M, N0, N1, K, ldx, ldw0, ldy0, ldw1, ldy1, sumsq, parts, eps, stream);
+}
+
+// tile width of the residual product for a shape (the one that needs the fewest workgroup rounds x
+// width on 256 CUs), and with it the number of partial sums a row gets
+static int residual_tile_width(int64_t M, int64_t N) {
+  const int64_t mt = (M + 255) / 256;
+  auto cost = [&](int bn) -> int64_t { return ((mt * ((N + bn - 1) / bn) + 255) / 256) * bn; };
+  const int64_t c256 = cost(256), c192 = cost(192), c128 = cost(128);
+  return (c256 <= c192 && c256 <= c128) ? 256 : c192 <= c128 ? 192 : 128;
+}
+
+extern "C" int32_t mvpa_linear_sumsq_parts(int64_t M, int64_t N) {
+  if (M <= 0 || N <= 0) return 0;
+  const int bn = residual_tile_width(M, N);
+  return (int32_t)(2 * ((N + bn - 1) / bn));
+}
+
+extern "C" int mvpa_linear_bf16_residual_sumsq(const void* x, const void* w, const void* r, void* y, float* sumsq,
+                                               int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw,
+                                               int64_t ldr, int64_t ldy, void* stream) {
+  if (!x || !w || !y || !r || !sumsq) return MVPA_ERR_NULL;
+  if (M <= 0 || N <= 0 || K <= 0 || ldx < K || ldw < K || ldy < N || ldr < N) return MVPA_ERR_SHAPE;
+  if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || (ldx & 7) || (ldw & 7)) return MVPA_ERR_ALIGN;
+  // whole 16-byte chunks of every output row, so that each takes the vector path of the epilogue
+  if (((uintptr_t)y & 15) || ((uintptr_t)r & 15) || (ldy & 7) || (ldr & 7) || (N & 7)) return MVPA_ERR_ALIGN;
+  const bool pair = M >= 512 && (K & 63) == 0 && K >= 128 && 256 * ldx < ((int64_t)1 << 30) &&
+                    256 * ldw < ((int64_t)1 << 30);
+  if (!pair) return MVPA_ERR_UNSUPPORTED;
+  hipStream_t s = (hipStream_t)stream;
+  const bf16_t *xp = (const bf16_t*)x, *wp = (const bf16_t*)w, *rp = (const bf16_t*)r;
+  const int bn = residual_tile_width(M, N);
+  const int32_t parts = (int32_t)(2 * ((N + bn - 1) / bn));
+  if (bn == 256) return mvpa::launch_pair_sumsq<256>(xp, wp, (bf16_t*)y, M, N, K, ldx, ldw, ldy, s, rp, ldr, sumsq, parts);
+  if (bn == 192) return mvpa::launch_pair_sumsq<192>(xp, wp, (bf16_t*)y, M, N, K, ldx, ldw, ldy, s, rp, ldr, sumsq, parts);
+  return mvpa::launch_pair_sumsq<128>(xp, wp, (bf16_t*)y, M, N, K, ldx, ldw, ldy, s, rp, ldr, sumsq, parts);
+}
+
+extern "C" int mvpa_row_sumsq_bf16(const void* x, float* sumsq, int64_t rows, int32_t cols, int64_t ldx, void* stream) {
+  if (!x || !sumsq) return MVPA_ERR_NULL;
+  if (rows <= 0 || cols <= 0 || ldx < cols) return MVPA_ERR_SHAPE;
+  if (((uintptr_t)x & 15) || (ldx & 7) || (cols & 7)) return MVPA_ERR_ALIGN;
+  MVPA_LAUNCH(mvpa::row_sumsq_bf16_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+              (const bf16_t*)x, sumsq, rows, cols, ldx);
+  return mvpa::take_launch_status();
 }
 
 // Y = X W^T + R in one kernel (the large-tile ring kernel only): at least 512 rows, K a multiple

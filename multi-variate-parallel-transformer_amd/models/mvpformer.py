@@ -134,6 +134,8 @@ class MVPFormerBlock(nn.Module):
         self.mlp = GatedMLP(config)
         self._tail_w = None
         self._tail_key = None
+        self._fold_w = None
+        self._fold_key = None
 
     def _tail_weight(self) -> torch.Tensor:
         """[c_proj | down_proj] side by side ([E, E + intermediate]), cached until one changes:
@@ -144,6 +146,50 @@ class MVPFormerBlock(nn.Module):
             self._tail_w = torch.cat([wc, wd], 1).detach().to(torch.bfloat16).contiguous()
             self._tail_key = key
         return self._tail_w
+
+    def _folded_weights(self):
+        """[q_attn; c_attn] and [gate; up] with ln_1's weight folded into their columns
+        (w[n][k] * ln_1[k], formed in fp32, rounded to bf16), cached until a source changes: the
+        operands of the products that apply ln_1 in their epilogue (forward_norm_fused)."""
+        wq, wg, ln = self.attn.qkv_weight(), self.mlp.gate_up_weight(), self.ln_1.weight
+        key = (wq.data_ptr(), wq._version, wg.data_ptr(), wg._version, ln.data_ptr(), ln._version)
+        if self._fold_key != key:
+            scale = ln.detach().float()[None, :]
+            self._fold_w = ((wq.float() * scale).to(torch.bfloat16).contiguous(),
+                            (wg.float() * scale).to(torch.bfloat16).contiguous())
+            self._fold_key = key
+        return self._fold_w
+
+    def norm_fused_supported(self, rows: int) -> bool:
+        e, inner = self.attn.embed_dim, self.mlp.down_proj.in_features
+        return (mvpa_hip.linear_dual_supported(rows, e) and mvpa_hip.linear_norm_fused_supported(rows, e + inner, e)
+                and mvpa_hip.linear_residual_supported(rows, e + inner))
+
+    @torch.no_grad()
+    def forward_norm_fused(self, hidden_states, sumsq, positional_embedding, channel_embedding,
+                           attention_mask=None, use_cache=False, both=None):
+        """The block on its RAW input, ln_1 applied inside the products (models/mvpformer.py:133):
+        `sumsq` holds the partial sums of squares of hidden_states' rows, as the previous block's
+        tail product (or mvpa_hip.row_sumsq) wrote them; the q/kv and gate/up products multiply
+        the raw rows with weights that carry ln_1's weight and scale each output row by its
+        rsqrt(mean square + eps) in the epilogue; the tail product writes the next block's
+        statistics beside its rows.  No norm kernel runs.  `both`: a [rows, E + intermediate]
+        bf16 scratch buffer to reuse.  Returns (outputs, sumsq of the output rows)."""
+        bsz, t_len, c_len, e = hidden_states.shape
+        inner = self.mlp.down_proj.in_features
+        rows = bsz * t_len * c_len
+        h, dh = self.attn.num_heads, self.attn.head_dim
+        if both is None:
+            both = torch.empty((rows, e + inner), dtype=torch.bfloat16, device=hidden_states.device)
+        merged = both[:, :e].unflatten(0, (bsz, t_len * c_len)).unflatten(2, (h, dh))
+        wq, wg = self._folded_weights()
+        x2 = hidden_states.reshape(rows, e)
+        qkv, _ = mvpa_hip.linear_dual(x2, wq, wg, out_gated=both[:, e:], sumsq=sumsq, eps=self.ln_1.eps)
+        _, present = self.attn.forward_merged(hidden_states, positional_embedding, channel_embedding, merged,
+                                              attention_mask=attention_mask, use_cache=use_cache, qkv=qkv)
+        out, sumsq = mvpa_hip.linear(both, self._tail_weight(), residual=x2, sumsq_out=True)
+        out = out.view(hidden_states.shape)
+        return ((out, present) if use_cache else (out,)), sumsq
 
     def forward(self, hidden_states, positional_embedding, channel_embedding, layer_past=None,
                 attention_mask=None, head_mask=None, encoder_hidden_states=None,
@@ -334,6 +380,24 @@ class MVPFormerModel(nn.Module):
         hidden_states, normed = inputs_embeds, None
         n_layers = len(self.h)
         presents = () if use_cache else None
+        rows = bsz * t_len * c_len
+        if (n_layers > 0 and past_key_values is None and not torch.is_grad_enabled() and hidden_states.is_cuda
+                and hidden_states.dtype == torch.bfloat16 and self.h[0].norm_fused_supported(rows)):
+            # every ln_1 inside the products around it: the statistics of a block's input come out of
+            # the previous block's tail product (of one small pass for the first block)
+            e = self.embed_dim
+            sumsq = mvpa_hip.row_sumsq(hidden_states.reshape(rows, e))
+            both = torch.empty((rows, e + self.h[0].mlp.down_proj.in_features), dtype=torch.bfloat16,
+                               device=hidden_states.device)
+            for block in self.h:
+                outputs, sumsq = block.forward_norm_fused(hidden_states, sumsq, position_embeds, channel_embeds,
+                                                          attention_mask=attention_mask, use_cache=use_cache,
+                                                          both=both)
+                hidden_states = outputs[0]
+                if use_cache:
+                    presents = presents + (outputs[1],)
+            out = self.ln_f(hidden_states).view(bsz, inputs_embeds.shape[1], c_len, -1)
+            return (out, presents) if use_cache else out
         for i, block in enumerate(self.h):
             next_norm = self.h[i + 1].ln_1 if i + 1 < n_layers else self.ln_f
             layer_past = past_key_values[i] if past_key_values is not None else None

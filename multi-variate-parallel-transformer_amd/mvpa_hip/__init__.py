@@ -110,6 +110,15 @@ def load_library() -> ctypes.CDLL:
     lib.mvpa_static_ws_init.argtypes = []
     lib.mvpa_backward.restype = ctypes.c_int
     lib.mvpa_backward.argtypes = [ctypes.POINTER(MvpaBwdArgs), vp]
+    lib.mvpa_linear_sumsq_parts.restype = ctypes.c_int32
+    lib.mvpa_linear_sumsq_parts.argtypes = [i64, i64]
+    lib.mvpa_linear_bf16_residual_sumsq.restype = ctypes.c_int
+    lib.mvpa_linear_bf16_residual_sumsq.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp]
+    lib.mvpa_row_sumsq_bf16.restype = ctypes.c_int
+    lib.mvpa_row_sumsq_bf16.argtypes = [vp, vp, i64, i32, i64, vp]
+    lib.mvpa_linear_bf16_dual_normed.restype = ctypes.c_int
+    lib.mvpa_linear_bf16_dual_normed.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, i64,
+                                                 vp, i32, f32, vp]
     lib.mvpa_linear_f32.restype = ctypes.c_int
     lib.mvpa_linear_f32.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, vp]
     lib.mvpa_fp8_prepare.restype = ctypes.c_int
@@ -423,10 +432,14 @@ def linear_dual_supported(M: int, K: int) -> bool:
 
 
 def linear_dual(x: torch.Tensor, w_plain: torch.Tensor, w_gated: torch.Tensor,
-                out_plain: Optional[torch.Tensor] = None, out_gated: Optional[torch.Tensor] = None):
+                out_plain: Optional[torch.Tensor] = None, out_gated: Optional[torch.Tensor] = None,
+                sumsq: Optional[torch.Tensor] = None, eps: float = 1e-5):
     """(x @ w_plain.T, silu(x @ gate.T) * (x @ up.T)) from ONE launch; w_gated stacks [gate; up]
     rows.  x is [rows, K] (or any shape with K last, contiguous); the outputs are 2-D, and either
-    may be a given [rows, N] view with unit last stride (a column slice of a wider buffer)."""
+    may be a given [rows, N] view with unit last stride (a column slice of a wider buffer).
+    sumsq ([rows, parts] fp32, from row_sumsq or linear(..., sumsq_out=True)): x holds RAW rows
+    whose RMSNorm is applied in the epilogue - every output row is scaled by
+    rsqrt(sum(sumsq[row]) / K + eps); the weights must carry the norm's weight in their columns."""
     lib = load_library()
     _need_cuda(x, w_plain, w_gated)
     if x.dtype != torch.bfloat16 or w_plain.dtype != torch.bfloat16 or w_gated.dtype != torch.bfloat16:
@@ -444,21 +457,50 @@ def linear_dual(x: torch.Tensor, w_plain: torch.Tensor, w_gated: torch.Tensor,
         elif o.dim() != 2 or tuple(o.shape) != (M, n) or o.stride(1) != 1 or o.dtype != torch.bfloat16:
             raise ValueError("linear_dual: outputs must be bf16 [rows, N] tensors or views with unit last stride")
         outs.append(o)
+    if sumsq is not None:
+        if sumsq.dtype != torch.float32 or sumsq.dim() != 2 or sumsq.shape[0] != M or not sumsq.is_contiguous():
+            raise ValueError("linear_dual: sumsq must be a contiguous fp32 [rows, parts] tensor")
+        _need_cuda(sumsq)
+        _check(lib.mvpa_linear_bf16_dual_normed(
+            x2.data_ptr(), w_plain.data_ptr(), outs[0].data_ptr(), w_gated.data_ptr(), outs[1].data_ptr(),
+            M, N0, N1, K, x2.stride(0), w_plain.stride(0), outs[0].stride(0), w_gated.stride(0),
+            outs[1].stride(0), sumsq.data_ptr(), sumsq.shape[1], float(eps), _stream()))
+        return outs[0], outs[1]
     _check(lib.mvpa_linear_bf16_dual(x2.data_ptr(), w_plain.data_ptr(), outs[0].data_ptr(), w_gated.data_ptr(),
                                      outs[1].data_ptr(), M, N0, N1, K, x2.stride(0), w_plain.stride(0),
                                      outs[0].stride(0), w_gated.stride(0), outs[1].stride(0), _stream()))
     return outs[0], outs[1]
 
 
+def row_sumsq(x: torch.Tensor) -> torch.Tensor:
+    """[rows, 1] fp32 sums of squares of bf16 rows ([rows, cols] view, unit last stride, cols a
+    multiple of 8): the row statistics an RMSNorm needs, in the form linear_dual(sumsq=...) takes."""
+    lib = load_library()
+    _need_cuda(x)
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or x.stride(1) != 1:
+        raise TypeError("row_sumsq: a bf16 [rows, cols] tensor or view with unit last stride")
+    out = torch.empty((x.shape[0], 1), dtype=torch.float32, device=x.device)
+    _check(lib.mvpa_row_sumsq_bf16(x.data_ptr(), out.data_ptr(), x.shape[0], x.shape[1], x.stride(0), _stream()))
+    return out
+
+
+def linear_norm_fused_supported(M: int, K: int, N: int) -> bool:
+    """Shapes for which the tail product can write row statistics (linear(..., sumsq_out=True))
+    and the dual product can consume them (linear_dual(sumsq=...))."""
+    return M >= 512 and K % 64 == 0 and K >= 128 and N % 8 == 0
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None,
            gated: bool = False, split_k: Optional[bool] = None,
-           residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+           residual: Optional[torch.Tensor] = None, sumsq_out: bool = False) -> torch.Tensor:
     """y = x @ weight.T in bf16 on MFMA.  gated=True: weight stacks [gate; up] rows and the
     result is silu(x@gate.T) * (x@up.T).  split_k: the K-split kernel pair through a workspace
     (at most 128 rows); None picks it for K >= 1536 and at most 4096 rows of weight.
     x may be a 2-D row-pitched view (unit last stride), out a 2-D view [rows, N] likewise.
     residual: [rows, N] bf16 added in the product's epilogue (shapes for which
-    linear_residual_supported holds; otherwise MvpaError)."""
+    linear_residual_supported holds; otherwise MvpaError).
+    sumsq_out (with residual): also returns the partial sums of squares of the output rows,
+    [rows, parts] fp32 - (out, sumsq) comes back - for a later linear_dual(sumsq=...)."""
     lib = load_library()
     _need_cuda(x, weight)
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
@@ -483,10 +525,18 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = 
         if tuple(r2.shape) != (M, N) or r2.stride(1) != 1 or r2.dtype != torch.bfloat16:
             raise ValueError("linear: residual must be bf16 [rows, N] with unit last stride")
         _need_cuda(r2)
+        if sumsq_out:
+            ss = torch.empty((M, lib.mvpa_linear_sumsq_parts(M, N)), dtype=torch.float32, device=x.device)
+            _check(lib.mvpa_linear_bf16_residual_sumsq(x2.data_ptr(), weight.data_ptr(), r2.data_ptr(), out.data_ptr(),
+                                                       ss.data_ptr(), M, N, K, x2.stride(0), weight.stride(0),
+                                                       r2.stride(0), out.stride(0), _stream()))
+            return (out if given else out.view(*x.shape[:-1], N)), ss
         _check(lib.mvpa_linear_bf16_residual(x2.data_ptr(), weight.data_ptr(), r2.data_ptr(), out.data_ptr(),
                                              M, N, K, x2.stride(0), weight.stride(0), r2.stride(0),
                                              out.stride(0), _stream()))
         return out if given else out.view(*x.shape[:-1], N)
+    if sumsq_out:
+        raise ValueError("linear: sumsq_out goes with residual")
     if split_k is None:
         # measured on graph replays (GPU time): [128x2048]x[2048x4096] 22.9 -> 18.6 us,
         # [128x5632]x[5632x2048] 58.1 -> 21.0 us, [64x1728]x[1728x768] 13.2 -> 10.0 us; the wide
