@@ -30,19 +30,33 @@ __global__ __launch_bounds__(FP8_THREADS) void fp8_amax_kernel(mvpa_fwd_args a, 
   const int64_t stride = is_q ? a.q_stride_n : a.k_stride_n;
   const bf16_t* bias = (const bf16_t*)a.bias_u + g * a.Dh;
   float mx = 0.f;
-  for (int64_t c = (int64_t)blockIdx.x * FP8_THREADS + threadIdx.x; c < rows * cpr;
-       c += (int64_t)gridDim.x * FP8_THREADS) {
-    const int64_t row = c / cpr;
-    const int col = (int)(c % cpr) * 8;
-    const u32x4 raw = *(const u32x4*)(base + row * stride + col);
-    u32x4 braw = {0u, 0u, 0u, 0u};
-    if (is_q) braw = *(const u32x4*)(bias + col);
+  // a thread keeps one column chunk (and its bias) and walks rows, four loads in flight at a time
+  const int tpr = FP8_THREADS / cpr * cpr;                    // threads in use (a whole number of rows)
+  const int col = (int)(threadIdx.x % cpr) * 8;
+  const int64_t rstep = (int64_t)gridDim.x * (tpr / cpr);
+  u32x4 braw = {0u, 0u, 0u, 0u};
+  if (is_q) braw = *(const u32x4*)(bias + col);
+  auto fold = [&](const u32x4& raw) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const float lo = __uint_as_float(raw[i] << 16) + __uint_as_float(braw[i] << 16);
       const float hi = __uint_as_float(raw[i] & 0xffff0000u) + __uint_as_float(braw[i] & 0xffff0000u);
       mx = fmaxf(mx, fmaxf(fabsf(lo), fabsf(hi)));
     }
+  };
+  if ((int)threadIdx.x < tpr) {
+    int64_t row = (int64_t)blockIdx.x * (tpr / cpr) + threadIdx.x / cpr;
+    for (; row + 3 * rstep < rows; row += 4 * rstep) {
+      const u32x4 r0 = *(const u32x4*)(base + row * stride + col);
+      const u32x4 r1 = *(const u32x4*)(base + (row + rstep) * stride + col);
+      const u32x4 r2 = *(const u32x4*)(base + (row + 2 * rstep) * stride + col);
+      const u32x4 r3 = *(const u32x4*)(base + (row + 3 * rstep) * stride + col);
+      fold(r0);
+      fold(r1);
+      fold(r2);
+      fold(r3);
+    }
+    for (; row < rows; row += rstep) fold(*(const u32x4*)(base + row * stride + col));
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
