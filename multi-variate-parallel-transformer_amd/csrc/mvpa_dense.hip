@@ -1039,10 +1039,6 @@ __device__ __forceinline__ void linear_pair_tile(int64_t tile, unsigned char* gs
   issue_block();
   issue_block();
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(A_LOADS + B_LOADS) : "memory");
-  if (STATS == 1) {
-    rpart += __shfl_xor(rpart, 1);
-    if ((tid & 1) == 0) ((float*)(gsm + STAGES * STAGE))[tid >> 1] = rsqrtf(rpart * rs->inv_cols + rs->eps);
-  }
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   bf16x8 xf0[2], wf0[NB];
 #pragma unroll
@@ -1097,6 +1093,12 @@ __device__ __forceinline__ void linear_pair_tile(int64_t tile, unsigned char* gs
     __builtin_amdgcn_sched_barrier(0);
     // the next block has landed, and every fragment of this one is in registers: publish / free
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (STATS == 1 && kb == 0) {
+      // (every load of this wave is back here, the partial sums among them: no wait of their own;
+      // the factors are published by the barriers of the blocks that follow)
+      rpart += __shfl_xor(rpart, 1);
+      if ((tid & 1) == 0) ((float*)(gsm + STAGES * STAGE))[tid >> 1] = rsqrtf(rpart * rs->inv_cols + rs->eps);
+    }
 #pragma unroll
     for (int j = 0; j < 2; ++j) xf0[j] = *(const bf16x8*)(sn + a_lane + j * 32 * ROWB + frag_off[0]);
 #pragma unroll
