@@ -142,6 +142,47 @@ def test_block_order_is_a_permutation_and_keeps_kv_groups_on_one_xcd(lib, B, H, 
                 assert len({p for p, _ in mine}) == grp and len({t for _, t in mine}) == 1
 
 
+def test_new_entry_points_reject_bad_arguments(lib):
+    """Host-side validation of the entry points around the fp8 content term, the fp32 product and
+    the norm-in-the-products path: every rejection comes back before anything is launched."""
+    buf = ctypes.create_string_buffer(256)
+    p16 = (ctypes.addressof(buf) + 15) & ~15
+    assert lib.mvpa_linear_f32(None, None, None, 1, 1, 1, 1, 1, 1, None) == -1
+    assert lib.mvpa_linear_f32(p16, p16, p16, 4, 4, 8, 4, 8, 4, None) == -5              # ldx < K
+    assert lib.mvpa_row_sumsq_bf16(None, None, 1, 8, 8, None) == -1
+    assert lib.mvpa_row_sumsq_bf16(p16, p16, 4, 12, 16, None) == -7                      # cols not a multiple of 8
+    assert lib.mvpa_row_sumsq_bf16(p16, p16, 4, 16, 8, None) == -5                       # ldx < cols
+    assert lib.mvpa_linear_sumsq_parts(16384, 768) == 8 and lib.mvpa_linear_sumsq_parts(65536, 2048) == 16
+    assert lib.mvpa_linear_sumsq_parts(0, 8) == 0
+    assert lib.mvpa_linear_bf16_residual_sumsq(p16, p16, p16, p16, None, 512, 64, 128, 128, 128, 64, 64, None) == -1
+    assert lib.mvpa_linear_bf16_residual_sumsq(p16, p16, p16, p16, p16, 512, 60, 128, 128, 128, 64, 64, None) == -7   # N % 8
+    assert lib.mvpa_linear_bf16_residual_sumsq(p16, p16, p16, p16, p16, 64, 64, 128, 128, 128, 64, 64, None) == -8    # too few rows
+    assert lib.mvpa_linear_bf16_dual_normed(p16, p16, p16, p16, p16, 512, 64, 64, 128, 128, 128, 64, 128, 64,
+                                            None, 8, 1e-5, None) == -1
+    assert lib.mvpa_linear_bf16_dual_normed(p16, p16, p16, p16, p16, 512, 64, 64, 128, 128, 128, 64, 128, 64,
+                                            p16, 0, 1e-5, None) == -5
+    a, keep = _args(B=1, H=2, Hkv=2, T=8, C=40, Dh=64, dtype=torch.bfloat16)
+    assert lib.mvpa_fp8_prepare(None, p16, p16, None, None) == -1
+    assert lib.mvpa_fp8_prepare(ctypes.byref(a), None, p16, None, None) == -1
+    a.struct_size = 16
+    assert lib.mvpa_fp8_prepare(ctypes.byref(a), p16, p16, None, None) == -9
+    a, keep = _args(B=1, H=2, Hkv=2, T=8, C=40, Dh=64, dtype=torch.float32)
+    assert lib.mvpa_fp8_prepare(ctypes.byref(a), p16, p16, None, None) == -8             # bf16 only
+    a, keep = _args(B=1, H=3, Hkv=2, T=8, C=40, Dh=64, dtype=torch.bfloat16)
+    assert lib.mvpa_fp8_prepare(ctypes.byref(a), p16, p16, None, None) == -3
+    # the column-split build needs the keys' e4m3 copy for the fp8 content term
+    a, keep = _args(B=1, H=2, Hkv=2, T=8, C=100, Dh=128, dtype=torch.bfloat16)
+    a.flags |= mvpa_hip.FLAG_FP8_QK
+    a.fp8_q_scale = a.fp8_k_scale = p16
+    a.kernel = mvpa_hip.KERNEL_MFMA_SPLIT
+    assert lib.mvpa_validate(ctypes.byref(a)) == -8
+    a.k_fp8 = p16
+    assert lib.mvpa_validate(ctypes.byref(a)) == 0
+    a.kernel = mvpa_hip.KERNEL_AUTO
+    a.k_fp8 = None
+    assert lib.mvpa_validate(ctypes.byref(a)) == 0          # AUTO then keeps the general kernel
+
+
 def test_null_block(lib):
     assert lib.mvpa_validate(None) == -1
 
