@@ -82,9 +82,10 @@ def algorithmic_flops(B, H, T, C, Dh, window=10):
     return B * H * 2 * Dh * (p_causal + p_window + n * (T + C))
 
 
-def _extra_workload(key, warmup=3, steps=5):
+def _extra_workload(key, warmup=3, steps=5, backward=True):
     """One of the other benchmark shapes on the library's own kernel choice: HIP-event time per
-    launch over `steps` launches, algorithmic TFLOP/s and the fraction of the dense bf16 peak."""
+    launch over `steps` launches, algorithmic TFLOP/s and the fraction of the dense bf16 peak;
+    with `backward`, the time of one mvpa_backward call on the same inputs beside it."""
     import torch
     import mvpa_hip
     from mvpa_hip.synthetic import make_mvpa_inputs
@@ -110,11 +111,28 @@ def _extra_workload(key, warmup=3, steps=5):
     ms = ev0.elapsed_time(ev1) / steps
     flops = algorithmic_flops(B, H, T, C, Dh)
     tf = flops / (ms * 1e-3) / 1e12
-    return {"workload": f"B={B} C={C} T={T} H={H} Hkv={Hkv} Dh={Dh}"
-                        + (", per-sample channel validity" if cfg["validity"] else ""),
-            "ms": round(ms, 4), "steps": steps, "tflops": round(tf, 1),
-            "frac": round(tf / BF16_DENSE_PEAK_TFLOPS, 4), "algorithmic_flops": flops,
-            "kernel": _forward_kernel_name(cfg)}
+    res = {"workload": f"B={B} C={C} T={T} H={H} Hkv={Hkv} Dh={Dh}"
+                       + (", per-sample channel validity" if cfg["validity"] else ""),
+           "ms": round(ms, 4), "steps": steps, "tflops": round(tf, 1),
+           "frac": round(tf / BF16_DENSE_PEAK_TFLOPS, 4), "algorithmic_flops": flops,
+           "kernel": _forward_kernel_name(cfg)}
+    if backward:
+        _, lse = mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan,
+                                       chan_valid=d.chan_valid, return_lse=True)
+        d_o = torch.randn_like(out)
+
+        def bwd():
+            return mvpa_hip.mvpa_backward(d.q, d.k, d.v, out, d_o, lse, d.u, d.vb, d.z, d.k_time,
+                                          d.k_chan, chan_valid=d.chan_valid)
+        bwd()
+        torch.cuda.synchronize()
+        ev0.record()
+        for _ in range(2):
+            bwd()
+        ev1.record()
+        torch.cuda.synchronize()
+        res["backward_ms"] = round(ev0.elapsed_time(ev1) / 2, 3)
+    return res
 
 
 def cpu_baseline(cfg, budget_s=8.0):
@@ -316,7 +334,7 @@ def main():
         # the base model
         for key in ("c3", "c5attn"):
             if key != args.workload:
-                line["mvpa_" + key] = _extra_workload(key)
+                line["mvpa_" + key] = _extra_workload(key, backward=not args.no_backward)
     if not args.no_model:
         try:
             from bench_model import mvpformer_s_windows_per_s

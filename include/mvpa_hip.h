@@ -245,7 +245,7 @@ typedef struct mvpa_bwd_args {
   float* ws_time;            /* workspace [B,H,N,T]                                           */
   float* ws_chan;            /* workspace [B,H,N,C rounded up to a multiple of 4]             */
   void* ws_qu;               /* nullable workspace [B,H,N,Dh] of `dtype`, 16-byte aligned; the
-                                matrix-core kernels (bf16, Dh = 64, C <= 128, no key_bias)
+                                matrix-core kernels (bf16, Dh = 64 or 128, C <= 128, no key_bias)
                                 run only when it is given                                     */
 } mvpa_bwd_args;
 

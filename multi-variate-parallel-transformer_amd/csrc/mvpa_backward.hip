@@ -323,7 +323,7 @@ extern "C" int mvpa_backward(const mvpa_bwd_args* a, void* stream) {
     return MVPA_ERR_NONCAUSAL_BIAS;
   if (a->dtype == MVPA_F32) return mvpa::launch_bwd_dh<float>(a, (hipStream_t)stream, true);
   if (a->dtype == MVPA_BF16) {
-    // bf16, Dh = 64, C <= 128: both passes run on MFMA
+    // bf16, Dh = 64 or 128, C <= 128: both passes run on MFMA
     if (mvpa_bwd_query_mfma_supported(a)) return mvpa_launch_bwd_mfma(a, (hipStream_t)stream);
     return mvpa::launch_bwd_dh<mvpa::bf16_t>(a, (hipStream_t)stream, true);
   }

@@ -1,4 +1,4 @@
-// MVPA backward on MFMA (bf16, Dh = 64, up to 64 channels per launch, 128 in parts): the QUERY pass (the KEY pass follows below).
+// MVPA backward on MFMA (bf16, Dh = 64 or 128, up to 64 channels per launch, 128 in parts): the QUERY pass (the KEY pass follows below).
 //
 // Same tiling as the forward kernel: queries and keys are tiled by time step, a wave owns 32
 // query channels of one time step, products are formed transposed (a lane owns one query), the
@@ -33,11 +33,14 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 #define BWD_LDS_PTR(T) __attribute__((address_space(3))) T*
 
-constexpr int DH = 64, KS = 4, MT = 2, ROWB = 128, NW = 4;
-constexpr int QSTAGES = 3, KSTAGES = 3;          // ring depth of the query / key pass
-// waves per workgroup of the query pass: with two channel tiles 8 waves (4 query time steps) share
-// the K/V ring and each SIMD holds two waves
-template <int NCT> constexpr int QUERY_WAVES = NCT == 2 ? 8 : 4;
+// Head dim DH is 64 or 128: KS = DH / 16 contraction blocks per product, MT = DH / 32 output tiles
+// of the gradients, rows of ROWB = 2 DH bytes (CPR = DH / 8 chunks of 16 bytes) in the LDS tiles.
+constexpr int KSTAGES = 3;                        // ring depth of the key pass
+// ring depth of the query pass: three stages, two where three would not fit the LDS
+template <int DH, int NCT> constexpr int QSTAGES = (DH == 128 && NCT == 2) ? 2 : 3;
+// waves per workgroup of the query pass: with two channel tiles of Dh 64 8 waves (4 query time
+// steps) share the K/V ring and each SIMD holds two waves
+template <int DH, int NCT> constexpr int QUERY_WAVES = (NCT == 2 && DH == 64) ? 8 : 4;
 // floats of per-wave scratch in the query pass: the two time-bias slabs [32][32] + [32][33]; the
 // channel tables of the set-up ([32 NCT][32]) and of the epilogue ([32][32 NCT + 1]) overlay them
 constexpr int WAVE_SCRATCH = 1024 + 32 * 33;
@@ -115,17 +118,18 @@ __device__ inline bf16x8 pack8(const f32x16& v, int base) {
 
 __device__ inline float xhalf_sum(float x) { return x + __shfl_xor(x, 32); }
 
-// chunk swizzles of a 128-byte row: row fragments / transposing reads (as in the forward)
-__device__ inline int swz_row(int row) { return (row >> 1) & 7; }
-__device__ inline int swz_tr(int row) { return ((row >> 1) & 1) << 2; }
+// chunk swizzles of a row of 2 DH bytes: row fragments / transposing reads (as in the forward)
+template <int DH> __device__ inline int swz_row(int row) { return DH == 64 ? ((row >> 1) & 7) : (row & 15); }
+template <int DH> __device__ inline int swz_tr(int row) { return DH == 64 ? (((row >> 1) & 1) << 2) : ((row & 3) << 2); }
 
-template <int NCT>
-__global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_args a, int q0, int k0, int accum) {
-  constexpr int NW = QUERY_WAVES<NCT>;
+template <int DH, int NCT>
+__global__ __launch_bounds__((QUERY_WAVES<DH, NCT> * 64)) void mvpa_bwd_query_mfma_kernel(mvpa_bwd_args a, int q0, int k0, int accum) {
+  constexpr int KS = DH / 16, MT = DH / 32, ROWB = 2 * DH, CPR = DH / 8;
+  constexpr int NW = QUERY_WAVES<DH, NCT>;
   constexpr int CP = NCT * 32, TQW = NW / NCT, TILE = CP * ROWB;
   static_assert(64 * 32 <= WAVE_SCRATCH && 32 * (CP + 1) <= WAVE_SCRATCH, "channel tables overlay the slabs");
-  constexpr int STAGES = QSTAGES, STAGE_BYTES = 3 * TILE;   // stage: V | K | K (transposing)
-  constexpr int LPW = CP / 8 / NW;                // 1 KiB wave loads per wave and tile copy
+  constexpr int STAGES = QSTAGES<DH, NCT>, STAGE_BYTES = 3 * TILE;   // stage: V | K | K (transposing)
+  constexpr int LPW = TILE / 1024 / NW;           // 1 KiB wave loads per wave and tile copy
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   float* wave_base = (float*)(smem + STAGES * STAGE_BYTES);
 
@@ -196,11 +200,11 @@ __global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_ker
 #pragma unroll
   for (int i = 0; i < LPW; ++i) {
     const int pc = (wave + NW * i) * 64 + lane;
-    const int r = pc >> 3, phys = pc & 7;
+    const int r = pc / CPR, phys = pc % CPR;
     const int rc = min(k0 + r, C_ - 1);           // key channels k0 .. of this launch
-    k_off_r[i] = rc * (int)a.k_stride_n + ((phys ^ swz_row(r)) << 3);
-    k_off_t[i] = rc * (int)a.k_stride_n + ((phys ^ swz_tr(r)) << 3);
-    v_off[i] = rc * (int)a.v_stride_n + ((phys ^ swz_row(r)) << 3);
+    k_off_r[i] = rc * (int)a.k_stride_n + ((phys ^ swz_row<DH>(r)) << 3);
+    k_off_t[i] = rc * (int)a.k_stride_n + ((phys ^ swz_tr<DH>(r)) << 3);
+    v_off[i] = rc * (int)a.v_stride_n + ((phys ^ swz_row<DH>(r)) << 3);
   }
   // first key step whose K is needed: the band of the earliest query step of the workgroup
   const int tk_near = !has_content ? tq_hi + 1 : (W <= 0 || tq_hi == T_ - 1) ? 0 : max(0, tq0 - W);
@@ -372,10 +376,10 @@ __global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_ker
     const int e = (ln & 15) >> 2, aa = ln & 3, grp = ln >> 4;
     const int row0 = 4 * hh + e;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) r_lane[ks] = ln * ROWB + (((2 * ks + hh) ^ swz_row(ln)) << 4);
+    for (int ks = 0; ks < KS; ++ks) r_lane[ks] = ln * ROWB + (((2 * ks + hh) ^ swz_row<DH>(ln)) << 4);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
-      t_lane[mt] = row0 * ROWB + (((4 * mt + 2 * grp + (aa >> 1)) ^ swz_tr(row0)) << 4) + ((aa & 1) << 3);
+      t_lane[mt] = row0 * ROWB + (((4 * mt + 2 * grp + (aa >> 1)) ^ swz_tr<DH>(row0)) << 4) + ((aa & 1) << 3);
   }
   auto tr_frag = [&](const unsigned char* tile_p, int t, int s, int mt) -> bf16x8 {
     const unsigned char* p = tile_p + t_lane[mt] + (32 * t + 16 * s) * ROWB;
@@ -645,7 +649,7 @@ __global__ __launch_bounds__(QUERY_WAVES<NCT> * 64) void mvpa_bwd_query_mfma_ker
 
 // 1 if the MFMA query pass can serve these (already validated) arguments
 int mvpa_bwd_query_mfma_supported(const mvpa_bwd_args* a) {
-  if (a->dtype != MVPA_BF16 || a->Dh != 64 || a->C > 128) return 0;
+  if (a->dtype != MVPA_BF16 || (a->Dh != 64 && a->Dh != 128) || a->C > 128) return 0;
   if (!(a->flags & MVPA_FLAG_CAUSAL) || a->key_bias || !a->ws_qu) return 0;
   const uintptr_t p = (uintptr_t)a->q | (uintptr_t)a->k | (uintptr_t)a->v | (uintptr_t)a->o |
                       (uintptr_t)a->d_o | (uintptr_t)a->bias_u | (uintptr_t)a->bias_v |
@@ -666,14 +670,14 @@ int mvpa_bwd_query_mfma_supported(const mvpa_bwd_args* a) {
   return 1;
 }
 
-template <int NCT>
+template <int DH, int NCT>
 static void launch_query(const mvpa_bwd_args* a, hipStream_t stream, int q0, int k0, int accum) {
   using namespace mvpa::bwdq;
-  constexpr int nw = QUERY_WAVES<NCT>, tqw = nw / NCT, cp = NCT * 32;
+  constexpr int nw = QUERY_WAVES<DH, NCT>, tqw = nw / NCT, cp = NCT * 32, ROWB = 2 * DH;
   const int nt = (a->T + tqw - 1) / tqw;
-  const size_t lds = (size_t)QSTAGES * 3 * cp * ROWB + (size_t)nw * WAVE_SCRATCH * sizeof(float);
+  const size_t lds = (size_t)QSTAGES<DH, NCT> * 3 * cp * ROWB + (size_t)nw * WAVE_SCRATCH * sizeof(float);
   dim3 grid((unsigned)(nt * a->B * a->H));
-  auto kern = mvpa_bwd_query_mfma_kernel<NCT>;
+  auto kern = mvpa_bwd_query_mfma_kernel<DH, NCT>;
   mvpa::want_dynamic_lds((const void*)kern, (int)lds);
   MVPA_LAUNCH(kern, grid, dim3(nw * 64), lds, stream, *a, q0, k0, accum);
 }
@@ -705,14 +709,15 @@ namespace bwdq {
 // SIMD holds two waves
 template <int NCT> constexpr int KEY_WAVES = NCT == 2 ? 8 : 4;
 
-template <int NCT, bool MASKED>
+template <int DH, int NCT, bool MASKED>
 __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(mvpa_bwd_args a, int k0, int q0, int accum) {
-  constexpr int NW = KEY_WAVES<NCT>;              // shadows the query pass's wave count
+  constexpr int KS = DH / 16, MT = DH / 32, ROWB = 2 * DH, CPR = DH / 8;
+  constexpr int NW = KEY_WAVES<NCT>;
   constexpr int CP = NCT * 32, KT = NW / NCT, TILE = CP * ROWB;
   constexpr int CS_BYTES = CP * CP * 4, SC_BYTES = (KT + 1) * 256;
   constexpr int STAGES = KSTAGES, STAGE_BYTES = 4 * TILE + CS_BYTES + SC_BYTES;
   static_assert(STAGES == 3, "the wait below counts the loads of exactly one younger step");
-  constexpr int LPW = CP / 8 / NW, CS_LPW = CS_BYTES / 1024 / NW;
+  constexpr int LPW = TILE / 1024 / NW, CS_LPW = CS_BYTES / 1024 / NW;
   // direct-to-LDS loads per wave and step
   constexpr int LPS_FAR = LPW + CS_LPW + 1, LPS_NEAR = 4 * LPW + CS_LPW + 2;
   // stage layout: dO (transposing) | Ec | scalars | dO (rows) | (q+u) (rows) | (q+u) (transposing)
@@ -765,12 +770,12 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
 #pragma unroll
   for (int i = 0; i < LPW; ++i) {
     const int pc = (wave + NW * i) * 64 + lane;
-    const int r = pc >> 3, phys = pc & 7;
+    const int r = pc / CPR, phys = pc % CPR;
     const int rc = min(q0 + r, C_ - 1);
-    q_off_r[i] = rc * DH + ((phys ^ swz_row(r)) << 3);
-    q_off_t[i] = rc * DH + ((phys ^ swz_tr(r)) << 3);
-    d_off_r[i] = rc * (int)a.do_stride_n + ((phys ^ swz_row(r)) << 3);
-    d_off_t[i] = rc * (int)a.do_stride_n + ((phys ^ swz_tr(r)) << 3);
+    q_off_r[i] = rc * DH + ((phys ^ swz_row<DH>(r)) << 3);
+    q_off_t[i] = rc * DH + ((phys ^ swz_tr<DH>(r)) << 3);
+    d_off_r[i] = rc * (int)a.do_stride_n + ((phys ^ swz_row<DH>(r)) << 3);
+    d_off_t[i] = rc * (int)a.do_stride_n + ((phys ^ swz_tr<DH>(r)) << 3);
   }
   // the Ec tile [C][C] lands with a row pitch of CP floats
 #pragma unroll
@@ -836,10 +841,10 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
     const int e = (ln & 15) >> 2, aa = ln & 3, grp16 = ln >> 4;
     const int row0 = 4 * hh + e;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) r_lane[ks] = ln * ROWB + (((2 * ks + hh) ^ swz_row(ln)) << 4);
+    for (int ks = 0; ks < KS; ++ks) r_lane[ks] = ln * ROWB + (((2 * ks + hh) ^ swz_row<DH>(ln)) << 4);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
-      t_lane[mt] = row0 * ROWB + (((4 * mt + 2 * grp16 + (aa >> 1)) ^ swz_tr(row0)) << 4) + ((aa & 1) << 3);
+      t_lane[mt] = row0 * ROWB + (((4 * mt + 2 * grp16 + (aa >> 1)) ^ swz_tr<DH>(row0)) << 4) + ((aa & 1) << 3);
   }
   auto tr_frag = [&](const unsigned char* tile_p, int qt, int s, int mt) -> bf16x8 {
     const unsigned char* p = tile_p + t_lane[mt] + (32 * qt + 16 * s) * ROWB;
@@ -1006,13 +1011,14 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
 }  // namespace bwdq
 }  // namespace mvpa
 
-template <int NCT, bool MASKED>
+template <int DH, int NCT, bool MASKED>
 static void launch_key(const mvpa_bwd_args* a, hipStream_t stream, int k0, int q0, int accum) {
   using namespace mvpa::bwdq;
-  constexpr int nw = KEY_WAVES<NCT>, cp = NCT * 32, kt = nw / NCT;
+  constexpr int nw = KEY_WAVES<NCT>, cp = NCT * 32, kt = nw / NCT, ROWB = 2 * DH;
+  static_assert((size_t)KSTAGES * (4 * cp * ROWB + cp * cp * 4 + (kt + 1) * 256) <= 160 * 1024, "key-pass ring exceeds the LDS");
   const size_t lds = (size_t)KSTAGES * (4 * cp * ROWB + cp * cp * 4 + (kt + 1) * 256);
   dim3 grid((unsigned)(((a->T + kt - 1) / kt) * a->B * a->Hkv));
-  auto kern = mvpa_bwd_key_mfma_kernel<NCT, MASKED>;
+  auto kern = mvpa_bwd_key_mfma_kernel<DH, NCT, MASKED>;
   mvpa::want_dynamic_lds((const void*)kern, (int)lds);
   MVPA_LAUNCH(kern, grid, dim3(nw * 64), lds, stream, *a, k0, q0, accum);
 }
@@ -1023,21 +1029,38 @@ static void launch_key(const mvpa_bwd_args* a, hipStream_t stream, int k0, int q
 // gradients) and of disjoint query channels (to dk, dv) simply add up, so every (query part, key
 // part) pair is one query-pass launch followed by the key-pass launch that consumes its
 // workspace; later launches add to what earlier ones wrote (one stream, hence ordered).
-int mvpa_launch_bwd_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
+// At Dh 128 a key-pass stage of 64 channels does not fit the LDS three times: the key pass then
+// takes the (query part, key part) pair of a query-pass launch in quarters of 32 x 32 channels
+// (the workspace is indexed by absolute channel, and its per-row maximum covers the whole key part).
+template <int DH>
+static void launch_bwd_parts(const mvpa_bwd_args* a, hipStream_t stream) {
   const int C = a->C;
+  constexpr int KEY_CP = DH == 64 ? 64 : 32;      // channels per key-pass launch
+  auto key_launches = [&](int q0, int k0, int span, bool first_q) {
+    for (int kk = k0; kk < min(k0 + span, C); kk += KEY_CP)
+      for (int qq = q0; qq < min(q0 + span, C); qq += KEY_CP) {
+        const int accum = !(first_q && qq == q0);
+        const bool full = C - qq >= KEY_CP && C - kk >= KEY_CP;
+        if (full) launch_key<DH, KEY_CP / 32, false>(a, stream, kk, qq, accum);
+        else launch_key<DH, KEY_CP / 32, true>(a, stream, kk, qq, accum);
+      }
+  };
   if (C <= 32) {
-    launch_query<1>(a, stream, 0, 0, 0);
-    if (C == 32) launch_key<1, false>(a, stream, 0, 0, 0);
-    else launch_key<1, true>(a, stream, 0, 0, 0);
+    launch_query<DH, 1>(a, stream, 0, 0, 0);
+    if (C == 32) launch_key<DH, 1, false>(a, stream, 0, 0, 0);
+    else launch_key<DH, 1, true>(a, stream, 0, 0, 0);
   } else {
     const int parts = (C + 63) / 64;
     for (int kp = 0; kp < parts; ++kp)
       for (int qp = 0; qp < parts; ++qp) {
-        const int q0 = qp * 64, k0 = kp * 64;
-        launch_query<2>(a, stream, q0, k0, kp > 0);
-        if (C - q0 >= 64 && C - k0 >= 64) launch_key<2, false>(a, stream, k0, q0, qp > 0);
-        else launch_key<2, true>(a, stream, k0, q0, qp > 0);
+        launch_query<DH, 2>(a, stream, qp * 64, kp * 64, kp > 0);
+        key_launches(qp * 64, kp * 64, 64, qp == 0);
       }
   }
+}
+
+int mvpa_launch_bwd_mfma(const mvpa_bwd_args* a, hipStream_t stream) {
+  if (a->Dh == 64) launch_bwd_parts<64>(a, stream);
+  else launch_bwd_parts<128>(a, stream);
   return mvpa::take_launch_status();
 }

@@ -116,12 +116,21 @@ BF16_CASES = [
     dict(B=1, C=32, T=21, H=2, Hkv=1, Dh=64, window=3),       # one channel tile, four key steps per workgroup, GQA
     dict(B=2, C=20, T=40, H=2, Hkv=2, Dh=64, window=5),       # one ragged channel tile, two slabs
     dict(B=1, C=64, T=45, H=1, Hkv=1, Dh=64, window=2),       # odd T: the last key pair of a workgroup is half empty
+    # head dim 128: rows of 256 bytes in the LDS tiles, the key pass in quarters of 32 x 32 channels
+    dict(B=1, C=32, T=21, H=2, Hkv=1, Dh=128, window=3),      # one channel tile, GQA
+    dict(B=2, C=20, T=40, H=2, Hkv=2, Dh=128, window=5),      # one ragged channel tile, two slabs
+    dict(B=1, C=64, T=12, H=2, Hkv=2, Dh=128, window=10),     # two channel tiles per query step, four key-pass launches
+    dict(B=1, C=40, T=37, H=2, Hkv=1, Dh=128, window=10),     # ragged second tile, two slabs, GQA
+    dict(B=1, C=117, T=9, H=2, Hkv=1, Dh=128, window=2),      # two channel parts: 4 query-pass, 16 key-pass launches
+    dict(B=1, C=128, T=6, H=1, Hkv=1, Dh=128, window=10),     # two full channel parts
+    dict(B=2, C=65, T=35, H=2, Hkv=2, Dh=128, window=3),      # second part of one channel; two slabs
+    dict(B=1, C=33, T=9, H=2, Hkv=2, Dh=128, window=0),       # content everywhere; odd C
 ]
 
 
-@pytest.mark.parametrize("case", BF16_CASES, ids=lambda c: "B{B}C{C}T{T}H{H}g{Hkv}w{window}".format(**c))
+@pytest.mark.parametrize("case", BF16_CASES, ids=lambda c: "B{B}C{C}T{T}H{H}g{Hkv}D{Dh}w{window}".format(**c))
 def test_backward_bf16_mfma_query_pass(case):
-    """bf16, Dh = 64, C <= 128 takes the MFMA passes (dq, dk, dv, bias-table gradients)."""
+    """bf16, Dh = 64 or 128, C <= 128 takes the MFMA passes (dq, dk, dv, bias-table gradients)."""
     cfg = dict(case)
     window = cfg.pop("window")
     inp = make_mvpa_inputs(seed=13, qkv_unit=True, **cfg).round_to(torch.bfloat16)
@@ -175,8 +184,12 @@ def test_backward_bf16_mfma_rows_are_causal():
     assert got["q"][:, :, 3 * 32:].abs().max().item() == 0.0
 
 
-def test_backward_bf16_full_size_invariants():
-    """At the benchmark shape (B4 C64 T128 H16 Dh64, too large for the float64 oracle) the
+@pytest.mark.parametrize("cfg", [dict(B=4, C=64, T=128, H=16, Hkv=16, Dh=64),
+                                 dict(B=1, C=128, T=128, H=4, Hkv=2, Dh=128)],
+                         ids=["c2", "C128-Dh128-GQA"])
+def test_backward_bf16_full_size_invariants(cfg):
+    """At the benchmark shape (B4 C64 T128 H16 Dh64, too large for the float64 oracle) and at the
+    base model's channels, head dim and head grouping (C128 Dh128, two query heads per kv head) the
     gradients must satisfy what the softmax fixes for ANY d_o:
       * dS rows sum to zero, so every row of dbias_time and of dbias_chan sums to zero
         (up to the bf16 rounding of the probabilities: <= 1e-2 of the absolute sum of the row of
@@ -184,7 +197,6 @@ def test_backward_bf16_full_size_invariants():
       * with d_o = 1 the columns of dv are the column sums of P, so dv summed over the keys of a
         (batch, kv head) equals the number of queries of the group's heads, N * H/Hkv."""
     import mvpa_hip
-    cfg = dict(B=4, C=64, T=128, H=16, Hkv=16, Dh=64)
     inp = make_mvpa_inputs(seed=0, **cfg).to("cuda", torch.bfloat16)
     out, lse = mvpa_hip.mvpa_forward(inp.q, inp.k, inp.v, inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan,
                                      return_lse=True)
