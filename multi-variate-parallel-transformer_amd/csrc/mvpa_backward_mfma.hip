@@ -699,7 +699,7 @@ static void launch_query(const mvpa_bwd_args* a, hipStream_t stream, int q0, int
 // swizzle, (q+u) * scale in both swizzles and delta; direct-to-LDS loads fetch it two steps
 // ahead.  The query steps are walked from the last one down and the workgroups of one
 // (b, kv head) sit on one XCD: they then read the same stage data at about the same time and
-// share it in L2.  MASKED: C is not a multiple of 32, padded query rows and key lanes are cut.
+// share it in L2.  MASKED: the query part holds fewer channels than its tiles, padded query rows are cut.
 // ==========================================================================================
 namespace mvpa {
 namespace bwdq {
@@ -754,7 +754,28 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
 
   const int ck = k0 + kt * 32 + ln;               // key channels k0 .., query channels q0 .. in this launch
   const int ckl = kt * 32 + ln;                   // ... local to the launch
-  const bool key_live = ck < C_;                  // invalid channels have Ec = 0 already
+  // Lanes of key channels beyond C own columns of dk / dv that are never stored, and a product's
+  // column depends on no other lane's operand: they need no masking.  Padded QUERY rows are the
+  // contraction index of both gradient products; their probabilities are cut after packing, with
+  // one mask per fragment dword (two queries) kept in registers (per-element predicates were
+  // hoisted out of the loop as 32 lane masks and spilled the scalar registers).
+  uint32_t qmask[NCT][8];
+#pragma unroll
+  for (int qt = 0; qt < NCT; ++qt)
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+      const int i = 2 * w;                        // elements i, i + 1 of the tile: queries qa, qa + 1
+      const int qa = q0 + qt * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
+      qmask[qt][w] = MASKED ? ((qa < C_ ? 0x0000ffffu : 0u) | (qa + 1 < C_ ? 0xffff0000u : 0u)) : 0xffffffffu;
+    }
+  auto cut = [&](bf16x8 f, int qt, int s) -> bf16x8 {
+    if (!MASKED) return f;
+    union { bf16x8 b; u32x4 u; } c;
+    c.b = f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) c.u[w] &= qmask[qt][4 * s + w];
+    return c.b;
+  };
   const int64_t nk = (int64_t)tkc * C_ + min(ck, C_ - 1);
   const bf16_t* krow = (const bf16_t*)a.k + b * a.k_stride_b + g * a.k_stride_h + nk * a.k_stride_n;
   const bf16_t* vrow = (const bf16_t*)a.v + b * a.v_stride_b + g * a.v_stride_h + nk * a.v_stride_n;
@@ -905,13 +926,12 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
         const float es[4] = {e4.x, e4.y, e4.z, e4.w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float p = Ecs[(rb + j) * CP] * es[j];
-          P[a4 * 4 + j] = (!MASKED || (key_live && q0 + rb + j < C_)) ? p : 0.f;
+          P[a4 * 4 + j] = Ecs[(rb + j) * CP] * es[j];
         }
       }
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        const bf16x8 pf = pack8(P, 8 * s);
+        const bf16x8 pf = cut(pack8(P, 8 * s), qt, s);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
           dV[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Dtr, qt, s, mt), pf, dV[mt], 0, 0, 0);
@@ -948,16 +968,15 @@ __global__ __launch_bounds__(KEY_WAVES<NCT> * 64) void mvpa_bwd_key_mfma_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int i = a4 * 4 + j;
-          float p = __builtin_amdgcn_exp2f(S[i] + tls[j]) * Ecs[(rb + j) * CP];
-          if (MASKED) p = (key_live && q0 + rb + j < C_) ? p : 0.f;
+          const float p = __builtin_amdgcn_exp2f(S[i] + tls[j]) * Ecs[(rb + j) * CP];
           S[i] = p;
           dS[i] = p * (dP[i] - des[j]) * (1.f / kLog2e);
         }
       }
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        const bf16x8 pf = pack8(S, 8 * s);
-        const bf16x8 sf = pack8(dS, 8 * s);
+        const bf16x8 pf = cut(pack8(S, 8 * s), qt, s);
+        const bf16x8 sf = cut(pack8(dS, 8 * s), qt, s);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           dV[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Dtr, qt, s, mt), pf, dV[mt], 0, 0, 0);
