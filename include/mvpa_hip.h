@@ -43,8 +43,10 @@ enum {
 enum {
   MVPA_F32 = 0,   /* fp32 in, fp32 math, fp32 out                                   */
   MVPA_BF16 = 1,  /* bf16 in/out, bf16 MFMA with fp32 accumulation                  */
-  MVPA_F16 = 2    /* fp16 in/out, fp32 math: forward only, on the row-per-lane kernel
-                     (the reference's kernel takes fp16 or bf16, attentions/attn.py:1064-1066) */
+  MVPA_F16 = 2    /* fp16 in/out, forward only: fp16 MFMA with fp32 accumulation on the general
+                     tiled kernel (the shapes and alignment the bf16 MFMA kernel takes), fp32 math
+                     on the row-per-lane kernel otherwise (the reference's kernel takes fp16 or
+                     bf16, attentions/attn.py:1064-1066) */
 };
 
 /* ---- kernel selector --------------------------------------------------------------- */

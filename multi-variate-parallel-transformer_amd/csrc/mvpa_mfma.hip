@@ -1,4 +1,4 @@
-// Tiled bf16 MFMA kernel for the MVPA forward on gfx950 (CDNA4, wave64).
+// Tiled MFMA kernel (bf16, or fp16 through the element-type parameter E) for the MVPA forward on gfx950 (CDNA4, wave64).
 //
 // Tokens are a T x C grid (n = t*C + c).  Both queries and keys are tiled BY TIME STEP: a key
 // tile is the C keys of one time step tk (channels padded to CP = 32/64/128), a query block is
@@ -66,8 +66,11 @@ struct Cfg {
   static_assert(WLOADS % NW == 0 || WLOADS < NW, "every loading wave issues the same number of loads");
 };
 
-template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8, int KH, bool RUNS>
+template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8, int KH, bool RUNS, typename E>
 __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args a) {
+  using x8 = typename E::x8;                     // fragments of the element type (bf16 or fp16)
+  using x4 = typename E::x4;
+  using x2 = typename E::x2;
   using G = Cfg<DH, NCT, NW, STAGES, KH>;
   constexpr int CP = G::CP, KS = G::KS, MT = G::MT, ROWB = G::ROWB, CHUNKS = G::CHUNKS;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
@@ -235,7 +238,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   // fragments are needed once per 32-step slab only and are re-formed there from q (an L2 hit)
   // instead of kept in registers.
   constexpr bool LEAN = KS * NCT > 8;
-  bf16x8 Qu[KS];                        // (q+u) * scale as QK^T B operand
+  x8 Qu[KS];                        // (q+u) * scale as QK^T B operand
   // fp8 content term: q' = (q+u)*scale/sq and k' = k/sk are rounded to e4m3 with the per-head
   // amax scales sq, sk chosen by the caller; the MFMA accumulates in units of 1/(sq*sk), the
   // channel-bias tile is pre-divided accordingly and the product sq*sk returns inside the exp2 fma
@@ -262,15 +265,15 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d0 = ks * 16 + hh * 8;
-      Qu[ks] = make_qfrag(raw[ks], bu + d0, sc2);
+      Qu[ks] = E::qfrag(raw[ks], bu + d0, sc2);
       if (FP8) Qu8[ks] = make_qfrag_fp8(raw[ks], bu + d0, sc2 / a.fp8_q_scale[h]);
-      if (SLAB_LDS && G::EARLY && slab_lds) *(bf16x8*)(qv_lds + ks * 1024) = make_qfrag(raw[ks], bv + d0, sc2);
-      const bf16x8 qz = make_qfrag(raw[ks], bz + d0, sc2);
+      if (SLAB_LDS && G::EARLY && slab_lds) *(x8*)(qv_lds + ks * 1024) = E::qfrag(raw[ks], bv + d0, sc2);
+      const x8 qz = E::qfrag(raw[ks], bz + d0, sc2);
 #pragma unroll
       for (int t = 0; t < G::QT; ++t) {
         const int j = min(t * 32 + ln, C_ - 1);
         const u32x4 er = *(const u32x4*)(kchan + (int64_t)j * DH + d0);
-        sct[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(er), qz, sct[t], 0, 0, 0);
+        sct[t] = E::mfma(E::as8(er), qz, sct[t], 0, 0, 0);
       }
     }
     float* scr = setup_all + wave * (CP * 32);
@@ -320,7 +323,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
   }
 
   float mc, sumEc;
-  bf16x8 Ec[NCT][2];         // exp2(Bc - mc) as PV B-operand fragments
+  x8 Ec[NCT][2];         // exp2(Bc - mc) as PV B-operand fragments
   {
     float mx = -INFINITY;
 #pragma unroll
@@ -340,8 +343,8 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
         e[i] = fast_exp2(Bc[t][i] - mc);
         se += e[i];
       }
-      Ec[t][0] = pack8(e, 0);
-      Ec[t][1] = pack8(e, 8);
+      Ec[t][0] = E::pack(e, 0);
+      Ec[t][1] = E::pack(e, 8);
     }
     sumEc = se;               // partial: this half-wave's keys only
   }
@@ -375,7 +378,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d0 = ks * 16 + hh * 8;
-      *(bf16x8*)(qv_lds + ks * 1024) = make_qfrag(*(const u32x4*)(qrow + d0), bv + d0, sc2);
+      *(x8*)(qv_lds + ks * 1024) = E::qfrag(*(const u32x4*)(qrow + d0), bv + d0, sc2);
     }
   }
 
@@ -401,10 +404,10 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) k_lane[ks] = ln * ROWB + (((2 * ks + hh) ^ swz_k<DH>(ln)) << 4);
   }
-  auto v_frag = [&](const unsigned char* stage, int t, int s, int mt) -> bf16x8 {
+  auto v_frag = [&](const unsigned char* stage, int t, int s, int mt) -> x8 {
     const unsigned char* p = stage + v_lane[mt] + (32 * t + 16 * s) * ROWB;
-    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((LDS_PTR(bf16x4))p);
-    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((LDS_PTR(bf16x4))(p + 8 * ROWB));
+    const x4 lo = E::read_tr(p);
+    const x4 hi = E::read_tr(p + 8 * ROWB);
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
 
@@ -422,9 +425,9 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
       const int sw = swz_k<DH>(row);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const bf16x8 rr = *(const bf16x8*)(rp + (((2 * ks + hh) ^ sw) << 4));
-        const bf16x8 qv = *(const bf16x8*)(qv_lds + ks * 1024);
-        stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rr, qv, stc, 0, 0, 0);
+        const x8 rr = *(const x8*)(rp + (((2 * ks + hh) ^ sw) << 4));
+        const x8 qv = *(const x8*)(qv_lds + ks * 1024);
+        stc = E::mfma(rr, qv, stc, 0, 0, 0);
       }
     } else if (has_time) {
       int j = min(j0 + ln, T_ - 1);                // rows past T-1 belong to tk > tq: never used
@@ -432,8 +435,8 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const u32x4 rr = *(const u32x4*)(ktime + (int64_t)j * DH + ks * 16 + hh * 8);
-        const bf16x8 qv = make_qfrag(*(const u32x4*)(qrow + ks * 16 + hh * 8), bv + ks * 16 + hh * 8, sc2);
-        stc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(rr), qv, stc, 0, 0, 0);
+        const x8 qv = E::qfrag(*(const u32x4*)(qrow + ks * 16 + hh * 8), bv + ks * 16 + hh * 8, sc2);
+        stc = E::mfma(E::as8(rr), qv, stc, 0, 0, 0);
       }
     }
     float cm = -INFINITY;
@@ -471,7 +474,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
       for (int s = 0; s < 2; ++s)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-          tmp[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(stage, t, s, mt), Ec[t][s], tmp[mt], 0, 0, 0);
+          tmp[mt] = E::mfma(v_frag(stage, t, s, mt), Ec[t][s], tmp[mt], 0, 0, 0);
     const float et = fast_exp2(st + mc - m_run);
     l_run += et * sumEc;
 #pragma unroll
@@ -527,32 +530,32 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
     } else {
       if (!LEAN) {
         // every K fragment of the step is requested before the first MFMA waits for one
-        bf16x8 ka[KS][NCT];
+        x8 ka[KS][NCT];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-          for (int t = 0; t < NCT; ++t) ka[ks][t] = *(const bf16x8*)(stage + k_lane[ks] + t * 32 * ROWB);
+          for (int t = 0; t < NCT; ++t) ka[ks][t] = *(const x8*)(stage + k_lane[ks] + t * 32 * ROWB);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < NCT; ++t)
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks)
-            S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][t], Qu[ks], S[t], 0, 0, 0);
+            S[t] = E::mfma(ka[ks][t], Qu[ks], S[t], 0, 0, 0);
       } else {
 #pragma unroll
         for (int t = 0; t < NCT; ++t) {
-          bf16x8 ka[KS];
+          x8 ka[KS];
 #pragma unroll
-          for (int ks = 0; ks < KS; ++ks) ka[ks] = *(const bf16x8*)(stage + k_lane[ks] + t * 32 * ROWB);
+          for (int ks = 0; ks < KS; ++ks) ka[ks] = *(const x8*)(stage + k_lane[ks] + t * 32 * ROWB);
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks)
-            S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], Qu[ks], S[t], 0, 0, 0);
+            S[t] = E::mfma(ka[ks], Qu[ks], S[t], 0, 0, 0);
         }
       }
     }
     // V^T fragments of one key tile, [s][mt]; PREFETCH: requested a tile ahead of their use
     constexpr bool PREFETCH = !LEAN;
-    bf16x8 vf[2][MT];
+    x8 vf[2][MT];
     if (PREFETCH) {
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -585,20 +588,20 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 #pragma unroll
       for (int i = 0; i < 16; ++i)
         S[t][i] = FP8 ? fast_exp2(__builtin_fmaf(S[t][i], fp8_d, off)) : fast_exp2(S[t][i] + off);
-      bf16x8 P[2];
-      P[0] = pack8(S[t], 0);
-      P[1] = pack8(S[t], 8);
+      x8 P[2];
+      P[0] = E::pack(S[t], 0);
+      P[1] = E::pack(S[t], 8);
       // the row sum is taken over the bf16 probabilities the PV product uses, two per
       // instruction (v_dot2c_f32_bf16 against a pair of ones), accumulated in fp32
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        union { bf16x8 v; bf16x2 q[4]; } u;
+        union { x8 v; x2 q[4]; } u;
         u.v = P[s];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) ls = __builtin_amdgcn_fdot2_f32_bf16(u.q[j], kOnes2, ls, false);
+        for (int j = 0; j < 4; ++j) ls = E::add_pair(u.q[j], ls);
       }
       if (PREFETCH) {
-        bf16x8 vn[2][MT];
+        x8 vn[2][MT];
         if (t + 1 < NCT) {
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -611,7 +614,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
         for (int s = 0; s < 2; ++s)
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[s][mt], P[s], acc[mt], 0, 0, 0);
+            acc[mt] = E::mfma(vf[s][mt], P[s], acc[mt], 0, 0, 0);
         if (t + 1 < NCT) {
 #pragma unroll
           for (int s = 0; s < 2; ++s)
@@ -623,7 +626,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
         for (int s = 0; s < 2; ++s)
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(stage, t, s, mt), P[s], acc[mt], 0, 0, 0);
+            acc[mt] = E::mfma(v_frag(stage, t, s, mt), P[s], acc[mt], 0, 0, 0);
       }
     }
     l_run += ls;
@@ -699,7 +702,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
           const float st = Stb[(tk & 31) * 32 + ln];
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
-            bf16x8 vf[NCT * 2];
+            x8 vf[NCT * 2];
 #pragma unroll
             for (int t = 0; t < NCT; ++t)
 #pragma unroll
@@ -713,7 +716,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
             for (int t = 0; t < NCT; ++t)
 #pragma unroll
               for (int s2 = 0; s2 < 2; ++s2)
-                ptmp[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[t * 2 + s2], Ec[t][s2], ptmp[mt], 0, 0, 0);
+                ptmp[mt] = E::mfma(vf[t * 2 + s2], Ec[t][s2], ptmp[mt], 0, 0, 0);
           }
           pet = fast_exp2(st + mc - m_run);
           l_run += pet * sumEc;
@@ -797,10 +800,10 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 #pragma unroll
         for (int a4 = 0; a4 < 4; ++a4) {
           const int d0 = mt * 32 + a4 * 8 + hh * 4;
-          bf16x4 w;
+          x4 w;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) w[r] = (__bf16)(acc[mt][a4 * 4 + r] * inv);
-          *(bf16x4*)(orow + d0) = w;
+          for (int r = 0; r < 4; ++r) w[r] = E::cvt(acc[mt][a4 * 4 + r] * inv);
+          *(x4*)(orow + d0) = w;
         }
       if (n_split > 1) {
         float* plse = (float*)((bf16_t*)a.split_ws + (int64_t)n_split * nbh * C_ * DH);
@@ -814,8 +817,9 @@ __global__ __launch_bounds__(NW * 64, MINB) void mvpa_mfma_kernel(mvpa_fwd_args 
 
 // Combines the runs of a split last-step launch: out = sum_r 2^(lse_r - lse) o_r with
 // lse = log2 sum_r 2^lse_r.  DH/8 lanes per output row, 16 bytes each.
-template <int DH>
+template <int DH, typename E>
 __global__ __launch_bounds__(256) void mvpa_split_merge_kernel(mvpa_fwd_args a) {
+  using x8 = typename E::x8;
   constexpr int LPR = DH / 8, RPB = 256 / LPR;         // lanes per row (8 elements each), rows per block
   const int sub = threadIdx.x % LPR;
   const int nbh = a.B * a.H, C_ = a.C, rows = nbh * C_;
@@ -831,20 +835,20 @@ __global__ __launch_bounds__(256) void mvpa_split_merge_kernel(mvpa_fwd_args a) 
   for (int r = 0; r < a.n_split; ++r) {
     const float w = fast_exp2(plse[(int64_t)r * rows + row] - m);
     l += w;
-    const bf16x8 v = *(const bf16x8*)(po + ((int64_t)r * rows + row) * DH + 8 * sub);
+    const x8 v = *(const x8*)(po + ((int64_t)r * rows + row) * DH + 8 * sub);
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] += w * (float)v[i];
   }
   const int bh = row / C_, cq = row % C_, b = bh / a.H, h = bh % a.H;
   const float inv = 1.f / l;
-  bf16x8 w8;
+  x8 w8;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) w8[i] = (__bf16)(acc[i] * inv);
-  *(bf16x8*)((bf16_t*)a.o + b * a.o_stride_b + h * a.o_stride_h + (int64_t)cq * a.o_stride_n + 8 * sub) = w8;
+  for (int i = 0; i < 8; ++i) w8[i] = E::cvt(acc[i] * inv);
+  *(x8*)((bf16_t*)a.o + b * a.o_stride_b + h * a.o_stride_h + (int64_t)cq * a.o_stride_n + 8 * sub) = w8;
   if (a.lse && sub == 0) a.lse[row] = m + log2f(l);
 }
 
-template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8, int KH>
+template <int DH, int NCT, int NW, int STAGES, int MINB, bool FP8, int KH, typename E>
 static int launch_one(const mvpa_fwd_args* a, hipStream_t stream) {
   using G = Cfg<DH, NCT, NW, STAGES, KH>;
   static_assert(KH <= 2 && (KH == 1 || G::TQW * G::QT * (2 + G::MT * 16) * 256 <= G::RING_BYTES), "merge buffer");
@@ -855,29 +859,31 @@ static int launch_one(const mvpa_fwd_args* a, hipStream_t stream) {
   const bool content = a->flags & MVPA_FLAG_CONTENT;
   if (ring && !content) return MVPA_ERR_UNSUPPORTED;      // the run build has no far path
   if (!content) n_split = 1;
-  auto kern = (n_split > 1 || ring) ? mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH, true>
-                          : mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH, false>;
+  auto kern = (n_split > 1 || ring) ? mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH, true, E>
+                          : mvpa_mfma_kernel<DH, NCT, NW, STAGES, MINB, FP8, KH, false, E>;
   mvpa::want_dynamic_lds((const void*)kern, (int)G::LDS_BYTES);
   const int nt = (G::TQW == 2 && STAGES == 4 && KH == 1) ? 1 + a->T / 2 : (a->T + G::TQW - 1) / G::TQW;   // as in the kernel
   dim3 grid((unsigned)((last ? n_split : nt) * a->B * a->H));
   MVPA_LAUNCH(kern, grid, dim3(G::THREADS), G::LDS_BYTES, stream, *a);
   if (n_split > 1) {
     const int rows = a->B * a->H * a->C;
-    MVPA_LAUNCH(mvpa_split_merge_kernel<DH>, dim3((unsigned)((rows + 2048 / DH - 1) / (2048 / DH))), dim3(256), 0, stream, *a);
+    MVPA_LAUNCH((mvpa_split_merge_kernel<DH, E>), dim3((unsigned)((rows + 2048 / DH - 1) / (2048 / DH))), dim3(256), 0, stream, *a);
   }
   return mvpa::take_launch_status();
 }
 
 template <int DH, int NCT, int NW, int STAGES, int MINB = 1, int KH = 1>
 static int launch_cfg(const mvpa_fwd_args* a, hipStream_t stream) {
-  if (a->flags & MVPA_FLAG_FP8_QK) return launch_one<DH, NCT, NW, STAGES, MINB, true, KH>(a, stream);
-  return launch_one<DH, NCT, NW, STAGES, MINB, false, KH>(a, stream);
+  if (a->dtype == MVPA_F16) return launch_one<DH, NCT, NW, STAGES, MINB, false, KH, el_f16>(a, stream);
+  if (a->flags & MVPA_FLAG_FP8_QK) return launch_one<DH, NCT, NW, STAGES, MINB, true, KH, el_bf16>(a, stream);
+  return launch_one<DH, NCT, NW, STAGES, MINB, false, KH, el_bf16>(a, stream);
 }
 
 }  // namespace mvpa
 
 int mvpa_mfma_supported(const mvpa_fwd_args* a) {
-  if (a->dtype != MVPA_BF16) return 0;
+  if (a->dtype != MVPA_BF16 && a->dtype != MVPA_F16) return 0;
+  if (a->dtype == MVPA_F16 && (a->flags & MVPA_FLAG_FP8_QK)) return 0;
   if (!(a->flags & MVPA_FLAG_CAUSAL)) return 0;
   if (a->key_bias) return 0;
   if (a->C > 128) return 0;

@@ -674,7 +674,7 @@ __global__ __launch_bounds__(NW * 64) void mvpa_mfma128_kernel(mvpa_fwd_args a) 
 // forward (no decoding step), bf16 or fp8 content term; everything else about the arguments is as
 // for the general kernel (mvpa_mfma_supported).
 int mvpa_mfma128_supported(const mvpa_fwd_args* a) {
-  if ((a->Dh != 128 && a->Dh != 64) || a->C <= 32 || a->C > 128) return 0;
+  if (a->dtype != MVPA_BF16 || (a->Dh != 128 && a->Dh != 64) || a->C <= 32 || a->C > 128) return 0;
   if (a->flags & (MVPA_FLAG_LAST_STEP | MVPA_FLAG_RING)) return 0;
   // the fp8 content term streams the keys' e4m3 copy (the general kernel rounds bf16 keys itself)
   if ((a->flags & MVPA_FLAG_FP8_QK) && (!a->k_fp8 || ((uintptr_t)a->k_fp8 & 15))) return 0;

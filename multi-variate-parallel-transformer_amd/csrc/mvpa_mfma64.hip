@@ -714,7 +714,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mvpa_mfma64_kernel(mvpa_fwd_args a
 // (no decoding step, no fp8 content term); everything else about the arguments is as for the
 // general kernel (mvpa_mfma_supported).
 int mvpa_mfma64_supported(const mvpa_fwd_args* a) {
-  if (a->Dh != 64 || a->C <= 32 || a->C > 64) return 0;
+  if (a->dtype != MVPA_BF16 || a->Dh != 64 || a->C <= 32 || a->C > 64) return 0;
   if (a->flags & (MVPA_FLAG_LAST_STEP | MVPA_FLAG_RING | MVPA_FLAG_FP8_QK)) return 0;
   return 1;
 }

@@ -1,4 +1,4 @@
-// Device helpers shared by the tiled bf16 MFMA forward kernels (gfx950, wave64): vector types,
+// Device helpers shared by the tiled MFMA forward kernels (gfx950, wave64): vector types,
 // LDS-direct tile loads, wait counters, fragment packing, the XOR swizzles of the K / V rows.
 #pragma once
 
@@ -146,6 +146,69 @@ __device__ inline bf16x8 pack8(const f32x16& v, int base) {
   for (int i = 0; i < 8; ++i) out[i] = (__bf16)v[base + i];
   return out;
 }
+
+// ---- element types of the general tiled kernel --------------------------------------------
+// The 16-bit storage type of q, k, v, the tables and the output: what differs between bf16 and
+// fp16 is the MFMA instruction, the conversions from and to fp32, and the pair-sum instruction.
+// Pointers stay 2-byte element pointers (bf16_t) in either case.
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+
+struct el_bf16 {
+  using x8 = bf16x8;
+  using x4 = bf16x4;
+  using x2 = bf16x2;
+  static __device__ inline f32x16 mfma(x8 a, x8 b, f32x16 c, int, int, int) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ inline x8 qfrag(u32x4 raw, const bf16_t* __restrict__ bias, float scale) { return make_qfrag(raw, bias, scale); }
+  static __device__ inline x8 as8(u32x4 v) { return as_bf16x8(v); }
+  static __device__ inline x8 pack(const f32x16& v, int base) { return pack8(v, base); }
+  static __device__ inline float add_pair(x2 p, float acc) { return __builtin_amdgcn_fdot2_f32_bf16(p, kOnes2, acc, false); }
+  static __device__ inline x4 read_tr(const unsigned char* p) { return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((LDS_PTR(bf16x4))p); }
+  static __device__ inline __bf16 cvt(float f) { return (__bf16)f; }
+};
+
+struct el_f16 {
+  using x8 = f16x8;
+  using x4 = f16x4;
+  using x2 = f16x2;
+  static __device__ inline f32x16 mfma(x8 a, x8 b, f32x16 c, int, int, int) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  // 8 fp16 of a q row + bias, scaled, back to an fp16 fragment
+  static __device__ inline x8 qfrag(u32x4 raw, const bf16_t* __restrict__ bias, float scale) {
+    union { u32x4 u; x8 h; } r, b;
+    r.u = raw;
+    b.u = *(const u32x4*)bias;
+    x8 out;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = (_Float16)(((float)r.h[i] + (float)b.h[i]) * scale);
+    return out;
+  }
+  static __device__ inline x8 as8(u32x4 v) {
+    union { u32x4 u; x8 h; } c;
+    c.u = v;
+    return c.h;
+  }
+  static __device__ inline x8 pack(const f32x16& v, int base) {
+    x8 out;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = (_Float16)v[base + i];
+    return out;
+  }
+  static __device__ inline float add_pair(x2 p, float acc) {
+    return __builtin_amdgcn_fdot2(p, f16x2{(_Float16)1.0f, (_Float16)1.0f}, acc, false);
+  }
+  // the transposing read moves 16-bit units whatever they hold
+  static __device__ inline x4 read_tr(const unsigned char* p) {
+    union { bf16x4 b; x4 h; } c;
+    c.b = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((LDS_PTR(bf16x4))p);
+    return c.h;
+  }
+  static __device__ inline _Float16 cvt(float f) { return (_Float16)f; }
+};
 
 // XOR swizzles of the 16-byte chunk index within a K / V row, chosen so that the lanes that
 // read LDS together (16 consecutive rows at one chunk for K; 4 consecutive rows x 4 chunks for

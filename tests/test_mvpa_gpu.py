@@ -162,18 +162,15 @@ def test_masks_are_exact_under_perturbation():
 @pytest.mark.parametrize("cfg", [dict(B=2, C=8, T=32, H=4, Dh=32), dict(B=1, C=20, T=14, H=2, Hkv=1, Dh=64, validity=True),
                                  dict(B=1, C=5, T=13, H=2, Dh=128)])
 def test_fp16_io_on_the_fp32_math_kernel(cfg):
-    """fp16 tensors (the reference's kernel takes fp16 or bf16, attentions/attn.py:1064-1066) run
-    on the fp32-math kernel: inputs rounded to fp16, fp32 arithmetic, one rounding of the output.
+    """fp16 tensors (the reference's kernel takes fp16 or bf16, attentions/attn.py:1064-1066) on
+    the fp32-math kernel: inputs rounded to fp16, fp32 arithmetic, one rounding of the output.
     Tolerance: max-abs 2e-3 against the oracle on the same rounded inputs; the log-sum-exp 1e-4."""
     inp = make_mvpa_inputs(seed=5, table_std=0.3, qkv_unit=True, **cfg).round_to(torch.float16)
-    out, lse = _gpu(inp, torch.float16, return_lse=True)
+    out, lse = _gpu(inp, torch.float16, return_lse=True, kernel=mvpa_hip.KERNEL_GENERIC)
     assert out.dtype == torch.float16
     ref, ref_lse = _oracle(inp, return_lse=True)
     assert (out.float().cpu().double() - ref).abs().max().item() <= 2e-3
     assert (lse.cpu().double() - ref_lse).abs().max().item() <= 1e-4
-    d = inp.to("cuda", torch.float16)
-    with pytest.raises(mvpa_hip.MvpaError):            # no matrix-core build for fp16
-        mvpa_hip.mvpa_forward(d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan, kernel=mvpa_hip.KERNEL_MFMA)
 
 
 MFMA_SHAPES = [
@@ -218,6 +215,46 @@ def test_bf16_mfma_shapes(cfg):
     ref, ref_lse = _oracle(inp, return_lse=True)
     _check_bf16(out, ref)
     assert (lse.cpu().double() - ref_lse).abs().max().item() <= 3e-2
+
+
+FP16_MAX_ABS, FP16_REL_L2, FP16_LSE = 5e-4, 1e-3, 1e-3
+
+
+@pytest.mark.parametrize("cfg", MFMA_SHAPES)
+def test_fp16_mfma_shapes(cfg):
+    """fp16 tensors on the matrix cores (the general tiled kernel with the fp16 MFMA; the
+    reference's kernel takes fp16 or bf16, attentions/attn.py:1064-1066).  Probabilities and the
+    far steps' channel factors pass through fp16 (11 significant bits) where the bf16 build has 8,
+    so the tolerance against the oracle on the same fp16-rounded inputs is tighter than bf16's:
+    max-abs 5e-4, rel-L2 1e-3, log-sum-exp 1e-3 (measured over these shapes: 1.5e-4, 2.9e-4,
+    2.5e-4)."""
+    inp = make_mvpa_inputs(seed=21, table_std=0.3, qkv_unit=True, **cfg).round_to(torch.float16)
+    out, lse = _gpu(inp, torch.float16, kernel=mvpa_hip.KERNEL_MFMA, return_lse=True)
+    assert out.dtype == torch.float16
+    ref, ref_lse = _oracle(inp, return_lse=True)
+    o = out.float().cpu()
+    err, rel = (o - ref.float()).abs().max().item(), _rel_l2(o, ref.float())
+    assert err <= FP16_MAX_ABS and rel <= FP16_REL_L2, f"max-abs {err:.3e}, rel-L2 {rel:.3e}"
+    assert (lse.cpu().double() - ref_lse).abs().max().item() <= FP16_LSE
+
+
+def test_fp16_dispatch_and_what_it_refuses():
+    """fp16 under the default selector takes the matrix-core kernel (bit for bit the forced
+    launch); the specialised bf16 builds and the fp8 content term refuse fp16 tensors."""
+    cfg = dict(B=1, C=64, T=140, H=2, Dh=64)
+    d = make_mvpa_inputs(seed=2, qkv_unit=True, **cfg).to("cuda", torch.float16)
+    args = (d.q, d.k, d.v, d.u, d.vb, d.z, d.k_time, d.k_chan)
+    auto = mvpa_hip.mvpa_forward(*args)
+    forced = mvpa_hip.mvpa_forward(*args, kernel=mvpa_hip.KERNEL_MFMA)
+    assert torch.equal(auto, forced)
+    generic = mvpa_hip.mvpa_forward(*args, kernel=mvpa_hip.KERNEL_GENERIC)
+    assert not torch.equal(auto, generic)
+    assert (auto.float() - generic.float()).abs().max().item() <= FP16_MAX_ABS
+    for kern in (mvpa_hip.KERNEL_MFMA_STEP, mvpa_hip.KERNEL_MFMA_SPLIT):
+        with pytest.raises(mvpa_hip.MvpaError):
+            mvpa_hip.mvpa_forward(*args, kernel=kern)
+    with pytest.raises(mvpa_hip.MvpaError):
+        mvpa_hip.mvpa_forward(*args, fp8_qk=True)
 
 
 # the build of the kernel in which a wave owns a whole time step (head size 64, 33..64 channels);
@@ -821,7 +858,7 @@ LAST_STEP_SHAPES = [
 
 
 @pytest.mark.parametrize("cfg", LAST_STEP_SHAPES, ids=lambda c: "B{B}C{C}T{T}H{H}D{Dh}".format(**c))
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "fp16"])
 def test_last_step_only_equals_last_rows_of_full_forward(cfg, dtype):
     """MVPA_FLAG_LAST_STEP (one step of incremental decoding: C queries against T*C cached keys)
     gives the rows of the last time step of the full forward: the same kernel code runs on the
@@ -829,7 +866,7 @@ def test_last_step_only_equals_last_rows_of_full_forward(cfg, dtype):
     inp = make_mvpa_inputs(seed=17, qkv_unit=True, **cfg).to("cuda", dtype)
     C = cfg["C"]
     tabs = (inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan)
-    kern = mvpa_hip.KERNEL_MFMA if dtype == torch.bfloat16 else mvpa_hip.KERNEL_GENERIC
+    kern = mvpa_hip.KERNEL_GENERIC if dtype == torch.float32 else mvpa_hip.KERNEL_MFMA
     full, lse_full = mvpa_hip.mvpa_forward(inp.q, inp.k, inp.v, *tabs, return_lse=True, kernel=kern)
     q_last = inp.q[:, :, -C:]
     step, lse_step = mvpa_hip.mvpa_forward(q_last, inp.k, inp.v, *tabs, return_lse=True,
@@ -851,12 +888,14 @@ SPLIT_CASES = [
 
 
 @pytest.mark.parametrize("cfg,n", SPLIT_CASES, ids=lambda c: "B{B}C{C}T{T}H{H}D{Dh}".format(**c) if isinstance(c, dict) else f"n{c}")
-@pytest.mark.parametrize("fp8", [False, True], ids=["bf16", "fp8qk"])
+@pytest.mark.parametrize("fp8", [False, True, "fp16"], ids=["bf16", "fp8qk", "fp16"])
 def test_last_step_key_splits_match_unsplit(cfg, n, fp8):
     """The key steps of a last-step launch cut into runs, each on its own workgroups, merged by the
     second kernel: within bf16 rounding of the one-workgroup result (the partial outputs pass
-    through bf16), log-sum-exp to 1e-3, with some channels absent."""
-    inp = make_mvpa_inputs(seed=23, qkv_unit=True, **cfg).to("cuda", torch.bfloat16)
+    through bf16; through fp16 for fp16 tensors), log-sum-exp to 1e-3, with some channels absent."""
+    dtype = torch.float16 if fp8 == "fp16" else torch.bfloat16
+    fp8 = fp8 is True
+    inp = make_mvpa_inputs(seed=23, qkv_unit=True, **cfg).to("cuda", dtype)
     C = cfg["C"]
     valid = torch.ones(cfg["B"], C, dtype=torch.bool, device="cuda")
     valid[:, 1::5] = False
