@@ -16,7 +16,8 @@ MVPFormer-S forward in windows per second, with the oracle stack on the host cor
 `mvpformer_s_stream` (one new segment of a stream against cached keys and values, beside the
 full forward over the same window), `mvpa_c3` and `mvpa_c5attn` (the irregular-channel
 configuration and the base model's attention shape, a few launches each: time, algorithmic
-TFLOP/s, fraction of the bf16 peak, kernel) and `mvpformer_base` (the base-size classification
+TFLOP/s, fraction of the bf16 peak, kernel, and the time of one mvpa_backward call on the same
+inputs) and `mvpformer_base` (the base-size classification
 forward at B1 C128 T512, bf16 and fp8 QK^T, with the logit gap between the two).
 
 The GPU's clocks take a few dozen milliseconds of work to reach their steady state after a
