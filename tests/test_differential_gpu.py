@@ -1,4 +1,4 @@
-"""Differential sweep on the GPU: the bf16 matrix-core kernels (forward, both backward passes)
+"""Differential sweep on the GPU: the bf16 and fp16 matrix-core kernels (forward, both backward passes)
 against the fp32 kernels of the same library, on seeded random shapes the oracle would take too
 long for (ragged channel counts up to 128, odd time lengths, GQA, narrow / vacuous / zero windows, absent
 channels).  The fp32 kernels are themselves pinned against the oracle in test_mvpa_gpu.py and
@@ -20,6 +20,29 @@ for p in (os.path.join(ROOT, "multi-variate-parallel-transformer_amd"), ROOT):
 from mvpa_hip.synthetic import make_mvpa_inputs  # noqa: E402
 
 pytestmark = pytest.mark.gpu
+
+
+def _compare_backward(d16, d32, o16, l16, o32, l32, live, seed, kw):
+    """Both backward passes on the matrix cores against the fp32 pair: every gradient rel-L2 <= 2e-2."""
+    import mvpa_hip
+    tabs16 = (d16.u, d16.vb, d16.z, d16.k_time, d16.k_chan)
+    tabs32 = (d32.u, d32.vb, d32.z, d32.k_time, d32.k_chan)
+    d_o = torch.randn(o32.shape, device="cuda",
+                      generator=torch.Generator("cuda").manual_seed(seed)).bfloat16()
+    g16 = mvpa_hip.mvpa_backward(d16.q, d16.k, d16.v, o16, d_o, l16, *tabs16, **kw)
+    g32 = mvpa_hip.mvpa_backward(d32.q, d32.k, d32.v, o32, d_o.float(), l32, *tabs32, **kw)
+    for name, a, b in zip(("dq", "dk", "dv", "dbias_time", "dbias_chan"), g16, g32):
+        if name in ("dq", "dbias_time", "dbias_chan"):       # per-query outputs
+            a, b = a * live, b * live
+        assert torch.isfinite(a).all(), name
+        ref_norm = b.norm()
+        if name == "dbias_time":
+            # both tables sum the same dS; with few time steps the rows of this one approach the
+            # row sums of dS, which are zero up to rounding (exactly so at T = 1): measure its
+            # error against the larger of the two tables
+            ref_norm = torch.maximum(ref_norm, (g32[4] * live).norm())
+        rel = ((a - b).norm() / ref_norm.clamp_min(1e-20)).item()
+        assert rel <= 2e-2, (name, rel)
 
 
 def _cases(n=24, seed=20240):
@@ -71,22 +94,7 @@ def test_mfma_paths_match_fp32_kernels(case):
                                            kernel=mvpa_hip.KERNEL_MFMA_STEP, **kw)
         assert ((o16s.float() - o32) * live).abs().max().item() <= 2e-2
         assert ((l16s - l32) * live[..., 0]).abs().max().item() <= 2e-2
-    d_o = torch.randn(o32.shape, device="cuda",
-                      generator=torch.Generator("cuda").manual_seed(case["seed"])).bfloat16()
-    g16 = mvpa_hip.mvpa_backward(d16.q, d16.k, d16.v, o16, d_o, l16, *tabs16, **kw)
-    g32 = mvpa_hip.mvpa_backward(d32.q, d32.k, d32.v, o32, d_o.float(), l32, *tabs32, **kw)
-    for name, a, b in zip(("dq", "dk", "dv", "dbias_time", "dbias_chan"), g16, g32):
-        if name in ("dq", "dbias_time", "dbias_chan"):       # per-query outputs
-            a, b = a * live, b * live
-        assert torch.isfinite(a).all(), name
-        ref_norm = b.norm()
-        if name == "dbias_time":
-            # both tables sum the same dS; with few time steps the rows of this one approach the
-            # row sums of dS, which are zero up to rounding (exactly so at T = 1): measure its
-            # error against the larger of the two tables
-            ref_norm = torch.maximum(ref_norm, (g32[4] * live).norm())
-        rel = ((a - b).norm() / ref_norm.clamp_min(1e-20)).item()
-        assert rel <= 2e-2, (name, rel)
+    _compare_backward(d16, d32, o16, l16, o32, l32, live, case["seed"], kw)
 
 
 def _forward_cases(n=20, seed=777):
@@ -107,7 +115,10 @@ def _forward_cases(n=20, seed=777):
     a="v" if c["absent"] else "", **c))
 def test_mfma_forward_matches_fp32_kernel_at_other_head_sizes(case):
     """Head sizes 32 and 128 (every build of the matrix-core forward the dispatcher can pick for
-    them, far steps included) against the fp32 kernel: output max-abs <= 2e-2, log-sum-exp 2e-2."""
+    them, far steps included) against the fp32 kernel: output max-abs <= 2e-2, log-sum-exp 2e-2.
+    The same inputs as fp16 tensors (bf16 values are fp16 values here) on the fp16 matrix-core
+    kernel: max-abs <= 1e-3, log-sum-exp 2e-3.  At head size 128 also both backward passes on the
+    matrix cores against the fp32 pair."""
     import mvpa_hip
     B, C, T, H, Hkv, Dh = (case[k] for k in ("B", "C", "T", "H", "Hkv", "Dh"))
     inp = make_mvpa_inputs(B=B, C=C, T=T, H=H, Hkv=Hkv, Dh=Dh, seed=case["seed"],
@@ -136,3 +147,12 @@ def test_mfma_forward_matches_fp32_kernel_at_other_head_sizes(case):
         assert torch.isfinite(o16s.float()).all()
         assert ((o16s.float() - o32) * live).abs().max().item() <= 2e-2
         assert ((l16s - l32) * live[..., 0]).abs().max().item() <= 2e-2
+    dh = inp.to("cuda", torch.float16)
+    oh, lh = mvpa_hip.mvpa_forward(dh.q, dh.k, dh.v, dh.u, dh.vb, dh.z, dh.k_time, dh.k_chan,
+                                   kernel=mvpa_hip.KERNEL_MFMA, **kw)
+    assert oh.dtype == torch.float16 and torch.isfinite(oh.float()).all()
+    assert ((oh.float() - o32) * live).abs().max().item() <= 1e-3
+    assert ((lh - l32) * live[..., 0]).abs().max().item() <= 2e-3
+    if Dh == 128:
+        _compare_backward(d16, d32, o16, l16, o32, l32, live, case["seed"],
+                          dict(window=case["window"], chan_valid=valid))
