@@ -45,30 +45,37 @@ class FlashMVPA(torch.autograd.Function):
         B, H, N, Dh = q.shape
         Hkv = k.shape[1]
         grp = H // Hkv
-        qf = q.float().reshape(B, Hkv, grp, N, Dh)
-        # time table (q+vb) @ k_time^T and channel table (q+z) @ k_chan^T, per kv head g
-        dbt = dbt.view(B, Hkv, grp, N, -1)
-        dbc = dbc.view(B, Hkv, grp, N, -1)
-        rt, ec = k_time.float(), k_chan.float()                    # [Hkv,T,Dh], [Hkv,C,Dh]
-        dq_cv = dq_c.view(B, Hkv, grp, N, Dh)
-        dq = dq_cv
-        du = dq_cv.sum(dim=(0, 2, 3)) if content else torch.zeros_like(u, dtype=torch.float32)
-        # a bias term that is switched off takes no part in the forward: its table, its query
-        # bias and the query get nothing through it
+        rows = grp * N                                  # the query rows of a kv head, heads side by side
+        qf = q.float().reshape(B, Hkv, rows, Dh)
+        dq = dq_c.view(B, Hkv, rows, Dh)
+        du = dq.sum(dim=(0, 2)) if content else torch.zeros_like(u, dtype=torch.float32)
+
+        # Per kv head g the table is (q + bias) @ table[g]^T, so with its gradient G [rows, J]:
+        #   d(q + bias) = G @ table[g]      - a batched product over (b, g), and
+        #   d table[g]  = sum_b G^T @ (q + bias)   - per sample a product with G read transposed in
+        # place (an einsum over (b, r, n) would first copy G, the largest tensor of the backward,
+        # into a [g, (b r n), J] layout).  A bias term that is switched off takes no part in the
+        # forward: its table, its query bias and the query get nothing through it.
+        def finish(grad_table, table, bias):
+            g2 = grad_table.view(B, Hkv, rows, -1)
+            tab = table.float()                                        # [Hkv,J,Dh]
+            dq_share = torch.matmul(g2, tab)                           # [B,Hkv,rows,Dh]
+            qb = qf + bias.float()[None, :, None, :]
+            dtab = torch.zeros_like(tab)
+            for b in range(B):
+                dtab = torch.baddbmm(dtab, g2[b].transpose(1, 2), qb[b])
+            return dq_share, dq_share.sum(dim=(0, 2)), dtab
+
         if time_bias:
-            dq_t = torch.einsum("bgrnj,gjd->bgrnd", dbt, rt)
+            dq_t, dvb, dk_time = finish(dbt, k_time, vb)
             dq = dq + dq_t
-            dvb = dq_t.sum(dim=(0, 2, 3))
-            dk_time = torch.einsum("bgrnj,bgrnd->gjd", dbt, qf + vb.float()[None, :, None, None, :])
         else:
-            dvb, dk_time = torch.zeros_like(vb, dtype=torch.float32), torch.zeros_like(rt)
+            dvb, dk_time = torch.zeros_like(vb, dtype=torch.float32), torch.zeros_like(k_time, dtype=torch.float32)
         if chan_bias:
-            dq_ch = torch.einsum("bgrnj,gjd->bgrnd", dbc, ec)
+            dq_ch, dz, dk_chan = finish(dbc, k_chan, z)
             dq = dq + dq_ch
-            dz = dq_ch.sum(dim=(0, 2, 3))
-            dk_chan = torch.einsum("bgrnj,bgrnd->gjd", dbc, qf + z.float()[None, :, None, None, :])
         else:
-            dz, dk_chan = torch.zeros_like(z, dtype=torch.float32), torch.zeros_like(ec)
+            dz, dk_chan = torch.zeros_like(z, dtype=torch.float32), torch.zeros_like(k_chan, dtype=torch.float32)
         return (dq.view(B, H, N, Dh).to(q.dtype), du.to(u.dtype), dvb.to(vb.dtype), dz.to(z.dtype),
                 dk.to(k.dtype), dk_time.to(k_time.dtype), dk_chan.to(k_chan.dtype), dv.to(v.dtype),
                 None, None, None, None, None, None, None, None)
