@@ -9,8 +9,9 @@ built - the kernel contracts the query with the small key tables itself.
 Autograd: when an input requires grad the call goes through `FlashMVPA`, whose backward runs
 `mvpa_backward` (the boundary of the reference's FlashMVPA.backward, attentions/attn.py:1140-1302)
 and finishes the bias-table gradients with the matrix products that autograd applies to
-attentions/attn.py:1305-1314.  Dropout (p_drop > 0) and a torch.Generator are not implemented
-and raise NotImplementedError.
+attentions/attn.py:1305-1314.  Attention dropout (p_drop > 0, optionally with a torch.Generator)
+drops whole key time steps and channels as the reference's kernel does; since the soft-max sum
+ignores the masks it is applied to the values in front of the kernel (dropout_key_scale).
 """
 from __future__ import annotations
 
@@ -81,6 +82,23 @@ class FlashMVPA(torch.autograd.Function):
                 None, None, None, None, None, None, None, None)
 
 
+def dropout_key_scale(p_drop, time_ctx, chan_ctx, device, generator=None, time_keep=None, chan_keep=None):
+    """The reference kernel's attention dropout (attentions/attn.py:1052-1059, 222-227): whole key
+    time steps and whole key channels are dropped, each with probability 1 - sqrt(1 - p_drop), the
+    same keys for every sample, head and query; the probabilities of dropped keys are zeroed AFTER
+    the soft-max sum and the others divided by 1 - p_drop.  The sum does not see the masks, so
+    this is the plain attention on values v[k] * keep[k] / (1 - p_drop): returns that factor per
+    key row [T*C] (fp32).  The masks are drawn as the reference draws them (channels first, then
+    time steps, torch.rand(...) > p_per_dim on the device) unless they are given."""
+    p_per_dim = 1.0 - (1.0 - p_drop) ** 0.5
+    if chan_keep is None:
+        chan_keep = torch.rand(chan_ctx, device=device, generator=generator) > p_per_dim
+    if time_keep is None:
+        time_keep = torch.rand(time_ctx, device=device, generator=generator) > p_per_dim
+    keep = time_keep.to(device=device, dtype=torch.bool)[:, None] & chan_keep.to(device=device, dtype=torch.bool)[None, :]
+    return keep.reshape(time_ctx * chan_ctx).to(torch.float32) / (1.0 - p_drop)
+
+
 def flash_mvpa(
     q,            # [B,H,N,Dh]
     q_bias,       # [1,Hkv,1,Dh]  content bias u
@@ -102,6 +120,8 @@ def flash_mvpa(
     chan_valid=None,     # extension: [B,C] channel-validity mask (1 = present)
     out=None,            # extension: preallocated output, any [B,H,N,Dh]-indexable view
     kernel=mvpa_hip.KERNEL_AUTO,
+    time_keep=None,      # extension: the dropout's keep masks [T] / [C] given instead of drawn
+    chan_keep=None,
 ):
     if rel_bias_chan or rel_bias_time:
         causal = True                                   # attentions/attn.py:1335-1336
@@ -113,9 +133,8 @@ def flash_mvpa(
     assert q.shape[-1] in {16, 32, 64, 128}
     assert time_ctx > 0 and chan_ctx > 0
     if p_drop and p_drop > 0:
-        raise NotImplementedError("flash_mvpa: attention dropout is not implemented (forward/eval only)")
-    if generator is not None:
-        raise NotImplementedError("flash_mvpa: generator is only meaningful with dropout")
+        v = v * dropout_key_scale(p_drop, time_ctx, chan_ctx, q.device, generator,
+                                  time_keep, chan_keep).to(v.dtype)[None, None, :, None]
     if window_size > 0 and not (rel_bias_chan or rel_bias_time):
         raise NotImplementedError(
             "flash_mvpa: a content window without relative biases (masking instead of zeroing) "

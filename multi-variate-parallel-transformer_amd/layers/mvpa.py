@@ -205,6 +205,7 @@ class MVPFormerGQAAttention(torch.nn.Module):
     # the flash subclass of the reference ignores attention_mask / head_mask
     # (layers/mvpa.py:341-397); this flag keeps that difference between the two classes
     _honours_masks = True
+    _key_dropout = False       # attn_pdrop acts on the attention weights (layers/mvpa.py:273)
 
     def __init__(self, config, is_cross_attention=False, layer_idx=None):
         super().__init__()
@@ -342,8 +343,16 @@ class MVPFormerGQAAttention(torch.nn.Module):
         merged heads; c_proj is then left to the caller and merged_out is what comes back.
         qkv: hidden_states @ [q_attn; c_attn]^T when the caller has already formed it."""
         if self.training and (self.attn_dropout.p > 0 or self.resid_dropout.p > 0):
-            raise NotImplementedError("MVPA HIP layer: dropout is not implemented; train with "
-                                      "attn_pdrop = resid_pdrop = 0 or call .eval()")
+            # dropout lives on the differentiable path (one launch per op); the fused inference
+            # path has none
+            if layer_past is not None or merged_out is not None or not torch.is_grad_enabled():
+                raise NotImplementedError("MVPA HIP layer: dropout in train() mode goes with the "
+                                          "whole-sequence forward in grad mode; call .eval() otherwise")
+            if self.attn_dropout.p > 0 and not self._key_dropout:
+                raise NotImplementedError(
+                    "MVPA HIP layer: dropout on the [B,H,N,N] attention weights (layers/mvpa.py:273) "
+                    "is not implemented - the weights are never formed; the flash layer's dropout "
+                    "of whole key steps and channels (layers/mvpa.py:394) is")
         if self.is_cross_attention:
             raise NotImplementedError(
                 "MVPA HIP layer: without the time-causal mask the relative-time shift of the "
@@ -414,11 +423,16 @@ class MVPFormerGQAAttention(torch.nn.Module):
         qkv = AG.linear(hidden_states, w_qkv).reshape(bsz, n, e + 2 * kv)
         q = qkv[:, :, :e].reshape(bsz, n, h, dh).permute(0, 2, 1, 3)
         k = qkv[:, :, e:e + kv].reshape(bsz, n, hkv, dh).permute(0, 2, 1, 3)
-        v = qkv[:, :, e + kv:].reshape(bsz, n, hkv, dh).permute(0, 2, 1, 3)
+        v = v_plain = qkv[:, :, e + kv:].reshape(bsz, n, hkv, dh).permute(0, 2, 1, 3)
         k_time = AG.linear(positional_embedding, self.position_net.weight).reshape(t_len, hkv, dh).permute(1, 0, 2)
         k_chan = AG.linear(channel_embedding, self.channel_net.weight).reshape(c_len, hkv, dh).permute(1, 0, 2)
         u, vb, z = (b.reshape(hkv, dh).to(dt) for b in self.attn_bias.split(kv, dim=0))
         chan_valid, key_bias = self._resolve_mask(attention_mask, bsz, t_len, c_len)
+        if self.training and self.attn_dropout.p > 0:
+            # layers/mvpa.py:394: whole key steps and channels dropped, the rest scaled up; the
+            # soft-max sum ignores the masks, so the values carry them (attentions.attn)
+            from attentions.attn import dropout_key_scale
+            v = v * dropout_key_scale(self.attn_dropout.p, t_len, c_len, v.device).to(dt)[None, None, :, None]
         out = FlashMVPA.apply(q, u, vb, z, k, k_time.contiguous(), k_chan.contiguous(), v, True,
                               self._scale(), window, True, True, chan_valid, self._content(), key_bias)
         merged = out.permute(0, 2, 1, 3)                                      # [B,N,H,Dh]
@@ -427,9 +441,10 @@ class MVPFormerGQAAttention(torch.nn.Module):
                 raise NotImplementedError("head_mask must hold one factor per head")
             merged = merged * head_mask.to(dt).reshape(1, 1, h, 1)
         out = AG.linear(merged.reshape(bsz, t_len, c_len, e), self.c_proj.weight)
+        out = self.resid_dropout(out)                                        # layers/mvpa.py:333, 401
         present = None
         if use_cache is True:
-            present = (k.reshape(bsz, hkv, t_len, c_len, dh), v.reshape(bsz, hkv, t_len, c_len, dh))
+            present = (k.reshape(bsz, hkv, t_len, c_len, dh), v_plain.reshape(bsz, hkv, t_len, c_len, dh))
         return out, present
 
     def _attend_step(self, hidden_states, positional_embedding, channel_embedding, attention_mask,
@@ -551,6 +566,7 @@ class MVPFormerGQAFlashAttention(MVPFormerGQAAttention):
     (see _attend_step)."""
 
     _honours_masks = False
+    _key_dropout = True        # attn_pdrop drops whole key steps / channels inside the operator
 
     # The reference's flash layer calls its kernel with sm_scale = 1/sqrt(Dh) and the content term
     # always on, whatever scale_attn_weights, scale_attn_by_inverse_layer_idx and global_att say

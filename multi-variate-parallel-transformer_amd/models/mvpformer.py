@@ -7,8 +7,8 @@ Two paths through every module.  Inference (eval() mode, or under torch.no_grad(
 launches, nothing kept for a backward.  Differentiable (grad mode on and either train() mode or
 an input that carries a graph): the same kernels one product at a time through
 mvpa_hip.autograd and attentions.attn.FlashMVPA, so that gradients reach the input and every
-parameter as they do through models/mvpformer.py:132-147 and layers/mvpa.py:280-337.  Dropout is
-not implemented: the *_pdrop values must be 0 in train() mode.
+parameter as they do through models/mvpformer.py:132-147 and layers/mvpa.py:280-337.  Dropout
+(embd_pdrop, resid_pdrop, and attn_pdrop as the flash layer applies it) acts on that path only.
 """
 from __future__ import annotations
 
@@ -326,13 +326,17 @@ class MVPFormerModel(nn.Module):
         repeats the same 0/1 pattern at every time step, without a look at its values.
 
         Gradients: with grad mode on and either train() mode or an inputs_embeds that carries a
-        graph, the whole-sequence forward is differentiable (dropout must be 0)."""
+        graph, the whole-sequence forward is differentiable; in train() mode the embedding,
+        residual and attention dropouts of the reference apply there (the attention's as the flash
+        layer has it: whole key steps and channels)."""
         if inputs_embeds is None:
             raise NotImplementedError
-        if self.training and self.drop.p > 0:
-            raise NotImplementedError("MVPFormer HIP stack: dropout is not implemented; train with "
-                                      "embd_pdrop = 0 or call .eval()")
         grad = torch.is_grad_enabled() and past_key_values is None and (self.training or inputs_embeds.requires_grad)
+        if self.training and self.drop.p > 0:
+            if not grad:
+                raise NotImplementedError("MVPFormer HIP stack: dropout in train() mode goes with the "
+                                          "whole-sequence forward in grad mode; call .eval() otherwise")
+            inputs_embeds = self.drop(inputs_embeds)                 # models/mvpformer.py:285
         with torch.set_grad_enabled(grad):
             return self._forward(past_key_values, inputs_embeds, attention_mask, use_cache, position_end,
                                  channel_validity)

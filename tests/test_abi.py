@@ -219,7 +219,10 @@ def test_python_operator_errors():
     b = torch.zeros(1, 4, 1, 32)
     with pytest.raises(AssertionError):      # N != T*C
         flashmvpa(q, b, b, b, kv, torch.zeros(1, 4, 5, 32), torch.zeros(1, 4, 3, 32), kv, True, 0.1)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(NotImplementedError):  # a content window without the relative biases
+        flashmvpa(q, b, b, b, kv, torch.zeros(1, 4, 4, 32), torch.zeros(1, 4, 3, 32), kv, False, 0.1,
+                  window_size=10, rel_bias_time=False, rel_bias_chan=False)
+    with pytest.raises(RuntimeError):        # CPU tensors: no fallback path, with dropout neither
         flashmvpa(q, b, b, b, kv, torch.zeros(1, 4, 4, 32), torch.zeros(1, 4, 3, 32), kv, True, 0.1,
                   p_drop=0.1)
     with pytest.raises(RuntimeError):        # CPU tensors: no fallback path

@@ -4,6 +4,8 @@ backward passes, FlashMVPA with the mvpa_backward kernels, RMSNorm - against rev
 differentiation of the CPU oracle on the same bf16-rounded weights, in float64.
 Tolerances are this build's statement for bf16 arithmetic: relative L2 error of every gradient
 <= 3e-2 (fp32 layer: <= 2e-4)."""
+import math
+
 import pytest
 import torch
 
@@ -118,10 +120,127 @@ def test_eval_forward_stays_on_the_fused_path():
     c = layer(hidden.clone().requires_grad_(True), pos, chan)[0]
     assert c.requires_grad
     assert (c.detach().float() - a.float()).abs().max().item() <= 2e-2
+    # dropout needs the differentiable path: train() mode under no_grad has none
     layer.train()
     layer.attn_dropout.p = 0.1
-    with pytest.raises(NotImplementedError):
+    with torch.no_grad(), pytest.raises(NotImplementedError):
         layer(hidden, pos, chan)
+    # the masked layer's dropout acts on the [B,H,N,N] weights, which are never formed
+    masked = MVPFormerGQAAttention(cfg, layer_idx=0).to(device="cuda", dtype=torch.bfloat16).train()
+    masked.attn_dropout.p = 0.1
+    with pytest.raises(NotImplementedError):
+        masked(hidden, pos, chan)
+
+
+def _keep_masks(T, C, drop_t, drop_c):
+    tk = torch.ones(T, dtype=torch.bool)
+    ck = torch.ones(C, dtype=torch.bool)
+    tk[list(drop_t)] = False
+    ck[list(drop_c)] = False
+    return tk, ck
+
+
+def test_attention_dropout_is_the_reference_kernels():
+    """attentions/attn.py:1052-1059, 222-227: whole key steps and channels are dropped, AFTER the
+    soft-max sum, the rest divided by 1 - p.  With v = 1 the output of a query is therefore its
+    kept probability mass / (1 - p) - below 1 / (1 - p) wherever a visible key was dropped (a
+    dropout that masked keys before the soft-max would give exactly 1 / (1 - p)) - and equals the
+    oracle's attention on the indicator of the kept keys; with random v output and gradients
+    equal the oracle's on values scaled key by key."""
+    import math
+    from attentions import flashmvpa
+    from mvpa_hip.synthetic import make_mvpa_inputs
+    B, C, T, H, Hkv, Dh, p = 2, 12, 9, 2, 1, 32, 0.25
+    inp = make_mvpa_inputs(B=B, C=C, T=T, H=H, Hkv=Hkv, Dh=Dh, seed=3, qkv_unit=True)
+    tk, ck = _keep_masks(T, C, drop_t=(2, 7), drop_c=(0, 5, 11))
+    keep = torch.zeros(T * C, dtype=torch.float64)
+    for t in range(T):
+        for c in range(C):
+            keep[t * C + c] = 1.0 if (tk[t] and ck[c]) else 0.0
+    d = inp.to("cuda", torch.float32)
+
+    def run(v, **kw):
+        return flashmvpa(d.q, d.u.view(1, Hkv, 1, Dh), d.vb.view(1, Hkv, 1, Dh), d.z.view(1, Hkv, 1, Dh), d.k,
+                         d.k_time.view(1, Hkv, T, Dh), d.k_chan.view(1, Hkv, C, Dh), v, True,
+                         1.0 / math.sqrt(Dh), window_size=10, **kw)
+    ones = torch.ones_like(d.v)
+    got = run(ones, p_drop=p, time_keep=tk.cuda(), chan_keep=ck.cuda()).double().cpu()
+    args64 = [t.double() for t in (inp.q, inp.k)]
+    tabs64 = [t.double() for t in (inp.u, inp.vb, inp.z, inp.k_time, inp.k_chan)]
+    mass = O.mvpa_direct(args64[0], args64[1], keep[None, None, :, None].expand(B, Hkv, T * C, Dh).contiguous(),
+                         *tabs64, window=10)
+    assert (got - mass / (1 - p)).abs().max().item() <= 1e-5
+    rows_with_a_dropped_key = got[:, :, 3 * C:, 0]                 # from time step 3 on, step 2 is visible
+    assert (rows_with_a_dropped_key < 1 / (1 - p) - 1e-4).all()
+    # random values, output and every gradient
+    leaves = {n: getattr(d, n).clone().requires_grad_(True) for n in ("q", "k", "v")}
+    out = flashmvpa(leaves["q"], d.u.view(1, Hkv, 1, Dh), d.vb.view(1, Hkv, 1, Dh), d.z.view(1, Hkv, 1, Dh),
+                    leaves["k"], d.k_time.view(1, Hkv, T, Dh), d.k_chan.view(1, Hkv, C, Dh), leaves["v"], True,
+                    1.0 / math.sqrt(Dh), window_size=10, p_drop=p, time_keep=tk.cuda(), chan_keep=ck.cuda())
+    g_out = torch.randn(out.shape, device="cuda", generator=torch.Generator("cuda").manual_seed(1))
+    out.backward(g_out)
+    ref_leaves = {n: getattr(inp, n).double().clone().requires_grad_(True) for n in ("q", "k", "v")}
+    ref = O.mvpa_direct(ref_leaves["q"], ref_leaves["k"], ref_leaves["v"] * (keep / (1 - p))[None, None, :, None],
+                        *tabs64, window=10)
+    (ref * g_out.double().cpu()).sum().backward()
+    assert (out.detach().double().cpu() - ref.detach()).abs().max().item() <= 1e-5
+    for n in ("q", "k", "v"):
+        err = (leaves[n].grad.double().cpu() - ref_leaves[n].grad).abs().max().item()
+        assert err <= 2e-5 + 1e-4 * ref_leaves[n].grad.abs().max().item(), (n, err)
+    assert leaves["v"].grad[:, :, keep == 0].abs().max().item() == 0.0     # dropped keys: no value gradient
+
+
+def test_attention_dropout_masks_are_drawn_as_the_reference_draws_them():
+    """Channels first, then time steps, `torch.rand(n) > 1 - sqrt(1 - p)` on the device from the
+    generator given (attentions/attn.py:1052-1059): the same generator state gives the same masks
+    as those two calls, and the keep rate per key is 1 - p."""
+    from attentions.attn import dropout_key_scale
+    T, C, p = 64, 128, 0.19
+    g = torch.Generator("cuda").manual_seed(123)
+    scale = dropout_key_scale(p, T, C, torch.device("cuda"), g)
+    g2 = torch.Generator("cuda").manual_seed(123)
+    per_dim = 1 - (1 - p) ** 0.5
+    chan = torch.rand(C, device="cuda", generator=g2) > per_dim
+    time = torch.rand(T, device="cuda", generator=g2) > per_dim
+    want = (time[:, None] & chan[None, :]).reshape(-1).float() / (1 - p)
+    assert torch.equal(scale, want)
+    rate = torch.stack([(dropout_key_scale(p, T, C, torch.device("cuda"), g) > 0).float().mean() for _ in range(200)]).mean().item()
+    assert abs(rate - (1 - p)) <= 0.02, rate
+
+
+def test_layer_and_stack_train_with_the_shipped_dropout_rates():
+    """train() mode with resid_pdrop = embd_pdrop = attn_pdrop = 0.1 (the reference's defaults,
+    models/mvpformer.py:43): the flash layer and the stack run forward and backward, the draw
+    follows torch's generator (same seed, same result; another seed, another result), eval() is
+    untouched, and every parameter receives a finite gradient."""
+    torch.manual_seed(11)
+    cfg = _config(resid_pdrop=0.1, embd_pdrop=0.1, attn_pdrop=0.1)
+    layer = MVPFormerGQAFlashAttention(cfg, layer_idx=0).to(device="cuda", dtype=torch.bfloat16)
+    hidden = torch.randn(2, 9, 33, 128, device="cuda").to(torch.bfloat16)
+    pos = torch.randn(1, 9, 128, device="cuda").to(torch.bfloat16)
+    chan = torch.randn(1, 33, 128, device="cuda").to(torch.bfloat16)
+    ref = layer.eval()(hidden, pos, chan)[0]
+    layer.train()
+    torch.manual_seed(1)
+    a = layer(hidden, pos, chan)[0]
+    torch.manual_seed(1)
+    b = layer(hidden, pos, chan)[0]
+    torch.manual_seed(2)
+    c = layer(hidden, pos, chan)[0]
+    assert torch.equal(a, b) and not torch.equal(a, c) and not torch.equal(a.detach(), ref)
+    assert torch.equal(layer.eval()(hidden, pos, chan)[0], ref)
+    L, B, T, C = 64, 2, 7, 33
+    model = HMVPFormer(cfg, WaveEncoder(L, cfg.n_embd), MVPFormerHead(cfg.n_embd, cfg.n_embd))
+    model = model.to(device="cuda", dtype=torch.bfloat16).train()
+    x = torch.randn(B, T, C, L, device="cuda")
+    out = model.predict_next_segment(x)
+    y = out[0] if isinstance(out, (tuple, list)) else out
+    y.float().pow(2).mean().backward()
+    used = [n for n, prm in model.named_parameters() if prm.grad is not None]
+    assert len(used) >= 10
+    for n, prm in model.named_parameters():
+        if prm.grad is not None:
+            assert torch.isfinite(prm.grad).all(), n
 
 
 def test_stack_gradients_bf16():
