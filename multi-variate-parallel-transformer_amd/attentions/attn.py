@@ -47,24 +47,23 @@ class FlashMVPA(torch.autograd.Function):
         Hkv = k.shape[1]
         grp = H // Hkv
         rows = grp * N                                  # the query rows of a kv head, heads side by side
-        qf = q.float().reshape(B, Hkv, rows, Dh)
         dq = dq_c.view(B, Hkv, rows, Dh)
         du = dq.sum(dim=(0, 2)) if content else torch.zeros_like(u, dtype=torch.float32)
+        # bf16 runs take these products in bf16 (fp32 accumulation), as the kernels take theirs
+        cd = torch.bfloat16 if q.dtype == torch.bfloat16 else torch.float32
+        q2 = q.reshape(B, Hkv, rows, Dh)
 
         # Per kv head g the table is (q + bias) @ table[g]^T, so with its gradient G [rows, J]:
-        #   d(q + bias) = G @ table[g]      - a batched product over (b, g), and
-        #   d table[g]  = sum_b G^T @ (q + bias)   - per sample a product with G read transposed in
-        # place (an einsum over (b, r, n) would first copy G, the largest tensor of the backward,
-        # into a [g, (b r n), J] layout).  A bias term that is switched off takes no part in the
-        # forward: its table, its query bias and the query get nothing through it.
+        #   d(q + bias) = G @ table[g]            - one batched product over (b, g), and
+        #   d table[g]  = sum_b G^T @ (q + bias)  - one batched product with G read transposed in
+        # place, then a sum over b (an einsum over (b, r, n) would first copy G, the largest tensor
+        # of the backward, into a [g, (b r n), J] layout).  A bias term that is switched off takes
+        # no part in the forward: its table, its query bias and the query get nothing through it.
         def finish(grad_table, table, bias):
-            g2 = grad_table.view(B, Hkv, rows, -1)
-            tab = table.float()                                        # [Hkv,J,Dh]
-            dq_share = torch.matmul(g2, tab)                           # [B,Hkv,rows,Dh]
-            qb = qf + bias.float()[None, :, None, :]
-            dtab = torch.zeros_like(tab)
-            for b in range(B):
-                dtab = torch.baddbmm(dtab, g2[b].transpose(1, 2), qb[b])
+            g2 = grad_table.view(B, Hkv, rows, -1).to(cd)
+            dq_share = torch.matmul(g2, table.to(cd)).float()          # [B,Hkv,rows,Dh]
+            qb = (q2.float() + bias.float()[None, :, None, :]).to(cd)
+            dtab = torch.matmul(g2.transpose(2, 3), qb).float().sum(0)  # [Hkv,J,Dh]
             return dq_share, dq_share.sum(dim=(0, 2)), dtab
 
         if time_bias:

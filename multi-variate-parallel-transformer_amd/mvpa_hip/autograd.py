@@ -39,10 +39,9 @@ class _LinearFn(torch.autograd.Function):
         dy2 = dy.reshape(-1, dy.shape[-1]).contiguous()
         dx = dw = None
         if ctx.needs_input_grad[0]:
-            dx = mvpa_hip.linear(_k8(dy2), _k8(w.t())).view(x.shape)              # [M,N] @ [N,K]
+            dx = torch.matmul(dy2, w).view(x.shape)                               # [M,N] @ [N,K]
         if ctx.needs_input_grad[1]:
-            x2 = x.reshape(-1, k)
-            dw = mvpa_hip.linear(_k8(dy2.t()), _k8(x2.t()))                       # [N,M] @ [M,K]
+            dw = torch.matmul(dy2.t(), x.reshape(-1, k))                          # [N,M] @ [M,K]
         return dx, dw
 
 
