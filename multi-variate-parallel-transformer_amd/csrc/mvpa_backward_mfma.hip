@@ -408,7 +408,10 @@ __global__ __launch_bounds__((QUERY_WAVES<DH, NCT> * 64)) void mvpa_bwd_query_mf
       const float g = Gtb[ln * GP + q];
       if (q < nq_live && ln < nj) {
         float* dst = a.dbias_time + (wrow0 + q) * T_ + j0 + ln;
-        *dst = accum ? *dst + g : g;              // launches of one stream: the key parts add up
+        // launches of one stream: the key parts add up.  An atomic add without a return value,
+        // not a load and a store: nothing waits for the old value (every address has one writer)
+        if (accum) atomicAdd(dst, g);
+        else *dst = g;
       }
     }
   };
@@ -638,7 +641,8 @@ __global__ __launch_bounds__((QUERY_WAVES<DH, NCT> * 64)) void mvpa_bwd_query_mf
       if (d > 0 && hi >= 0 && hi < CP) g += g2;
       if (q < nq_live && col < C_) {
         float* dst = a.dbias_chan + (wrow0 + q) * C_ + col;
-        *dst = accum ? *dst + g : g;
+        if (accum) atomicAdd(dst, g);
+        else *dst = g;
       }
     }
   }
