@@ -1,9 +1,12 @@
 """Differentiable wrappers of the library's dense ops, for gradients through the layer and stack
 modules (the reference trains through layers/mvpa.py:280-337 and models/mvpformer.py:132-147).
 
-Forward passes are the library's kernels; backward passes of the products are two more products
-on the same MFMA GEMM (dX = dY W, dW = dY^T X), the norm's backward is a few fp32 tensor ops.
-The attention operator itself is `attentions.attn.FlashMVPA` (mvpa_backward kernels).
+Forward passes are the library's kernels.  The backward passes of the bf16 products are the two
+plain products dX = dY W and dW = dY^T X on the vendor library through torch.matmul: it reads
+the transposed operand in place and splits the long contraction of a weight gradient (a small
+[N,K] output over all rows), which this library's GEMM would run on a few dozen tiles.  The
+norm's backward is a few fp32 tensor ops.  The attention operator itself is
+`attentions.attn.FlashMVPA` (mvpa_backward kernels).
 """
 from __future__ import annotations
 
@@ -16,16 +19,8 @@ def wants_grad(*tensors) -> bool:
     return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
 
 
-def _k8(t: torch.Tensor) -> torch.Tensor:
-    """[rows, K] contiguous with K padded by zero columns to a multiple of 8 (the GEMM fetches rows
-    in 16-byte chunks); zero columns add nothing to a product."""
-    pad = (-t.shape[-1]) % 8
-    t = torch.nn.functional.pad(t, (0, pad)) if pad else t
-    return t.contiguous()
-
-
 class _LinearFn(torch.autograd.Function):
-    """y = x @ w^T, bf16 on the GPU library, any leading shape of x."""
+    """y = x @ w^T, bf16, any leading shape of x: forward on the GPU library, backward on the vendor GEMM."""
 
     @staticmethod
     def forward(ctx, x, w):
